@@ -1,0 +1,188 @@
+/*
+ * mi355_convbias.h -- C ABI of the MI355X (gfx950) quantized ConvBias / RelayoutFormat path.
+ *
+ * This is the boundary a MegDNN handle backend binds: plain C types, caller-owned
+ * device pointers, no allocation, no exceptions.  Every entry point returns an
+ * mi355_status; the C++ operator classes turn a non-zero status into megdnn_throw.
+ *
+ * Reference interfaces each entry point stands in for (paths relative to the
+ * MegEngine tree):
+ *   mi355_conv_desc            <- param::ConvBias (dnn/scripts/opr_param_defs.py:199-215)
+ *                                 + ConvolutionBase::CanonizedFilterMeta
+ *                                 (dnn/include/megdnn/oprs/nn.h:82-135)
+ *                                 + the QuantizedS8/QuantizedS32 dtype scales
+ *                                 (dnn/include/megdnn/dtype.h:835-898)
+ *   mi355_convbias_s8_query    <- ConvBiasForward::get_workspace_in_bytes
+ *                                 (dnn/include/megdnn/oprs/nn.h:419-422) and
+ *                                 get_algorithm_heuristic (dnn/include/megdnn/oprs/base.h:595-614)
+ *   mi355_convbias_s8_exec     <- ConvBiasForward::exec (dnn/include/megdnn/oprs/nn.h:381-385),
+ *                                 arithmetic of naive::ConvBiasForwardImpl::exec
+ *                                 (dnn/src/naive/conv_bias/opr_impl.cpp:211-292)
+ *   mi355_convbias_algo_*      <- MultiAlgoOpr::get_all_algorithms / Algorithm::name
+ *                                 (dnn/include/megdnn/oprs/base.h:545-615)
+ *   mi355_relayout_exec        <- RelayoutFormat::exec (dnn/include/megdnn/oprs/general.h:1353-1359),
+ *                                 arithmetic of naive::RelayoutFormatImpl::exec
+ *                                 (dnn/src/naive/relayout_format/opr_impl.cpp:486-773)
+ *   mi355_status_string        <- ErrorHandler::on_megdnn_error message path
+ *                                 (dnn/include/megdnn/basic_types.h:21-58)
+ */
+#ifndef MI355_CONVBIAS_H_
+#define MI355_CONVBIAS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_CONVBIAS_ABI_VERSION 1
+
+typedef enum mi355_status {
+    MI355_OK = 0,
+    MI355_ERR_BAD_ARG = 1,       /* null pointer / malformed descriptor */
+    MI355_ERR_UNSUPPORTED = 2,   /* legal megdnn request this backend does not cover */
+    MI355_ERR_SHAPE = 3,         /* shapes inconsistent (channel/group/pack mismatch) */
+    MI355_ERR_WORKSPACE = 4,     /* workspace smaller than query() reported */
+    MI355_ERR_LAUNCH = 5,        /* HIP launch or runtime error */
+    MI355_ERR_NO_DEVICE = 6,     /* no gfx950 device visible */
+    MI355_ERR_ALGO = 7           /* algorithm id unknown or not usable for this descriptor */
+} mi355_status;
+
+/* values of param::ConvBias::Format (opr_param_defs.py:96-113) */
+enum {
+    MI355_FMT_NCHW = 0,
+    MI355_FMT_NCHW4 = 3,
+    MI355_FMT_NCHW32 = 5,
+    MI355_FMT_NCHW44 = 7,
+    MI355_FMT_NCHW4_NCHW32 = 9,
+    MI355_FMT_NCHW32_NCHW4 = 10
+};
+/* param::ConvBias::NonlineMode (opr_param_defs.py:5-35); SIGMOID (2) is rejected for
+ * quantized data exactly as naive does (conv_bias/opr_impl.cpp:79-88). */
+enum { MI355_NL_IDENTITY = 0, MI355_NL_RELU = 1, MI355_NL_SIGMOID = 2, MI355_NL_H_SWISH = 3 };
+/* param::ConvBias::Mode */
+enum { MI355_MODE_CROSS_CORRELATION = 0, MI355_MODE_CONVOLUTION = 1 };
+/* param::ConvBias::Sparse */
+enum { MI355_SPARSE_DENSE = 0, MI355_SPARSE_GROUP = 1 };
+/* ConvBiasForward::BiasMode (nn.h:449-453) */
+enum { MI355_BIAS_NONE = 0, MI355_BIAS_BROADCAST_CHANNEL = 1, MI355_BIAS_FULL = 2 };
+/* dst dtype */
+enum { MI355_DT_QS8 = 0, MI355_DT_QS32 = 1 };
+
+/*
+ * One ConvBias problem.  Channel counts are LOGICAL channels (ic = group * icpg,
+ * oc = group * ocpg); packed formats store ic/4 or ic/32 blocks.
+ *
+ * Tensor layouts (all int8 unless noted, innermost dimension last):
+ *   NCHW    src (n, ic, ih, iw)        filter (oc, ic, fh, fw) | (g, ocpg, icpg, fh, fw)
+ *   NCHW4   src (n, ic/4, ih, iw, 4)   filter (oc, ic/4, fh, fw, 4) | (g, ocpg, icpg/4, fh, fw, 4)
+ *   NCHW32  same with 32
+ *   NCHW44  src (n, ic/4, ih, iw, 4)   filter dense (oc/4, ic/4, fh, fw, 4ic, 4oc),
+ *           group (g, ocpg/4, icpg/4, fh, fw, 4ic, 4oc), channel-wise (g/4, 1, 1, fh, fw, 4)
+ *   NCHW4 with sparse=GROUP and icpg == ocpg == 1 is accepted as an extension and uses the
+ *   NCHW44 channel-wise filter layout (g/4, 1, 1, fh, fw, 4); the reference cannot express
+ *   icpg < 4 under Format::NCHW4 (dnn/src/common/convolution.cpp:392-407).
+ *   NCHW4_NCHW32 / NCHW32_NCHW4: src+filter in the first pack, dst/bias in the second.
+ *   bias: int32, (1, oc, 1, 1) / (1, oc/p, 1, 1, p) of the dst pack, or the full dst shape.
+ *   z:    dst dtype and shape, own scale.
+ * src/dst/z may have a non-contiguous batch dimension: *_stride_n are in elements, 0 = dense.
+ */
+typedef struct mi355_conv_desc {
+    uint32_t format;
+    uint32_t sparse;
+    uint32_t nonline;
+    uint32_t mode;
+    uint32_t n, ic, ih, iw;
+    uint32_t oc, fh, fw;
+    uint32_t group;
+    uint32_t pad_h, pad_w, stride_h, stride_w, dilate_h, dilate_w;
+    uint32_t dst_dtype;
+    uint32_t bias_mode;
+    uint32_t has_z;
+    float scale_bias; /* scale stored on the bias dtype (QuantizedS32), used even when bias is absent */
+    float scale_z;
+    float scale_dst;
+    int64_t src_stride_n, dst_stride_n, z_stride_n;
+} mi355_conv_desc;
+
+/* Opaque-ish algorithm choice: id indexes the static algorithm table; the tile fields are
+ * filled by query() and must be passed back unchanged. */
+typedef struct mi355_algo {
+    int32_t id;
+    int32_t tile_cfg;
+    uint64_t reserved;
+} mi355_algo;
+
+#define MI355_ALGO_HEURISTIC (-1)
+
+/* ---- library / device ---- */
+int mi355_abi_version(void);
+const char* mi355_status_string(int status);
+/* last error text of the calling thread (HIP error string, failed check) */
+const char* mi355_last_error(void);
+
+typedef struct mi355_device_info {
+    int32_t device;
+    int32_t compute_units;
+    int32_t clock_khz;
+    int32_t lds_bytes_per_cu;
+    int64_t hbm_bytes;
+    char arch[32];
+    char name[96];
+} mi355_device_info;
+int mi355_get_device_info(int device, mi355_device_info* out);
+
+/* ---- ConvBias ---- */
+/* output spatial size: floor((i + 2p - ((f-1)d+1)) / s) + 1  (dnn/src/common/utils.cpp:130-138) */
+int mi355_convbias_deduce_out(const mi355_conv_desc* d, uint32_t* oh, uint32_t* ow);
+
+/* number of algorithms in the static table, their names ("MI355_IGEMM_MFMA_I8", ...) */
+int mi355_convbias_algo_count(void);
+const char* mi355_convbias_algo_name(int id);
+/* MI355_OK if algorithm `id` can run descriptor `d` */
+int mi355_convbias_algo_usable(const mi355_conv_desc* d, int id);
+
+/* Validate d, pick an algorithm (algo_request = MI355_ALGO_HEURISTIC or a table id) and
+ * report the workspace it needs. */
+int mi355_convbias_s8_query(const mi355_conv_desc* d, int algo_request, mi355_algo* algo_out,
+                            size_t* workspace_bytes);
+
+/* Launch on `stream` (a hipStream_t; NULL = default stream).  Asynchronous. */
+int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_algo* algo,
+                           const int8_t* src, const int8_t* filter, const int32_t* bias,
+                           const int8_t* z, void* dst, void* workspace, size_t workspace_bytes);
+
+/* ---- RelayoutFormat ---- */
+/* param::RelayoutFormat::Mode values (opr_param_defs.py:1069-1111); 32/33 and 34/35 are
+ * extensions of this backend (the reference has no NCHW32 relayout mode). */
+enum {
+    MI355_RL_NCHW_NCHW4_IC_SMALL = 22,
+    MI355_RL_NCHW_NCHW4 = 24,
+    MI355_RL_NCHW4_NCHW = 25,
+    MI355_RL_NCHW_NCHW4_WEIGHT = 26,
+    MI355_RL_NCHW_NCHW32 = 32,
+    MI355_RL_NCHW32_NCHW = 33,
+    MI355_RL_NCHW4_NCHW32 = 34,
+    MI355_RL_NCHW32_NCHW4 = 35
+};
+
+typedef struct mi355_relayout_desc {
+    uint32_t mode;
+    uint32_t ndim;         /* src ndim */
+    uint32_t shape[7];     /* src shape */
+    uint32_t group;        /* param.group (>= 1) */
+    uint32_t oc;           /* param.oc (0 = keep all channels) */
+    uint32_t elem_bytes;   /* 1 (int8) or 4 (int32/float32: pure permutation) */
+    float scale_src;       /* QuantizedS8 scales; equal scales = pure byte permutation */
+    float scale_dst;
+} mi355_relayout_desc;
+
+/* dst shape for the descriptor (dnn/src/common/relayout_format.cpp:7-296) */
+int mi355_relayout_deduce(const mi355_relayout_desc* d, uint32_t* ndim, uint32_t shape[7]);
+int mi355_relayout_exec(void* stream, const mi355_relayout_desc* d, const void* src, void* dst);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_CONVBIAS_H_ */

@@ -1,0 +1,136 @@
+"""ctypes mirror of include/mi355_convbias.h (struct layouts and enum values).
+
+Only plain data lives here, so both the product binding (megengine_amd.lib) and the CPU
+parity checker's wrapper can share one definition of the descriptors.
+"""
+import ctypes as C
+
+ABI_VERSION = 1
+
+# mi355_status
+OK, ERR_BAD_ARG, ERR_UNSUPPORTED, ERR_SHAPE, ERR_WORKSPACE, ERR_LAUNCH, ERR_NO_DEVICE, ERR_ALGO = range(8)
+
+# param::ConvBias::Format
+FMT_NCHW, FMT_NCHW4, FMT_NCHW32, FMT_NCHW44, FMT_NCHW4_NCHW32, FMT_NCHW32_NCHW4 = 0, 3, 5, 7, 9, 10
+FORMAT_NAMES = {
+    "NCHW": FMT_NCHW, "NCHW4": FMT_NCHW4, "NCHW32": FMT_NCHW32, "NCHW44": FMT_NCHW44,
+    "NCHW4_NCHW32": FMT_NCHW4_NCHW32, "NCHW32_NCHW4": FMT_NCHW32_NCHW4,
+}
+# param::ConvBias::NonlineMode
+NL_IDENTITY, NL_RELU, NL_SIGMOID, NL_H_SWISH = 0, 1, 2, 3
+NONLINE_NAMES = {"IDENTITY": NL_IDENTITY, "RELU": NL_RELU, "SIGMOID": NL_SIGMOID, "H_SWISH": NL_H_SWISH}
+MODE_CROSS_CORRELATION, MODE_CONVOLUTION = 0, 1
+SPARSE_DENSE, SPARSE_GROUP = 0, 1
+BIAS_NONE, BIAS_BROADCAST_CHANNEL, BIAS_FULL = 0, 1, 2
+DT_QS8, DT_QS32 = 0, 1
+
+ALGO_HEURISTIC = -1
+
+# param::RelayoutFormat::Mode (+ extension modes 32..35)
+RL_NCHW_NCHW4_IC_SMALL = 22
+RL_NCHW_NCHW4 = 24
+RL_NCHW4_NCHW = 25
+RL_NCHW_NCHW4_WEIGHT = 26
+RL_NCHW_NCHW32 = 32
+RL_NCHW32_NCHW = 33
+RL_NCHW4_NCHW32 = 34
+RL_NCHW32_NCHW4 = 35
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [
+        ("format", C.c_uint32), ("sparse", C.c_uint32), ("nonline", C.c_uint32), ("mode", C.c_uint32),
+        ("n", C.c_uint32), ("ic", C.c_uint32), ("ih", C.c_uint32), ("iw", C.c_uint32),
+        ("oc", C.c_uint32), ("fh", C.c_uint32), ("fw", C.c_uint32),
+        ("group", C.c_uint32),
+        ("pad_h", C.c_uint32), ("pad_w", C.c_uint32), ("stride_h", C.c_uint32), ("stride_w", C.c_uint32),
+        ("dilate_h", C.c_uint32), ("dilate_w", C.c_uint32),
+        ("dst_dtype", C.c_uint32), ("bias_mode", C.c_uint32), ("has_z", C.c_uint32),
+        ("scale_bias", C.c_float), ("scale_z", C.c_float), ("scale_dst", C.c_float),
+        ("src_stride_n", C.c_int64), ("dst_stride_n", C.c_int64), ("z_stride_n", C.c_int64),
+    ]
+
+    def key(self):
+        return tuple(getattr(self, f) for f, _ in self._fields_)
+
+
+class Algo(C.Structure):
+    _fields_ = [("id", C.c_int32), ("tile_cfg", C.c_int32), ("reserved", C.c_uint64)]
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [
+        ("device", C.c_int32), ("compute_units", C.c_int32), ("clock_khz", C.c_int32),
+        ("lds_bytes_per_cu", C.c_int32), ("hbm_bytes", C.c_int64),
+        ("arch", C.c_char * 32), ("name", C.c_char * 96),
+    ]
+
+
+class RelayoutDesc(C.Structure):
+    _fields_ = [
+        ("mode", C.c_uint32), ("ndim", C.c_uint32), ("shape", C.c_uint32 * 7),
+        ("group", C.c_uint32), ("oc", C.c_uint32), ("elem_bytes", C.c_uint32),
+        ("scale_src", C.c_float), ("scale_dst", C.c_float),
+    ]
+
+
+def in_pack(fmt):
+    return {FMT_NCHW: 1, FMT_NCHW4: 4, FMT_NCHW44: 4, FMT_NCHW4_NCHW32: 4}.get(fmt, 32)
+
+
+def out_pack(fmt):
+    return {FMT_NCHW: 1, FMT_NCHW4: 4, FMT_NCHW44: 4, FMT_NCHW32_NCHW4: 4}.get(fmt, 32)
+
+
+def out_size(i, f, d, s, p):
+    """infer_conv_shape (dnn/src/common/utils.cpp:130-138)."""
+    return (i + 2 * p - ((f - 1) * d + 1)) // s + 1
+
+
+def make_conv_desc(fmt, n, ic, ih, iw, oc, fh, fw=None, *, group=1, pad=0, stride=1, dilate=1,
+                   nonline=NL_IDENTITY, mode=MODE_CROSS_CORRELATION, bias_mode=BIAS_BROADCAST_CHANNEL,
+                   has_z=False, scale_bias=1.0, scale_z=1.0, scale_dst=1.0, dst_dtype=DT_QS8,
+                   src_stride_n=0, dst_stride_n=0, z_stride_n=0):
+    if isinstance(fmt, str):
+        fmt = FORMAT_NAMES[fmt]
+    if isinstance(nonline, str):
+        nonline = NONLINE_NAMES[nonline]
+    fw = fh if fw is None else fw
+    ph, pw = (pad, pad) if isinstance(pad, int) else pad
+    sh, sw = (stride, stride) if isinstance(stride, int) else stride
+    dh, dw = (dilate, dilate) if isinstance(dilate, int) else dilate
+    return ConvDesc(
+        format=fmt, sparse=SPARSE_GROUP if group > 1 else SPARSE_DENSE, nonline=nonline, mode=mode,
+        n=n, ic=ic, ih=ih, iw=iw, oc=oc, fh=fh, fw=fw, group=group,
+        pad_h=ph, pad_w=pw, stride_h=sh, stride_w=sw, dilate_h=dh, dilate_w=dw,
+        dst_dtype=dst_dtype, bias_mode=bias_mode, has_z=1 if has_z else 0,
+        scale_bias=scale_bias, scale_z=scale_z, scale_dst=scale_dst,
+        src_stride_n=src_stride_n, dst_stride_n=dst_stride_n, z_stride_n=z_stride_n)
+
+
+def conv_shapes(d):
+    """(src, filter, bias, dst) shapes for a descriptor, in the reference's layouts."""
+    pi, po = in_pack(d.format), out_pack(d.format)
+    oh = out_size(d.ih, d.fh, d.dilate_h, d.stride_h, d.pad_h)
+    ow = out_size(d.iw, d.fw, d.dilate_w, d.stride_w, d.pad_w)
+    icpg, ocpg, g = d.ic // d.group, d.oc // d.group, d.group
+    dw4 = d.format in (FMT_NCHW4, FMT_NCHW44) and g > 1 and icpg == 1 and ocpg == 1
+    if d.format == FMT_NCHW:
+        src = (d.n, d.ic, d.ih, d.iw)
+        flt = (d.oc, d.ic, d.fh, d.fw) if g == 1 else (g, ocpg, icpg, d.fh, d.fw)
+        dst = (d.n, d.oc, oh, ow)
+        bias = (1, d.oc, 1, 1)
+    else:
+        src = (d.n, d.ic // pi, d.ih, d.iw, pi)
+        dst = (d.n, d.oc // po, oh, ow, po)
+        bias = (1, d.oc // po, 1, 1, po)
+        if dw4:
+            flt = (g // 4, 1, 1, d.fh, d.fw, 4)
+        elif d.format == FMT_NCHW44:
+            flt = (d.oc // 4, d.ic // 4, d.fh, d.fw, 4, 4) if g == 1 else \
+                (g, ocpg // 4, icpg // 4, d.fh, d.fw, 4, 4)
+        else:
+            flt = (d.oc, d.ic // pi, d.fh, d.fw, pi) if g == 1 else (g, ocpg, icpg // pi, d.fh, d.fw, pi)
+    if d.bias_mode == BIAS_FULL:
+        bias = dst
+    return src, flt, bias, dst

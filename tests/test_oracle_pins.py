@@ -1,0 +1,328 @@
+"""Pins the CPU parity checker (oracle/) against evidence that does not come from itself:
+the reference's own known-answer vectors, torch's float64 conv2d (exact for these magnitudes),
+closed-form numpy permutations, and IEEE-754 facts about the epilogue.  CPU only."""
+import ctypes as C
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from megengine_amd import _abi
+from tests import util
+
+
+# ----------------------------------------------------------------------------------------
+# reference known-answer vectors
+# ----------------------------------------------------------------------------------------
+
+def test_kat_conv_bias_quantized8x8x32(oracle, kats):
+    k = kats["conv_bias_quantized8x8x32"]
+    s_src, s_flt = np.float32(0.1), np.float32(0.2)
+    d = _abi.make_conv_desc("NCHW", 1, 1, 4, 4, 3, 3, has_z=True, dst_dtype=_abi.DT_QS32,
+                            scale_bias=float(np.float32(0.02)), scale_z=float(np.float32(0.3)),
+                            scale_dst=float(s_src * s_flt))
+    src = np.array(k["src"], np.int8).reshape(1, 1, 4, 4)
+    flt = np.array(k["filter"], np.int8).reshape(3, 1, 3, 3)
+    bias = np.array(k["bias"], np.int32).reshape(1, 3, 1, 1)
+    z = np.array(k["z"], np.int32).reshape(1, 3, 2, 2)
+    out = oracle.conv_bias(d, src, flt, bias, z)
+    assert out.reshape(-1).tolist() == k["dst"]
+
+
+def test_kat_convolution_quantized8x8x32(oracle, kats):
+    k = kats["convolution_quantized8x8x32"]
+    d = _abi.make_conv_desc("NCHW", 1, 1, 4, 4, 3, 3, bias_mode=_abi.BIAS_NONE)
+    src = np.array(k["src"], np.int8).reshape(1, 1, 4, 4)
+    flt = np.array(k["filter"], np.int8).reshape(3, 1, 3, 3)
+    assert oracle.conv_acc(d, src, flt).reshape(-1).tolist() == k["acc"]
+
+
+@pytest.mark.parametrize("name", ["nchw44_dense", "nchw44_dw", "nchw44_group"])
+def test_kat_nchw44(oracle, kats, name):
+    k = kats[name]
+    d = _abi.make_conv_desc("NCHW44", k["n"], k["ic"], k["ih"], k["iw"], k["oc"], k["fh"], pad=k["pad"],
+                            group=k["group"])
+    src_s, flt_s, bias_s, _ = _abi.conv_shapes(d)
+    src = np.array(k["src"], np.int8).reshape(src_s)
+    flt = np.array(k["filter"], np.int8).reshape(flt_s)
+    bias = np.array(k["bias"], np.int32).reshape(bias_s)
+    assert oracle.conv_acc(d, src, flt, bias).reshape(-1).tolist() == k["acc_plus_bias"]
+    if name == "nchw44_dw":
+        # the same problem stated under Format::NCHW4 (packed-by-4 channel-wise extension)
+        d4 = _abi.make_conv_desc("NCHW4", k["n"], k["ic"], k["ih"], k["iw"], k["oc"], k["fh"], pad=k["pad"],
+                                 group=k["group"])
+        assert oracle.conv_acc(d4, src, flt, bias).reshape(-1).tolist() == k["acc_plus_bias"]
+
+
+def test_kat_relayout(oracle, kats):
+    modes = {"NCHW4_NCHW": _abi.RL_NCHW4_NCHW, "NCHW_NCHW4": _abi.RL_NCHW_NCHW4,
+             "NCHW_NCHW4_WEIGHT": _abi.RL_NCHW_NCHW4_WEIGHT}
+    for name, k in kats["relayout"].items():
+        for eb, dt in ((1, np.int8), (4, np.int32)):
+            d = oracle.relayout_desc(modes[k["mode"]], k["src_shape"], group=k["group"], oc=k["oc"], elem_bytes=eb)
+            assert list(oracle.relayout_deduce(d)) == k["dst_shape"], name
+            out = oracle.relayout(d, np.array(k["src"], dt).reshape(k["src_shape"]))
+            assert out.reshape(-1).tolist() == k["dst"], name
+
+
+# ----------------------------------------------------------------------------------------
+# integer convolution vs torch float64 (exact: |acc| < 2^53)
+# ----------------------------------------------------------------------------------------
+
+def torch_conv_acc(src_nchw, flt, bias, stride, pad, dilate, groups, flip=False):
+    w = torch.from_numpy(flt.astype(np.float64))
+    if w.ndim == 5:
+        g, ocpg, icpg, fh, fw = w.shape
+        w = w.reshape(g * ocpg, icpg, fh, fw)
+    if flip:
+        w = torch.flip(w, dims=(2, 3))
+    y = torch.nn.functional.conv2d(torch.from_numpy(src_nchw.astype(np.float64)), w, None, stride, pad, dilate,
+                                   groups)
+    y = y.numpy().astype(np.int64)
+    if bias is not None:
+        y = y + bias.reshape(1, -1, 1, 1).astype(np.int64)
+    return y
+
+
+NCHW_CASES = [
+    # n, ic, ih, iw, oc, fh, fw, group, pad, stride, dilate, flip
+    (2, 3, 7, 9, 5, 3, 3, 1, (1, 1), (1, 1), (1, 1), False),
+    (1, 8, 8, 8, 12, 3, 2, 4, (1, 0), (2, 1), (1, 1), False),
+    (2, 4, 11, 10, 6, 3, 3, 2, (2, 2), (1, 2), (2, 2), False),
+    (1, 5, 9, 9, 5, 5, 5, 5, (2, 2), (1, 1), (1, 1), False),
+    (1, 3, 8, 8, 4, 3, 3, 1, (1, 1), (1, 1), (1, 1), True),
+    (1, 2, 9, 7, 4, 2, 3, 2, (0, 1), (2, 2), (1, 1), True),
+    (3, 16, 5, 5, 8, 1, 1, 1, (0, 0), (1, 1), (1, 1), False),
+]
+
+
+@pytest.mark.parametrize("case", NCHW_CASES)
+def test_acc_nchw_vs_torch(oracle, case):
+    n, ic, ih, iw, oc, fh, fw, g, pad, stride, dil, flip = case
+    d = _abi.make_conv_desc("NCHW", n, ic, ih, iw, oc, fh, fw, group=g, pad=pad, stride=stride, dilate=dil,
+                            mode=_abi.MODE_CONVOLUTION if flip else _abi.MODE_CROSS_CORRELATION)
+    src, flt, bias, _ = util.make_tensors(d, seed=hash(case) % 1000)
+    got = oracle.conv_acc(d, src, flt, bias)
+    want = torch_conv_acc(src, flt, bias, stride, pad, dil, g, flip)
+    assert np.array_equal(got.astype(np.int64), want)
+
+
+PACKED_CASES = [
+    # n, ic, ih, iw, oc, f, group, pad, stride
+    (2, 32, 4, 4, 32, 3, 1, 1, 1),      # shape of CONV_BIAS_QUANTIZED8x8x32_NCHW32 (conv_bias.cpp:163-285)
+    (1, 64, 6, 5, 96, 1, 1, 0, 1),
+    (2, 64, 9, 9, 64, 3, 2, 1, 2),
+    (1, 32, 12, 12, 64, 5, 1, 2, 1),
+    (1, 128, 7, 7, 32, 7, 1, 3, 2),
+]
+
+
+@pytest.mark.parametrize("case", PACKED_CASES)
+def test_acc_packed_formats_equal_nchw(oracle, case):
+    """NCHW4 / NCHW32 / NCHW44 / mixed formats are re-layouts of the NCHW problem (the
+    reference's own metamorphic tests: naive/conv_bias.cpp:163-285, naive/convolution.cpp:141-220)."""
+    n, ic, ih, iw, oc, f, g, pad, stride = case
+    base = _abi.make_conv_desc("NCHW", n, ic, ih, iw, oc, f, group=g, pad=pad, stride=stride)
+    src, flt, bias, _ = util.make_tensors(base, seed=7 + n + ic)
+    want = torch_conv_acc(src, flt, bias, stride, pad, 1, g)
+    for fmt in ("NCHW4", "NCHW32", "NCHW44", "NCHW4_NCHW32", "NCHW32_NCHW4"):
+        d = _abi.make_conv_desc(fmt, n, ic, ih, iw, oc, f, group=g, pad=pad, stride=stride)
+        pi, po = _abi.in_pack(d.format), _abi.out_pack(d.format)
+        if (ic // g) % pi or oc % po or (fmt == "NCHW44" and (oc // g) % 4):
+            continue
+        s = util.nchw_to_packed(src, pi)
+        w = util.filter_nchw_to_nchw44(flt) if fmt == "NCHW44" else util.filter_nchw_to_packed(flt, pi)
+        b = util.bias_to_packed(bias, po)
+        got = oracle.conv_acc(d, s, w, b)
+        assert np.array_equal(util.packed_to_nchw(got).astype(np.int64), want), fmt
+
+
+@pytest.mark.parametrize("shape", [(2, 8, 9, 9, 3, 1, 1), (1, 16, 10, 7, 3, 1, 2), (1, 4, 6, 6, 5, 2, 1)])
+def test_acc_depthwise_packed4_equals_nchw(oracle, shape):
+    n, c, ih, iw, f, pad, stride = shape
+    base = _abi.make_conv_desc("NCHW", n, c, ih, iw, c, f, group=c, pad=pad, stride=stride)
+    src, flt, bias, _ = util.make_tensors(base, seed=c)
+    want = torch_conv_acc(src, flt, bias, stride, pad, 1, c)
+    for fmt in ("NCHW4", "NCHW44"):
+        d = _abi.make_conv_desc(fmt, n, c, ih, iw, c, f, group=c, pad=pad, stride=stride)
+        got = oracle.conv_acc(d, util.nchw_to_packed(src, 4), util.filter_dw_nchw_to_dw4(flt),
+                              util.bias_to_packed(bias, 4))
+        assert np.array_equal(util.packed_to_nchw(got).astype(np.int64), want)
+
+
+def test_acc_brute_force_tiny(oracle):
+    """Pure-python 7-deep loop from the formula on a tiny NCHW4 group case."""
+    d = _abi.make_conv_desc("NCHW4", 1, 8, 3, 4, 8, 2, 3, group=2, pad=(1, 1), stride=(1, 2))
+    src, flt, bias, _ = util.make_tensors(d, seed=3)
+    got = oracle.conv_acc(d, src, flt, bias)
+    oh, ow = got.shape[2], got.shape[3]
+    for oc in range(8):
+        g, ocg = divmod(oc, 4)
+        for y in range(oh):
+            for x in range(ow):
+                acc = int(bias[0, oc // 4, 0, 0, oc % 4])
+                for fh in range(2):
+                    for fw in range(3):
+                        ih, iw = y + fh - 1, 2 * x + fw - 1
+                        if not (0 <= ih < 3 and 0 <= iw < 4):
+                            continue
+                        for icg in range(4):
+                            ic = g * 4 + icg
+                            acc += int(src[0, ic // 4, ih, iw, ic % 4]) * int(flt[g, ocg, icg // 4, fh, fw, icg % 4])
+                assert got[0, oc // 4, y, x, oc % 4] == acc
+
+
+def test_bias_full_and_none(oracle):
+    d = _abi.make_conv_desc("NCHW4", 1, 8, 5, 5, 8, 3, pad=1, bias_mode=_abi.BIAS_FULL)
+    src, flt, bias, _ = util.make_tensors(d, seed=11)
+    d0 = _abi.make_conv_desc("NCHW4", 1, 8, 5, 5, 8, 3, pad=1, bias_mode=_abi.BIAS_NONE)
+    base = oracle.conv_acc(d0, src, flt)
+    assert np.array_equal(oracle.conv_acc(d, src, flt, bias), base + bias)
+
+
+# ----------------------------------------------------------------------------------------
+# epilogue: IEEE-754 binary32 facts
+# ----------------------------------------------------------------------------------------
+
+def np_epilogue(sfb, s_b, z, s_z, nonline, s_d):
+    """Independent statement with numpy float32 scalars (each op rounds separately)."""
+    f = np.float32
+    r = f(f(np.int32(sfb)) * f(s_b))
+    if z is not None:
+        r = f(r + f(f(np.int8(z)) * f(s_z)))
+    if nonline == _abi.NL_RELU:
+        r = f(0) if r <= 0 else r
+    elif nonline == _abi.NL_H_SWISH:
+        t = f(r + f(3))
+        t = min(max(t, f(0)), f(6))
+        r = f(f(r * t) * f(f(1) / f(6)))
+    q = f(r / f(s_d))
+    a = abs(float(q))                          # float32 -> double is exact
+    v = math.copysign(math.floor(a + 0.5), float(q))   # ties away from zero, exact in double
+    return int(min(max(-128.0, v), 127.0))
+
+
+def test_epilogue_vs_numpy_float32(oracle):
+    rng = np.random.RandomState(5)
+    L = oracle.lib()
+    for _ in range(4000):
+        s_b = float(np.float32(np.exp(rng.uniform(np.log(1e-6), np.log(1e-2)))))
+        s_z = float(np.float32(np.exp(rng.uniform(np.log(1e-3), np.log(0.2)))))
+        s_d = float(np.float32(np.exp(rng.uniform(np.log(1e-3), np.log(0.5)))))
+        sfb = int(rng.randint(-2 ** 20, 2 ** 20))
+        z = int(rng.randint(-128, 128))
+        for nl in (_abi.NL_IDENTITY, _abi.NL_RELU, _abi.NL_H_SWISH):
+            for has_z in (0, 1):
+                got = L.oracle_epilogue_s8(sfb, s_b, has_z, z, s_z, nl, s_d)
+                assert got == np_epilogue(sfb, s_b, z if has_z else None, s_z, nl, s_d)
+
+
+def test_epilogue_closed_forms(oracle):
+    L = oracle.lib()
+    # integer scales: everything is exact integer arithmetic (the trick the reference's CUDA
+    # tests use, dnn/test/cuda/conv_bias_int8.cpp:748-759)
+    for sfb in range(-300, 300, 7):
+        for z in (-128, -3, 0, 5, 127):
+            want = max(-128, min(127, math.floor(abs((sfb * 2 + z * 4) / 2) + 0.5) * (1 if sfb * 2 + z * 4 >= 0 else -1)))
+            assert L.oracle_epilogue_s8(sfb, 2.0, 1, z, 4.0, _abi.NL_IDENTITY, 2.0) == want
+    # s_dst == s_bias, IDENTITY, no z  =>  clamp(sfb)
+    for s in (0.05, 0.0123, 1.0):
+        for sfb in (-1000, -129, -128, -1, 0, 1, 126, 127, 128, 999):
+            assert L.oracle_epilogue_s8(sfb, s, 0, 0, 1.0, _abi.NL_IDENTITY, s) == max(-128, min(127, sfb))
+    # RELU => never negative, equals IDENTITY for positive inputs
+    for sfb in range(-500, 500, 13):
+        r = L.oracle_epilogue_s8(sfb, 0.01, 0, 0, 1.0, _abi.NL_RELU, 0.05)
+        i = L.oracle_epilogue_s8(sfb, 0.01, 0, 0, 1.0, _abi.NL_IDENTITY, 0.05)
+        assert r == max(i, 0)
+    # an all-zero z with any scale reproduces the no-z branch bit for bit
+    for sfb in range(-5000, 5000, 37):
+        for nl in (0, 1, 3):
+            assert L.oracle_epilogue_s8(sfb, 2e-4, 1, 0, 0.37, nl, 0.05) == \
+                L.oracle_epilogue_s8(sfb, 2e-4, 0, 0, 1.0, nl, 0.05)
+    # ties round away from zero: 2.5 -> 3, -2.5 -> -3, 0.5 -> 1, -0.5 -> -1
+    assert L.oracle_quantize_s8(2.5, 1.0) == 3 and L.oracle_quantize_s8(-2.5, 1.0) == -3
+    assert L.oracle_quantize_s8(0.5, 1.0) == 1 and L.oracle_quantize_s8(-0.5, 1.0) == -1
+    assert L.oracle_quantize_s8(float(np.float32(0.49999997)), 1.0) == 0
+    assert L.oracle_quantize_s8(1e9, 1.0) == 127 and L.oracle_quantize_s8(-1e9, 1.0) == -128
+    assert L.oracle_quantize_s8(float("nan"), 1.0) == -128
+    # H_SWISH fixed points: x <= -3 -> 0 ; x >= 3 -> x * 6 * (1/6) (one extra rounding) ; x = 0 -> 0
+    assert L.oracle_activation(-3.0, 3) == 0.0 and L.oracle_activation(-10.0, 3) == 0.0
+    assert L.oracle_activation(0.0, 3) == 0.0
+    for x in (3.0, 4.5, 100.0):
+        assert L.oracle_activation(x, 3) == float(np.float32(np.float32(x * 6.0) * np.float32(1.0 / 6.0)))
+    assert L.oracle_activation(1.0, 3) == float(np.float32(np.float32(4.0) * np.float32(np.float32(1) / np.float32(6))))
+
+
+def test_epilogue_monotone(oracle):
+    L = oracle.lib()
+    prev = -128
+    for sfb in range(-40000, 40000, 11):
+        v = L.oracle_epilogue_s8(sfb, 2e-4, 0, 0, 1.0, _abi.NL_IDENTITY, 0.05)
+        assert v >= prev
+        prev = v
+
+
+def test_full_operator_composes(oracle):
+    """conv_bias == elementwise epilogue over conv_acc, incl. strided batch for src/dst/z."""
+    d = _abi.make_conv_desc("NCHW32", 2, 64, 6, 6, 32, 3, pad=1, nonline="H_SWISH", has_z=True,
+                            scale_bias=2e-4, scale_z=0.05, scale_dst=0.05)
+    src, flt, bias, z = util.make_tensors(d, seed=21)
+    out = oracle.conv_bias(d, src, flt, bias, z)
+    sfb = oracle.conv_acc(d, src, flt, bias)
+    L = oracle.lib()
+    want = np.array([L.oracle_epilogue_s8(int(a), d.scale_bias, 1, int(b), d.scale_z, d.nonline, d.scale_dst)
+                     for a, b in zip(sfb.reshape(-1), z.reshape(-1))], np.int8).reshape(out.shape)
+    assert np.array_equal(out, want)
+    # strided batch views
+    per_n_src, per_n_dst = src[0].size, out[0].size
+    src_p = np.zeros((2, per_n_src + 64), np.int8)
+    src_p[:, :per_n_src] = src.reshape(2, -1)
+    z_p = np.zeros((2, per_n_dst + 32), np.int8)
+    z_p[:, :per_n_dst] = z.reshape(2, -1)
+    d2 = _abi.make_conv_desc("NCHW32", 2, 64, 6, 6, 32, 3, pad=1, nonline="H_SWISH", has_z=True,
+                             scale_bias=2e-4, scale_z=0.05, scale_dst=0.05,
+                             src_stride_n=per_n_src + 64, z_stride_n=per_n_dst + 32, dst_stride_n=per_n_dst + 96)
+    assert np.array_equal(oracle.conv_bias(d2, src_p, flt, bias, z_p), out)
+
+
+# ----------------------------------------------------------------------------------------
+# device arithmetic schemes restated on the host (rounding and division without a divide)
+# ----------------------------------------------------------------------------------------
+
+def bits(x):
+    return int(np.float32(x).view(np.uint32))
+
+
+def test_round_scheme_exhaustive_band(oracle):
+    """clamp + trunc(q + copysign(pred(0.5), q)) == clamp(roundf(q)) for EVERY float of
+    magnitude up to 2^31 (both signs): all bit patterns 0..bits(2^31)."""
+    L = oracle.lib()
+    bad = C.c_float()
+    hi = bits(2.0 ** 31)
+    assert L.oracle_round_sweep(0, hi, C.byref(bad)) == 0, bad.value
+    assert L.oracle_round_sweep(0x80000000, 0x80000000 + hi, C.byref(bad)) == 0, bad.value
+
+
+def test_fastdiv_matches_true_division(oracle):
+    """q = fma(r, y, q0) scheme equals a / b bit for bit (sampled numerators x many divisors)."""
+    L = oracle.lib()
+    bad = C.c_float()
+    rng = np.random.RandomState(9)
+    divisors = [0.05, 0.02, 0.01, 1.0, 2.0, 3.0, 0.1, 0.3, 1e-3, 5e-2, float(np.float32(1.9999999)),
+                float(np.float32(1.0000001))]
+    divisors += [float(np.float32(np.exp(rng.uniform(np.log(1e-4), np.log(10.0))))) for _ in range(40)]
+    for b in divisors:
+        # positive and negative numerators over the whole exponent range that can matter:
+        # stride through bit patterns of [2^-40, 2^40]
+        lo, hi = bits(2.0 ** -40), bits(2.0 ** 40)
+        count = 400000
+        step = max(1, (hi - lo) // count)
+        start = lo + int(rng.randint(0, step))
+        assert L.oracle_fastdiv_sweep(b, start, step, count, C.byref(bad)) == 0, (b, bad.value)
+        assert L.oracle_fastdiv_sweep(b, start | 0x80000000, step, count, C.byref(bad)) == 0, (b, bad.value)
+    # dense sweep around quotients that are ties for the later round-to-integer (k + 0.5)
+    for b in (0.05, 0.3, float(np.float32(0.0123))):
+        for k in (0, 1, 2, 63, 100, 126):
+            centre = bits(np.float32((k + 0.5) * b))
+            assert L.oracle_fastdiv_sweep(b, centre - 50000, 1, 100000, C.byref(bad)) == 0, (b, k, bad.value)

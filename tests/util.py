@@ -1,0 +1,78 @@
+"""Shared helpers for the parity tests: portable seeded tensors and layout converters."""
+import numpy as np
+
+from megengine_amd import _abi
+
+
+def splitmix64(seed, n):
+    """Portable generator: n uint64 values from splitmix64(seed) (same bytes on every host)."""
+    out = np.empty(n, dtype=np.uint64)
+    x = np.uint64(seed)
+    with np.errstate(over="ignore"):
+        idx = np.arange(1, n + 1, dtype=np.uint64)
+        z = x + idx * np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        out = z ^ (z >> np.uint64(31))
+    return out
+
+
+def uniform_int(seed, shape, lo, hi, dtype):
+    n = int(np.prod(shape))
+    r = splitmix64(seed, n)
+    v = (r % np.uint64(hi - lo + 1)).astype(np.int64) + lo
+    return v.astype(dtype).reshape(shape)
+
+
+def make_tensors(desc, seed=1, src_range=(-128, 127), flt_range=(-128, 127), bias_range=(-1000, 1000),
+                 z_range=(-128, 127)):
+    src_s, flt_s, bias_s, dst_s = _abi.conv_shapes(desc)
+    src = uniform_int(seed * 4 + 0, src_s, *src_range, np.int8)
+    flt = uniform_int(seed * 4 + 1, flt_s, *flt_range, np.int8)
+    bias = uniform_int(seed * 4 + 2, bias_s, *bias_range, np.int32) if desc.bias_mode else None
+    z = None
+    if desc.has_z:
+        zdt = np.int8 if desc.dst_dtype == _abi.DT_QS8 else np.int32
+        z = uniform_int(seed * 4 + 3, dst_s, *z_range, zdt)
+    return src, flt, bias, z
+
+
+# ---- layout converters written from the closed-form definition (numpy reshape/transpose) ----
+
+def nchw_to_packed(x, p):
+    n, c, h, w = x.shape
+    assert c % p == 0
+    return np.ascontiguousarray(x.reshape(n, c // p, p, h, w).transpose(0, 1, 3, 4, 2))
+
+
+def packed_to_nchw(x):
+    n, cb, h, w, p = x.shape
+    return np.ascontiguousarray(x.transpose(0, 1, 4, 2, 3).reshape(n, cb * p, h, w))
+
+
+def filter_nchw_to_packed(f, p):
+    """(OC, IC, FH, FW) -> (OC, IC/p, FH, FW, p); group (G, OCpg, ICpg, FH, FW) likewise."""
+    if f.ndim == 4:
+        oc, ic, fh, fw = f.shape
+        return np.ascontiguousarray(f.reshape(oc, ic // p, p, fh, fw).transpose(0, 1, 3, 4, 2))
+    g, oc, ic, fh, fw = f.shape
+    return np.ascontiguousarray(f.reshape(g, oc, ic // p, p, fh, fw).transpose(0, 1, 2, 4, 5, 3))
+
+
+def filter_nchw_to_nchw44(f):
+    """(OC, IC, FH, FW) -> (OC/4, IC/4, FH, FW, 4ic, 4oc); group adds a leading G."""
+    if f.ndim == 4:
+        oc, ic, fh, fw = f.shape
+        return np.ascontiguousarray(f.reshape(oc // 4, 4, ic // 4, 4, fh, fw).transpose(0, 2, 4, 5, 3, 1))
+    g, oc, ic, fh, fw = f.shape
+    return np.ascontiguousarray(f.reshape(g, oc // 4, 4, ic // 4, 4, fh, fw).transpose(0, 1, 3, 5, 6, 4, 2))
+
+
+def filter_dw_nchw_to_dw4(f):
+    """depthwise (C, 1, 1, FH, FW) -> (C/4, 1, 1, FH, FW, 4)."""
+    c, _, _, fh, fw = f.shape
+    return np.ascontiguousarray(f.reshape(c // 4, 4, fh, fw).transpose(0, 2, 3, 1).reshape(c // 4, 1, 1, fh, fw, 4))
+
+
+def bias_to_packed(b, p):
+    return np.ascontiguousarray(b.reshape(1, -1, p, 1, 1).transpose(0, 1, 3, 4, 2))
