@@ -153,6 +153,10 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
                            const int8_t* src, const int8_t* filter, const int32_t* bias,
                            const int8_t* z, void* dst, void* workspace, size_t workspace_bytes);
 
+/* tile configurations of the MFMA implicit-GEMM algorithm (values of mi355_algo.tile_cfg) */
+int mi355_igemm_tile_count(void);
+const char* mi355_igemm_tile_name(int tile_cfg);
+
 /* ---- RelayoutFormat ---- */
 /* param::RelayoutFormat::Mode values (opr_param_defs.py:1069-1111); 32/33 and 34/35 are
  * extensions of this backend (the reference has no NCHW32 relayout mode). */

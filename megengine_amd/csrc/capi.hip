@@ -1,0 +1,370 @@
+// C ABI of the MI355X quantized ConvBias / RelayoutFormat path (declared in
+// include/mi355_convbias.h): descriptor validation, the shape-keyed algorithm chooser and the
+// kernel dispatch.  No allocation, no exceptions; every entry point returns an mi355_status.
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <mutex>
+
+#include "common.h"
+
+using namespace mi355;
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail(int status, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int in_pack(uint32_t fmt) {
+    switch (fmt) {
+        case MI355_FMT_NCHW: return 1;
+        case MI355_FMT_NCHW4: case MI355_FMT_NCHW44: case MI355_FMT_NCHW4_NCHW32: return 4;
+        case MI355_FMT_NCHW32: case MI355_FMT_NCHW32_NCHW4: return 32;
+        default: return 0;
+    }
+}
+int out_pack(uint32_t fmt) {
+    switch (fmt) {
+        case MI355_FMT_NCHW: return 1;
+        case MI355_FMT_NCHW4: case MI355_FMT_NCHW44: case MI355_FMT_NCHW32_NCHW4: return 4;
+        case MI355_FMT_NCHW32: case MI355_FMT_NCHW4_NCHW32: return 32;
+        default: return 0;
+    }
+}
+
+// The fast epilogue form needs: positive normal dst scale (RELU folds into the clamp, the
+// reciprocal pair is exact enough), and magnitudes that keep every intermediate finite:
+// |r| <= 2^31*s_b + 128*s_z, H_SWISH multiplies by at most 6, then r * y_hi.
+bool epi_fast_ok(float s_b, float s_z, float s_d, bool has_z) {
+    auto sane = [](float s) { return s >= 0x1p-60f && s <= 0x1p40f; };
+    if (!(s_d >= 0x1p-40f && s_d <= 0x1p40f)) return false;
+    if (!sane(s_b)) return false;
+    if (has_z && !sane(s_z)) return false;
+    return true;
+}
+
+// Validation of a descriptor: the checks of ConvolutionBase::deduce_layout_fwd
+// (dnn/src/common/convolution.cpp:633-1049) and do_check_exec_common
+// (dnn/src/common/conv_bias.cpp:8-133) that survive the translation to a flat descriptor.
+int canonize(const mi355_conv_desc* d, ConvProblem* p) {
+    if (!d) return fail(MI355_ERR_BAD_ARG, "null descriptor");
+    const int pi = in_pack(d->format), po = out_pack(d->format);
+    if (!pi) return fail(MI355_ERR_UNSUPPORTED, "format %u not supported by this backend", d->format);
+    if (d->sparse > MI355_SPARSE_GROUP) return fail(MI355_ERR_BAD_ARG, "invalid convolution sparse type");
+    if (d->mode > MI355_MODE_CONVOLUTION) return fail(MI355_ERR_BAD_ARG, "invalid conv mode");
+    if (!d->group || !d->fh || !d->fw || !d->stride_h || !d->stride_w || !d->dilate_h || !d->dilate_w)
+        return fail(MI355_ERR_BAD_ARG, "zero group/filter/stride/dilation");
+    if (d->sparse == MI355_SPARSE_DENSE && d->group != 1)
+        return fail(MI355_ERR_SHAPE, "dense convolution with group=%u", d->group);
+    if (d->ic % d->group || d->oc % d->group)
+        return fail(MI355_ERR_SHAPE, "group conv channel mismatch: ic=%u oc=%u group=%u", d->ic, d->oc, d->group);
+    p->d = *d;
+    p->icpg = d->ic / d->group;
+    p->ocpg = d->oc / d->group;
+    p->pin = pi;
+    p->pout = po;
+    p->dw4 = (d->format == MI355_FMT_NCHW44 || d->format == MI355_FMT_NCHW4) && d->group > 1 && p->icpg == 1 &&
+             p->ocpg == 1;
+    if (d->format != MI355_FMT_NCHW && (d->dilate_h != 1 || d->dilate_w != 1))
+        return fail(MI355_ERR_SHAPE, "NCHWx has invalid dilation %ux%u, require to be 1", d->dilate_h, d->dilate_w);
+    if (p->dw4) {
+        if (d->group % 4) return fail(MI355_ERR_SHAPE, "channel-wise packed conv needs channels %% 4 == 0");
+    } else {
+        if (p->icpg % pi)
+            return fail(MI355_ERR_SHAPE, "input channels per group (%u) not a multiple of the pack (%d)", p->icpg, pi);
+        if (d->format == MI355_FMT_NCHW44 && (p->ocpg % 4))
+            return fail(MI355_ERR_SHAPE, "NCHW44 needs output channels per group %% 4 == 0");
+    }
+    if (d->oc % po) return fail(MI355_ERR_SHAPE, "output channels (%u) not a multiple of the pack (%d)", d->oc, po);
+    if (d->nonline == MI355_NL_SIGMOID)
+        return fail(MI355_ERR_UNSUPPORTED, "SIGMOID is not defined for quantized ConvBias");
+    if (d->nonline > MI355_NL_H_SWISH) return fail(MI355_ERR_BAD_ARG, "invalid nonlineMode %u", d->nonline);
+    if (d->bias_mode > MI355_BIAS_FULL) return fail(MI355_ERR_BAD_ARG, "invalid bias mode");
+    if (d->dst_dtype > MI355_DT_QS32) return fail(MI355_ERR_BAD_ARG, "invalid dst dtype");
+    if (d->has_z && (d->format == MI355_FMT_NCHW4_NCHW32 || d->format == MI355_FMT_NCHW32_NCHW4))
+        return fail(MI355_ERR_SHAPE, "z is not allowed for NCHW4_NCHW32 / NCHW32_NCHW4");
+    const uint32_t dfh = (d->fh - 1) * d->dilate_h + 1, dfw = (d->fw - 1) * d->dilate_w + 1;
+    if (d->ih + 2 * d->pad_h < dfh || d->iw + 2 * d->pad_w < dfw)
+        return fail(MI355_ERR_SHAPE, "filter %ux%u larger than padded input %ux%u", dfh, dfw, d->ih + 2 * d->pad_h,
+                    d->iw + 2 * d->pad_w);
+    p->oh = conv_out_size(d->ih, d->fh, d->dilate_h, d->stride_h, d->pad_h);
+    p->ow = conv_out_size(d->iw, d->fw, d->dilate_w, d->stride_w, d->pad_w);
+    const int64_t src_img = (int64_t)d->ic * d->ih * d->iw, dst_img = (int64_t)d->oc * p->oh * p->ow;
+    p->src_sn = d->src_stride_n ? d->src_stride_n : src_img;
+    p->dst_sn = d->dst_stride_n ? d->dst_stride_n : dst_img;
+    p->z_sn = d->z_stride_n ? d->z_stride_n : dst_img;
+    if (p->src_sn < src_img || p->dst_sn < dst_img || p->z_sn < dst_img)
+        return fail(MI355_ERR_SHAPE, "batch stride smaller than one image");
+    p->epi.s_b = d->scale_bias;
+    p->epi.s_z = d->scale_z;
+    p->epi.s_d = d->scale_dst;
+    p->epi.nonline = (int)d->nonline;
+    p->epi.has_z = d->has_z ? 1 : 0;
+    p->epi.fast = d->dst_dtype == MI355_DT_QS8 && epi_fast_ok(d->scale_bias, d->scale_z, d->scale_dst, d->has_z != 0);
+    p->epi.y_hi = 1.0f / d->scale_dst;
+    p->epi.y_lo = (float)(1.0 / (double)d->scale_dst - (double)p->epi.y_hi);
+    return MI355_OK;
+}
+
+struct DevInfo {
+    bool ok = false;
+    int cu = 0;
+};
+DevInfo g_dev[64];
+std::mutex g_dev_mu;
+
+int cu_count() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    std::lock_guard<std::mutex> lk(g_dev_mu);
+    if (!g_dev[dev].ok) {
+        hipDeviceProp_t pr;
+        if (hipGetDeviceProperties(&pr, dev) != hipSuccess) return 0;
+        g_dev[dev].cu = pr.multiProcessorCount;
+        g_dev[dev].ok = true;
+    }
+    return g_dev[dev].cu;
+}
+
+const char* kAlgoNames[ALGO_COUNT] = {"MI355_DIRECT_DOT4", "MI355_IGEMM_MFMA_I8", "MI355_DEPTHWISE_DOT4"};
+
+bool algo_usable(const ConvProblem& p, int id) {
+    switch (id) {
+        case ALGO_DIRECT: return true;
+        case ALGO_IGEMM_MFMA: return igemm_usable(p);
+        case ALGO_DEPTHWISE: return depthwise_usable(p);
+        default: return false;
+    }
+}
+
+// Heuristic order (cf. the reference's per-backend get_algorithm_heuristic, e.g.
+// dnn/src/cuda/conv_bias/opr_impl.cpp:44-238): channel-wise kernel, then the MFMA implicit GEMM,
+// then the generic direct kernel.
+int pick_algo(const ConvProblem& p) {
+    if (depthwise_usable(p)) return ALGO_DEPTHWISE;
+    if (igemm_usable(p)) return ALGO_IGEMM_MFMA;
+    return ALGO_DIRECT;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace
+
+extern "C" {
+
+int mi355_abi_version(void) { return MI355_CONVBIAS_ABI_VERSION; }
+
+const char* mi355_status_string(int status) {
+    switch (status) {
+        case MI355_OK: return "ok";
+        case MI355_ERR_BAD_ARG: return "bad argument";
+        case MI355_ERR_UNSUPPORTED: return "unsupported by the MI355 backend";
+        case MI355_ERR_SHAPE: return "inconsistent shapes";
+        case MI355_ERR_WORKSPACE: return "workspace too small";
+        case MI355_ERR_LAUNCH: return "HIP launch/runtime error";
+        case MI355_ERR_NO_DEVICE: return "no usable device";
+        case MI355_ERR_ALGO: return "algorithm not usable for this problem";
+        default: return "unknown status";
+    }
+}
+
+const char* mi355_last_error(void) { return g_err; }
+
+int mi355_get_device_info(int device, mi355_device_info* out) {
+    if (!out) return fail(MI355_ERR_BAD_ARG, "null out");
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || device < 0 || device >= n) {
+        (void)hipGetLastError();
+        return fail(MI355_ERR_NO_DEVICE, "device %d not available", device);
+    }
+    hipDeviceProp_t pr;
+    hipError_t e = hipGetDeviceProperties(&pr, device);
+    if (e != hipSuccess) return fail(MI355_ERR_NO_DEVICE, "%s", hipGetErrorString(e));
+    memset(out, 0, sizeof(*out));
+    out->device = device;
+    out->compute_units = pr.multiProcessorCount;
+    out->clock_khz = pr.clockRate;
+    out->lds_bytes_per_cu = (int32_t)pr.maxSharedMemoryPerMultiProcessor;
+    out->hbm_bytes = (int64_t)pr.totalGlobalMem;
+    snprintf(out->arch, sizeof(out->arch), "%s", pr.gcnArchName);
+    snprintf(out->name, sizeof(out->name), "%s", pr.name);
+    return MI355_OK;
+}
+
+int mi355_convbias_deduce_out(const mi355_conv_desc* d, uint32_t* oh, uint32_t* ow) {
+    ConvProblem p;
+    int st = canonize(d, &p);
+    if (st) return st;
+    if (oh) *oh = p.oh;
+    if (ow) *ow = p.ow;
+    return MI355_OK;
+}
+
+int mi355_convbias_algo_count(void) { return ALGO_COUNT; }
+
+const char* mi355_convbias_algo_name(int id) { return id >= 0 && id < ALGO_COUNT ? kAlgoNames[id] : NULL; }
+
+int mi355_convbias_algo_usable(const mi355_conv_desc* d, int id) {
+    ConvProblem p;
+    int st = canonize(d, &p);
+    if (st) return st;
+    if (id < 0 || id >= ALGO_COUNT) return fail(MI355_ERR_ALGO, "unknown algorithm id %d", id);
+    return algo_usable(p, id) ? MI355_OK : fail(MI355_ERR_ALGO, "%s cannot run this problem", kAlgoNames[id]);
+}
+
+int mi355_convbias_s8_query(const mi355_conv_desc* d, int algo_request, mi355_algo* algo_out,
+                            size_t* workspace_bytes) {
+    ConvProblem p;
+    int st = canonize(d, &p);
+    if (st) return st;
+    int id = algo_request;
+    if (id == MI355_ALGO_HEURISTIC) {
+        id = pick_algo(p);
+    } else if (id < 0 || id >= ALGO_COUNT) {
+        return fail(MI355_ERR_ALGO, "unknown algorithm id %d", id);
+    } else if (!algo_usable(p, id)) {
+        return fail(MI355_ERR_ALGO, "%s cannot run this problem", kAlgoNames[id]);
+    }
+    if (algo_out) {
+        algo_out->id = id;
+        algo_out->tile_cfg = id == ALGO_IGEMM_MFMA ? igemm_pick_cfg(p, cu_count()) : 0;
+        algo_out->reserved = 0;
+    }
+    // every kernel reads the reference layouts in place: no filter repack, no float staging
+    if (workspace_bytes) *workspace_bytes = 0;
+    return MI355_OK;
+}
+
+int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src,
+                           const int8_t* filter, const int32_t* bias, const int8_t* z, void* dst, void* workspace,
+                           size_t workspace_bytes) {
+    (void)workspace;
+    (void)workspace_bytes;
+    ConvProblem p;
+    int st = canonize(d, &p);
+    if (st) return st;
+    if (!src || !filter || !dst) return fail(MI355_ERR_BAD_ARG, "null tensor pointer");
+    if (d->bias_mode != MI355_BIAS_NONE && !bias) return fail(MI355_ERR_BAD_ARG, "bias_mode set but bias is null");
+    if (d->has_z && !z) return fail(MI355_ERR_BAD_ARG, "has_z set but z is null");
+    int id = algo ? algo->id : MI355_ALGO_HEURISTIC;
+    int cfg = algo ? algo->tile_cfg : -1;
+    if (id == MI355_ALGO_HEURISTIC) {
+        id = pick_algo(p);
+        cfg = -1;
+    }
+    if (id < 0 || id >= ALGO_COUNT) return fail(MI355_ERR_ALGO, "unknown algorithm id %d", id);
+    if (!algo_usable(p, id)) return fail(MI355_ERR_ALGO, "%s cannot run this problem", kAlgoNames[id]);
+    // the tiled kernels use 16-byte vector accesses; misaligned tensors take the generic kernel
+    if (id != ALGO_DIRECT) {
+        bool al = aligned16(src) && aligned16(filter) && aligned16(dst) && (!bias || aligned16(bias)) &&
+                  (!z || aligned16(z)) && p.src_sn % 16 == 0 && p.dst_sn % 16 == 0 && p.z_sn % 16 == 0;
+        if (!al) {
+            if (algo && algo->id != MI355_ALGO_HEURISTIC)
+                return fail(MI355_ERR_ALGO, "%s needs 16-byte aligned tensors", kAlgoNames[id]);
+            id = ALGO_DIRECT;
+        }
+    }
+    hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    int rc = 0;
+    switch (id) {
+        case ALGO_DIRECT:
+            rc = launch_conv_direct(hs, p, src, filter, bias, z, dst);
+            break;
+        case ALGO_IGEMM_MFMA:
+            if (cfg < 0 || cfg >= igemm_num_cfgs()) cfg = igemm_pick_cfg(p, cu_count());
+            rc = launch_conv_igemm(hs, p, cfg, src, filter, bias, z, reinterpret_cast<int8_t*>(dst));
+            break;
+        case ALGO_DEPTHWISE:
+            rc = launch_conv_depthwise(hs, p, src, filter, bias, z, reinterpret_cast<int8_t*>(dst));
+            break;
+    }
+    if (rc) return fail(MI355_ERR_LAUNCH, "%s: %s", kAlgoNames[id], hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
+}
+
+int mi355_igemm_tile_count(void) { return igemm_num_cfgs(); }
+const char* mi355_igemm_tile_name(int cfg) { return igemm_cfg_name(cfg); }
+
+// ---- RelayoutFormat ----
+static uint32_t cdiv(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
+int mi355_relayout_deduce(const mi355_relayout_desc* d, uint32_t* ndim, uint32_t shape[7]) {
+    if (!d || !ndim || !shape) return fail(MI355_ERR_BAD_ARG, "null argument");
+    if (d->elem_bytes != 1 && d->elem_bytes != 4) return fail(MI355_ERR_UNSUPPORTED, "element size %u", d->elem_bytes);
+    const uint32_t* s = d->shape;
+    const uint32_t g = d->group ? d->group : 1;
+    for (int i = 0; i < 7; ++i) shape[i] = 0;
+    switch (d->mode) {
+        case MI355_RL_NCHW_NCHW4_IC_SMALL:
+            if (d->ndim != 4) return fail(MI355_ERR_SHAPE, "src must be 4-dim");
+            if (s[1] > 4) return fail(MI355_ERR_SHAPE, "ic should be less equal 4");
+            *ndim = 5; shape[0] = s[0]; shape[1] = cdiv(s[1], 4); shape[2] = s[2]; shape[3] = s[3]; shape[4] = 4;
+            return MI355_OK;
+        case MI355_RL_NCHW_NCHW4:
+        case MI355_RL_NCHW_NCHW32: {
+            const uint32_t p = d->mode == MI355_RL_NCHW_NCHW4 ? 4 : 32;
+            if (d->ndim != 4) return fail(MI355_ERR_SHAPE, "src must be 4-dim");
+            if (s[1] % g) return fail(MI355_ERR_SHAPE, "channels %u not divisible by group %u", s[1], g);
+            *ndim = 5; shape[0] = s[0]; shape[1] = g * cdiv(s[1] / g, p); shape[2] = s[2]; shape[3] = s[3];
+            shape[4] = p;
+            return MI355_OK;
+        }
+        case MI355_RL_NCHW4_NCHW:
+        case MI355_RL_NCHW32_NCHW: {
+            const uint32_t p = d->mode == MI355_RL_NCHW4_NCHW ? 4 : 32;
+            if (d->ndim != 5 || s[4] != p) return fail(MI355_ERR_SHAPE, "src must be (n, c/%u, h, w, %u)", p, p);
+            const uint32_t c = d->oc ? d->oc : s[1] * p;
+            if (c % g) return fail(MI355_ERR_SHAPE, "oc %u not divisible by group %u", c, g);
+            if (c > s[1] * p || g * cdiv(c / g, p) != s[1])
+                return fail(MI355_ERR_SHAPE, "oc %u / group %u do not match %u packed blocks", c, g, s[1]);
+            *ndim = 4; shape[0] = s[0]; shape[1] = c; shape[2] = s[2]; shape[3] = s[3];
+            return MI355_OK;
+        }
+        case MI355_RL_NCHW_NCHW4_WEIGHT:
+            if (d->ndim == 4) {
+                *ndim = 5; shape[0] = cdiv(s[0], 4) * 4; shape[1] = cdiv(s[1], 4); shape[2] = s[2]; shape[3] = s[3];
+                shape[4] = 4;
+                return MI355_OK;
+            }
+            if (d->ndim == 5) {
+                *ndim = 6; shape[0] = s[0]; shape[1] = cdiv(s[1], 4) * 4; shape[2] = cdiv(s[2], 4); shape[3] = s[3];
+                shape[4] = s[4]; shape[5] = 4;
+                return MI355_OK;
+            }
+            return fail(MI355_ERR_SHAPE, "weight must be 4-dim (dense) or 5-dim (group)");
+        case MI355_RL_NCHW4_NCHW32:
+            if (d->ndim != 5 || s[4] != 4 || s[1] % 8) return fail(MI355_ERR_SHAPE, "src must be (n, c/4, h, w, 4), c %% 32 == 0");
+            *ndim = 5; shape[0] = s[0]; shape[1] = s[1] / 8; shape[2] = s[2]; shape[3] = s[3]; shape[4] = 32;
+            return MI355_OK;
+        case MI355_RL_NCHW32_NCHW4:
+            if (d->ndim != 5 || s[4] != 32) return fail(MI355_ERR_SHAPE, "src must be (n, c/32, h, w, 32)");
+            *ndim = 5; shape[0] = s[0]; shape[1] = s[1] * 8; shape[2] = s[2]; shape[3] = s[3]; shape[4] = 4;
+            return MI355_OK;
+        default:
+            return fail(MI355_ERR_UNSUPPORTED, "Invalid RelayoutFormat Mode %u", d->mode);
+    }
+}
+
+int mi355_relayout_exec(void* stream, const mi355_relayout_desc* d, const void* src, void* dst) {
+    uint32_t ondim = 0, oshape[7];
+    int st = mi355_relayout_deduce(d, &ondim, oshape);
+    if (st) return st;
+    if (!src || !dst) return fail(MI355_ERR_BAD_ARG, "null tensor pointer");
+    // the byte-transposing kernels use 16-byte vectors; misaligned tensors take the generic kernel
+    const bool fast = aligned16(src) && aligned16(dst);
+    int rc = launch_relayout(reinterpret_cast<hipStream_t>(stream), *d, oshape, ondim, src, dst, fast);
+    if (rc) return fail(MI355_ERR_LAUNCH, "relayout: %s", hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,55 @@
+// Internal declarations shared by the host C-ABI layer and the HIP kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/mi355_convbias.h"
+#include "epilogue.h"
+
+namespace mi355 {
+
+// ---- algorithm table ids (order is the ABI of mi355_convbias_algo_name) ----
+enum AlgoId {
+    ALGO_DIRECT = 0,       // generic one-thread-per-output kernel: every format / mode
+    ALGO_IGEMM_MFMA = 1,   // dense implicit GEMM on int8 MFMA (NCHW4 / NCHW32 / mixed)
+    ALGO_DEPTHWISE = 2,    // channel-wise, bandwidth bound (NCHW4-packed and NCHW)
+    ALGO_COUNT = 3
+};
+
+// Canonical problem description used by every launcher (derived from mi355_conv_desc)
+struct ConvProblem {
+    mi355_conv_desc d;
+    uint32_t oh, ow;
+    uint32_t icpg, ocpg;
+    int pin, pout;     // channel pack of src/filter and of dst/bias/z
+    bool dw4;          // packed-by-4 channel-wise filter layout
+    int64_t src_sn, dst_sn, z_sn;  // batch strides in elements
+    EpiParams epi;
+};
+
+// ---- launchers (each returns a hipError_t-compatible int; 0 = success) ----
+int launch_conv_direct(hipStream_t st, const ConvProblem& p, const int8_t* src, const int8_t* flt,
+                       const int32_t* bias, const void* z, void* dst);
+
+// tile_cfg: index into the igemm tile table, -1 = pick by heuristic
+int igemm_num_cfgs();
+const char* igemm_cfg_name(int cfg);
+bool igemm_usable(const ConvProblem& p);
+int igemm_pick_cfg(const ConvProblem& p, int cu_count);
+int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int tile_cfg, const int8_t* src, const int8_t* flt,
+                      const int32_t* bias, const int8_t* z, int8_t* dst);
+
+bool depthwise_usable(const ConvProblem& p);
+int launch_conv_depthwise(hipStream_t st, const ConvProblem& p, const int8_t* src, const int8_t* flt,
+                          const int32_t* bias, const int8_t* z, int8_t* dst);
+
+int launch_relayout(hipStream_t st, const mi355_relayout_desc& d, const uint32_t* oshape, uint32_t ondim,
+                    const void* src, void* dst, bool allow_fast);
+
+static inline uint32_t conv_out_size(uint32_t i, uint32_t f, uint32_t dil, uint32_t s, uint32_t p) {
+    uint32_t df = (f - 1) * dil + 1;
+    return (i + 2 * p - df) / s + 1;
+}
+
+}  // namespace mi355

@@ -1,0 +1,159 @@
+// Generic direct int8 ConvBias kernel: one thread per output element, 64-bit indexing.
+// Covers every descriptor the C ABI accepts (all formats, group, dilation, CONVOLUTION mode,
+// full-shape bias, QuantizedS32 dst, strided batch) and is the algorithm of last resort of the
+// chooser.  Semantics: naive compute2d (dnn/src/naive/convolution/helper.h:466-502) followed by
+// the epilogue in epilogue.h.
+#include "common.h"
+
+namespace mi355 {
+namespace {
+
+struct DirectArgs {
+    const int8_t* src;
+    const int8_t* flt;
+    const int32_t* bias;
+    const void* z;
+    void* dst;
+    uint32_t format;
+    uint32_t N, IC, IH, IW, OC, OH, OW, FH, FW, G, icpg, ocpg;
+    int ph, pw, sh, sw, dh, dw;  // dh/dw negated and offsets shifted when the filter is flipped
+    int h_off, w_off;
+    int pin, pout;
+    int dw4;
+    int bias_mode;
+    int dst_s32;
+    int64_t src_sn, dst_sn, z_sn;
+    EpiParams epi;
+};
+
+__device__ __forceinline__ int64_t filter_offset(const DirectArgs& a, uint32_t g, uint32_t oc_in_g, uint32_t ic_in_g,
+                                                 uint32_t fh, uint32_t fw) {
+    const int64_t FH = a.FH, FW = a.FW;
+    if (a.dw4) return (int64_t)(g >> 2) * (FH * FW * 4) + (fh * FW + fw) * 4 + (g & 3);
+    if (a.format == MI355_FMT_NCHW) {
+        int64_t fs_oc = FH * FW * a.icpg;
+        return ((int64_t)g * a.ocpg + oc_in_g) * fs_oc + ic_in_g * (FH * FW) + fh * FW + fw;
+    }
+    if (a.format == MI355_FMT_NCHW44) {
+        // (g, ocpg/4, icpg/4, fh, fw, 4ic, 4oc)
+        int64_t blk = ((((int64_t)g * (a.ocpg >> 2) + (oc_in_g >> 2)) * (a.icpg >> 2) + (ic_in_g >> 2)) * FH + fh) * FW + fw;
+        return blk * 16 + (ic_in_g & 3) * 4 + (oc_in_g & 3);
+    }
+    // (g, ocpg, icpg/p, fh, fw, p)
+    const int p = a.pin;
+    int64_t blk = ((((int64_t)g * a.ocpg + oc_in_g) * (a.icpg / p) + ic_in_g / p) * FH + fh) * FW + fw;
+    return blk * p + (ic_in_g % p);
+}
+
+__global__ __launch_bounds__(256) void conv_direct_kernel(DirectArgs a) {
+    const int64_t per_n = (int64_t)a.OC * a.OH * a.OW;
+    const int64_t total = per_n * a.N;
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    // decode dst-layout linear index -> (n, oc, oh, ow)
+    const uint32_t n = (uint32_t)(idx / per_n);
+    int64_t r = idx - (int64_t)n * per_n;
+    uint32_t oc, oh, ow;
+    {
+        const int po = a.pout;
+        uint32_t k = (uint32_t)(r % po);
+        int64_t t = r / po;
+        ow = (uint32_t)(t % a.OW);
+        t /= a.OW;
+        oh = (uint32_t)(t % a.OH);
+        uint32_t ocb = (uint32_t)(t / a.OH);
+        oc = ocb * po + k;
+    }
+    const uint32_t g = oc / a.ocpg, oc_in_g = oc - g * a.ocpg;
+    const int pi = a.pin;
+    const int8_t* sp = a.src + (int64_t)n * a.src_sn;
+    int acc = 0;
+    for (uint32_t fh = 0; fh < a.FH; ++fh) {
+        int ih = (int)(oh * a.sh) + (int)fh * a.dh + a.h_off;
+        if (ih < 0 || ih >= (int)a.IH) continue;
+        for (uint32_t fw = 0; fw < a.FW; ++fw) {
+            int iw = (int)(ow * a.sw) + (int)fw * a.dw + a.w_off;
+            if (iw < 0 || iw >= (int)a.IW) continue;
+            const bool vec4 = (pi >= 4) && !a.dw4 && a.format != MI355_FMT_NCHW44;
+            if (vec4) {
+                // src pack and filter pack share the channel order: 4 channels per dot4
+                for (uint32_t ic = 0; ic < a.icpg; ic += 4) {
+                    uint32_t c = g * a.icpg + ic;
+                    int64_t so = ((int64_t)(c / pi) * a.IH + ih) * a.IW * pi + (int64_t)iw * pi + (c % pi);
+                    int64_t fo = filter_offset(a, g, oc_in_g, ic, fh, fw);
+                    int sv = *reinterpret_cast<const int*>(sp + so);
+                    int fv = *reinterpret_cast<const int*>(a.flt + fo);
+                    acc = __builtin_amdgcn_sdot4(sv, fv, acc, false);
+                }
+            } else {
+                for (uint32_t ic = 0; ic < a.icpg; ++ic) {
+                    uint32_t c = g * a.icpg + ic;
+                    int64_t so = ((int64_t)(c / pi) * a.IH + ih) * a.IW * pi + (int64_t)iw * pi + (c % pi);
+                    int64_t fo = filter_offset(a, g, oc_in_g, ic, fh, fw);
+                    acc += (int)sp[so] * (int)a.flt[fo];
+                }
+            }
+        }
+    }
+    if (a.bias_mode == MI355_BIAS_BROADCAST_CHANNEL)
+        acc += a.bias[oc];
+    else if (a.bias_mode == MI355_BIAS_FULL)
+        acc += a.bias[idx];
+    const bool hz = a.epi.has_z != 0;
+    if (a.dst_s32) {
+        int zv = hz ? reinterpret_cast<const int*>(a.z)[(int64_t)n * a.z_sn + r] : 0;
+        reinterpret_cast<int*>(a.dst)[(int64_t)n * a.dst_sn + r] = requant_s32_exact(acc, hz, zv, a.epi);
+    } else {
+        int zv = hz ? (int)reinterpret_cast<const int8_t*>(a.z)[(int64_t)n * a.z_sn + r] : 0;
+        int out;
+        if (a.epi.fast) {
+            // exercise the same fast form the tiled kernels use
+            if (hz) {
+                out = a.epi.nonline == NL_RELU      ? requant_s8_fast<NL_RELU, true>(acc, zv, a.epi)
+                      : a.epi.nonline == NL_H_SWISH ? requant_s8_fast<NL_H_SWISH, true>(acc, zv, a.epi)
+                                                    : requant_s8_fast<NL_IDENTITY, true>(acc, zv, a.epi);
+            } else {
+                out = a.epi.nonline == NL_RELU      ? requant_s8_fast<NL_RELU, false>(acc, zv, a.epi)
+                      : a.epi.nonline == NL_H_SWISH ? requant_s8_fast<NL_H_SWISH, false>(acc, zv, a.epi)
+                                                    : requant_s8_fast<NL_IDENTITY, false>(acc, zv, a.epi);
+            }
+        } else {
+            out = requant_s8_exact(acc, hz, zv, a.epi);
+        }
+        reinterpret_cast<int8_t*>(a.dst)[(int64_t)n * a.dst_sn + r] = (int8_t)out;
+    }
+}
+
+}  // namespace
+
+int launch_conv_direct(hipStream_t st, const ConvProblem& p, const int8_t* src, const int8_t* flt,
+                       const int32_t* bias, const void* z, void* dst) {
+    DirectArgs a;
+    const mi355_conv_desc& d = p.d;
+    a.src = src; a.flt = flt; a.bias = bias; a.z = z; a.dst = dst;
+    a.format = d.format;
+    a.N = d.n; a.IC = d.ic; a.IH = d.ih; a.IW = d.iw; a.OC = d.oc; a.OH = p.oh; a.OW = p.ow;
+    a.FH = d.fh; a.FW = d.fw; a.G = d.group; a.icpg = p.icpg; a.ocpg = p.ocpg;
+    a.ph = d.pad_h; a.pw = d.pad_w; a.sh = d.stride_h; a.sw = d.stride_w;
+    a.dh = d.dilate_h; a.dw = d.dilate_w;
+    a.h_off = -(int)d.pad_h; a.w_off = -(int)d.pad_w;
+    if (d.mode == MI355_MODE_CONVOLUTION) {
+        a.h_off += (int)((d.fh - 1) * d.dilate_h);
+        a.w_off += (int)((d.fw - 1) * d.dilate_w);
+        a.dh = -a.dh;
+        a.dw = -a.dw;
+    }
+    a.pin = p.pin; a.pout = p.pout; a.dw4 = p.dw4 ? 1 : 0;
+    a.bias_mode = d.bias_mode;
+    a.dst_s32 = d.dst_dtype == MI355_DT_QS32;
+    a.src_sn = p.src_sn; a.dst_sn = p.dst_sn; a.z_sn = p.z_sn;
+    a.epi = p.epi;
+    const int64_t total = (int64_t)d.n * d.oc * p.oh * p.ow;
+    if (total == 0) return 0;
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(conv_direct_kernel, dim3((unsigned)blocks), dim3(256), 0, st, a);
+    return (int)hipGetLastError();
+}
+
+}  // namespace mi355

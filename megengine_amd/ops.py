@@ -1,0 +1,94 @@
+"""Host-side Python mirror of the two operators, over torch device tensors.
+
+PyTorch is plumbing only here: it owns device memory and the stream.  All arithmetic happens in
+the HIP kernels behind the C ABI; a missing library or a non-GPU tensor raises.
+
+The calls mirror megdnn::ConvBiasForward (dnn/include/megdnn/oprs/nn.h:358-536):
+    deduce_layout            -> conv_bias_deduce_layout(desc)
+    get_workspace_in_bytes   -> conv_bias_workspace(desc, algo)
+    get_algorithm_heuristic  -> conv_bias_query(desc)
+    exec(src, filter, bias, z, dst, workspace) -> conv_bias_exec(...)
+and megdnn::RelayoutFormat (dnn/include/megdnn/oprs/general.h:1348-1373).
+"""
+import ctypes as C
+
+import torch
+
+from . import _abi
+from .lib import check, lib
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise RuntimeError("mi355 operators take GPU tensors only (got %s)" % t.device)
+    if not t.is_contiguous():
+        raise RuntimeError("tensor must be contiguous")
+    return C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def conv_bias_deduce_layout(desc):
+    oh, ow = C.c_uint32(), C.c_uint32()
+    check(lib().mi355_convbias_deduce_out(C.byref(desc), C.byref(oh), C.byref(ow)))
+    return _abi.conv_shapes(desc)[3]
+
+
+def conv_bias_query(desc, algo=_abi.ALGO_HEURISTIC):
+    """-> (Algo, workspace_bytes)"""
+    a = _abi.Algo()
+    ws = C.c_size_t()
+    check(lib().mi355_convbias_s8_query(C.byref(desc), algo, C.byref(a), C.byref(ws)))
+    return a, ws.value
+
+
+def conv_bias_workspace(desc, algo=_abi.ALGO_HEURISTIC):
+    return conv_bias_query(desc, algo)[1]
+
+
+def conv_bias_exec(desc, src, flt, bias=None, z=None, dst=None, algo=None, workspace=None):
+    if algo is None:
+        algo, ws_bytes = conv_bias_query(desc)
+    elif isinstance(algo, int):
+        algo, ws_bytes = conv_bias_query(desc, algo)
+    else:
+        ws_bytes = 0
+    if dst is None:
+        shape = _abi.conv_shapes(desc)[3]
+        dt = torch.int8 if desc.dst_dtype == _abi.DT_QS8 else torch.int32
+        if desc.dst_stride_n:
+            dst = torch.empty((desc.n, desc.dst_stride_n), dtype=dt, device=src.device)
+        else:
+            dst = torch.empty(shape, dtype=dt, device=src.device)
+    if workspace is None and ws_bytes:
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=src.device)
+    wsn = workspace.numel() if workspace is not None else 0
+    check(lib().mi355_convbias_s8_exec(_stream(), C.byref(desc), C.byref(algo), _ptr(src), _ptr(flt), _ptr(bias),
+                                      _ptr(z), _ptr(dst), _ptr(workspace), wsn))
+    return dst
+
+
+def relayout_desc(mode, shape, group=1, oc=0, elem_bytes=1, scale_src=1.0, scale_dst=1.0):
+    d = _abi.RelayoutDesc(mode=mode, ndim=len(shape), group=group, oc=oc, elem_bytes=elem_bytes,
+                          scale_src=scale_src, scale_dst=scale_dst)
+    for i, s in enumerate(shape):
+        d.shape[i] = s
+    return d
+
+
+def relayout_deduce_layout(d):
+    nd = C.c_uint32()
+    shp = (C.c_uint32 * 7)()
+    check(lib().mi355_relayout_deduce(C.byref(d), C.byref(nd), shp))
+    return tuple(shp[i] for i in range(nd.value))
+
+
+def relayout_exec(d, src, dst=None):
+    if dst is None:
+        dst = torch.empty(relayout_deduce_layout(d), dtype=src.dtype, device=src.device)
+    check(lib().mi355_relayout_exec(_stream(), C.byref(d), _ptr(src), _ptr(dst)))
+    return dst

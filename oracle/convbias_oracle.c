@@ -187,16 +187,11 @@ static int check_desc(const mi355_conv_desc* d, uint32_t* icpg, uint32_t* ocpg) 
     return MI355_OK;
 }
 
-/* integer part: naive compute2d (helper.h:466-502) + bias add (helper.h:732-803),
- * writes the int32 "sfb" tensor in dst layout (shape and pack of dst, dense batch). */
-int oracle_convbias_s8_acc(const mi355_conv_desc* d, const int8_t* src, const int8_t* flt, const int32_t* bias,
-                           int32_t* sfb) {
-    uint32_t icpg, ocpg;
-    int st = check_desc(d, &icpg, &ocpg);
-    if (st) return st;
-    const int pi = in_pack(d->format), po = out_pack(d->format);
-    const uint32_t OH = out_size(d->ih, d->fh, d->dilate_h, d->stride_h, d->pad_h);
-    const uint32_t OW = out_size(d->iw, d->fw, d->dilate_w, d->stride_w, d->pad_w);
+/* one output element of naive compute2d (helper.h:466-502): the fh/fw/ic loops with zero
+ * padding by skipping out-of-range taps and int32 wraparound accumulation. */
+static int32_t acc_one(const mi355_conv_desc* d, uint32_t icpg, uint32_t ocpg, const int8_t* src, const int8_t* flt,
+                       uint32_t n, uint32_t oc, uint32_t oh, uint32_t ow) {
+    const int pi = in_pack(d->format);
     /* should_flip (helper.h:285-290): h_offset += dilated_spatial - 1, dilation negated */
     int h_offset = -(int)d->pad_h, w_offset = -(int)d->pad_w;
     int dh = (int)d->dilate_h, dw = (int)d->dilate_w;
@@ -206,27 +201,39 @@ int oracle_convbias_s8_acc(const mi355_conv_desc* d, const int8_t* src, const in
         dh = -dh;
         dw = -dw;
     }
+    const uint32_t g = oc / ocpg, oc_in_g = oc % ocpg; /* GroupCounter, helper.h:12-24 */
+    int32_t acc = 0;                                    /* StrategyFwd::init_dval, helper.h:37-40 */
+    for (uint32_t fh = 0; fh < d->fh; ++fh)
+        for (uint32_t fw = 0; fw < d->fw; ++fw) {
+            int64_t ih = (int64_t)d->stride_h * oh + (int64_t)fh * dh + h_offset;
+            int64_t iw = (int64_t)d->stride_w * ow + (int64_t)fw * dw + w_offset;
+            if (ih < 0 || ih >= (int64_t)d->ih || iw < 0 || iw >= (int64_t)d->iw) continue;
+            for (uint32_t ic = 0; ic < icpg; ++ic) {
+                int32_t s = src[act_off(d->src_stride_n, pi, d->ic, d->ih, d->iw, n, (int64_t)g * icpg + ic, ih, iw)];
+                int32_t f = flt[flt_off(d, icpg, ocpg, g, oc_in_g, ic, fh, fw)];
+                /* StrategyFwd::on for qint8: int32 multiply-add with wraparound (helper.h:67-74) */
+                acc = (int32_t)((uint32_t)acc + (uint32_t)(s * f));
+            }
+        }
+    return acc;
+}
+
+/* integer part: naive compute2d + bias add (helper.h:732-803), writes the int32 "sfb" tensor in
+ * dst layout (shape and pack of dst, dense batch). */
+int oracle_convbias_s8_acc(const mi355_conv_desc* d, const int8_t* src, const int8_t* flt, const int32_t* bias,
+                           int32_t* sfb) {
+    uint32_t icpg, ocpg;
+    int st = check_desc(d, &icpg, &ocpg);
+    if (st) return st;
+    const int po = out_pack(d->format);
+    const uint32_t OH = out_size(d->ih, d->fh, d->dilate_h, d->stride_h, d->pad_h);
+    const uint32_t OW = out_size(d->iw, d->fw, d->dilate_w, d->stride_w, d->pad_w);
 #pragma omp parallel for collapse(2) schedule(static)
     for (uint32_t n = 0; n < d->n; ++n) {
         for (uint32_t oc = 0; oc < d->oc; ++oc) {
-            const uint32_t g = oc / ocpg, oc_in_g = oc % ocpg; /* GroupCounter, helper.h:12-24 */
             for (uint32_t oh = 0; oh < OH; ++oh)
                 for (uint32_t ow = 0; ow < OW; ++ow) {
-                    int32_t acc = 0; /* StrategyFwd::init_dval, helper.h:37-40 */
-                    for (uint32_t fh = 0; fh < d->fh; ++fh)
-                        for (uint32_t fw = 0; fw < d->fw; ++fw) {
-                            int64_t ih = (int64_t)d->stride_h * oh + (int64_t)fh * dh + h_offset;
-                            int64_t iw = (int64_t)d->stride_w * ow + (int64_t)fw * dw + w_offset;
-                            if (ih < 0 || ih >= (int64_t)d->ih || iw < 0 || iw >= (int64_t)d->iw) continue;
-                            for (uint32_t ic = 0; ic < icpg; ++ic) {
-                                int32_t s = src[act_off(d->src_stride_n, pi, d->ic, d->ih, d->iw, n,
-                                                        (int64_t)g * icpg + ic, ih, iw)];
-                                int32_t f = flt[flt_off(d, icpg, ocpg, g, oc_in_g, ic, fh, fw)];
-                                /* StrategyFwd::on for qint8: int32 multiply-add with wraparound
-                                 * (helper.h:67-74) */
-                                acc = (int32_t)((uint32_t)acc + (uint32_t)(s * f));
-                            }
-                        }
+                    int32_t acc = acc_one(d, icpg, ocpg, src, flt, n, oc, oh, ow);
                     int64_t o = act_off(0, po, d->oc, OH, OW, n, oc, oh, ow);
                     if (d->bias_mode == MI355_BIAS_BROADCAST_CHANNEL)
                         acc = (int32_t)((uint32_t)acc + (uint32_t)bias[oc]); /* bias is linear in channel */
@@ -235,6 +242,40 @@ int oracle_convbias_s8_acc(const mi355_conv_desc* d, const int8_t* src, const in
                     sfb[o] = acc;
                 }
         }
+    }
+    return MI355_OK;
+}
+
+/* The operator evaluated at `count` chosen output elements only (for spot checks at sizes where
+ * the whole tensor would take too long).  idx[i] is a linear index into the dense dst tensor
+ * (n, oc/p, oh, ow, p); QuantizedS8 dst only.  z is addressed with z_stride_n. */
+int oracle_convbias_s8_points(const mi355_conv_desc* d, const int8_t* src, const int8_t* flt, const int32_t* bias,
+                              const int8_t* z, const int64_t* idx, int64_t count, int8_t* out) {
+    uint32_t icpg, ocpg;
+    int st = check_desc(d, &icpg, &ocpg);
+    if (st) return st;
+    if (d->dst_dtype != MI355_DT_QS8) return MI355_ERR_UNSUPPORTED;
+    const int po = out_pack(d->format);
+    const int64_t OH = out_size(d->ih, d->fh, d->dilate_h, d->stride_h, d->pad_h);
+    const int64_t OW = out_size(d->iw, d->fw, d->dilate_w, d->stride_w, d->pad_w);
+    const int64_t per_n = (int64_t)d->oc * OH * OW;
+    const int64_t zsn = d->z_stride_n ? d->z_stride_n : per_n;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < count; ++i) {
+        int64_t t = idx[i];
+        int64_t n = t / per_n, r = t % per_n;
+        int64_t k = r % po, q = r / po;
+        int64_t ow = q % OW;
+        q /= OW;
+        int64_t oh = q % OH, ocb = q / OH;
+        uint32_t oc = (uint32_t)(ocb * po + k);
+        int32_t acc = acc_one(d, icpg, ocpg, src, flt, (uint32_t)n, oc, (uint32_t)oh, (uint32_t)ow);
+        if (d->bias_mode == MI355_BIAS_BROADCAST_CHANNEL)
+            acc = (int32_t)((uint32_t)acc + (uint32_t)bias[oc]);
+        else if (d->bias_mode == MI355_BIAS_FULL)
+            acc = (int32_t)((uint32_t)acc + (uint32_t)bias[t]);
+        int8_t zv = d->has_z ? z[n * zsn + r] : 0;
+        out[i] = oracle_epilogue_s8(acc, d->scale_bias, d->has_z, zv, d->scale_z, d->nonline, d->scale_dst);
     }
     return MI355_OK;
 }

@@ -40,6 +40,9 @@ def lib():
         L.oracle_convbias_s8.restype = C.c_int
         L.oracle_convbias_s8.argtypes = [P(_abi.ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                          C.c_void_p]
+        L.oracle_convbias_s8_points.restype = C.c_int
+        L.oracle_convbias_s8_points.argtypes = [P(_abi.ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                                C.c_void_p, C.c_int64, C.c_void_p]
         L.oracle_relayout_deduce.restype = C.c_int
         L.oracle_relayout_deduce.argtypes = [P(_abi.RelayoutDesc), P(C.c_uint32), P(C.c_uint32)]
         L.oracle_relayout.restype = C.c_int
@@ -90,6 +93,17 @@ def conv_acc(desc, src, flt, bias=None):
     if st:
         raise OracleError(st)
     return sfb
+
+
+def conv_bias_points(desc, src, flt, bias, z, idx):
+    """Operator output at the dense-dst linear indices `idx` (int64 array) only."""
+    idx = np.ascontiguousarray(idx, dtype=np.int64)
+    out = np.zeros(idx.shape, dtype=np.int8)
+    st = lib().oracle_convbias_s8_points(C.byref(desc), _ptr(src), _ptr(flt), _ptr(bias), _ptr(z), _ptr(idx),
+                                         idx.size, _ptr(out))
+    if st:
+        raise OracleError(st)
+    return out
 
 
 def relayout_desc(mode, shape, group=1, oc=0, elem_bytes=1, scale_src=1.0, scale_dst=1.0):

@@ -1,0 +1,131 @@
+"""C-ABI checks that need no GPU: the library loads, exports every symbol the header declares,
+and the descriptor validation / shape deduction / chooser surface behave like the reference's
+host-side checks (dnn/src/common/conv_bias.cpp:8-133, dnn/src/common/convolution.cpp:633-1049)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from megengine_amd import _abi, lib, ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_loads_and_exports_header_symbols():
+    L = lib.lib()
+    assert L.mi355_abi_version() == _abi.ABI_VERSION
+    hdr = open(os.path.join(ROOT, "include", "mi355_convbias.h")).read()
+    declared = set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", hdr))
+    assert declared, "no declarations found"
+    for name in declared:
+        assert hasattr(L, name), "library does not export %s" % name
+    assert declared == set(lib.EXPORTS)
+
+
+def test_struct_layout_matches_header():
+    # sizes fixed by the C header (checked against a C compiler in test_host_cpp)
+    assert C.sizeof(_abi.ConvDesc) == 4 * 24 + 8 * 3
+    assert C.sizeof(_abi.Algo) == 16
+    assert C.sizeof(_abi.RelayoutDesc) == 4 * 2 + 28 + 4 * 5
+
+
+def test_status_strings():
+    L = lib.lib()
+    for st in range(8):
+        assert L.mi355_status_string(st)
+    assert L.mi355_status_string(99) == b"unknown status"
+
+
+def test_algorithm_table():
+    names = lib.algo_names()
+    assert names == ["MI355_DIRECT_DOT4", "MI355_IGEMM_MFMA_I8", "MI355_DEPTHWISE_DOT4"]
+    assert lib.lib().mi355_convbias_algo_name(17) is None
+    assert len(lib.tile_names()) >= 3
+
+
+@pytest.mark.parametrize("fmt,n,ic,ih,iw,oc,f,kw,want", [
+    ("NCHW4", 16, 64, 56, 56, 64, 3, dict(pad=1), (16, 16, 56, 56, 4)),
+    ("NCHW32", 64, 256, 56, 56, 64, 1, {}, (64, 2, 56, 56, 32)),
+    ("NCHW4", 64, 4, 224, 224, 64, 7, dict(pad=3, stride=2), (64, 16, 112, 112, 4)),
+    ("NCHW32", 128, 512, 32, 32, 1024, 3, dict(pad=1, stride=2), (128, 32, 16, 16, 32)),
+    ("NCHW", 2, 3, 9, 9, 5, 3, dict(dilate=2), (2, 5, 5, 5)),
+    ("NCHW4_NCHW32", 1, 8, 6, 6, 32, 3, dict(pad=1), (1, 1, 6, 6, 32)),
+])
+def test_deduce_layout(fmt, n, ic, ih, iw, oc, f, kw, want):
+    d = _abi.make_conv_desc(fmt, n, ic, ih, iw, oc, f, **kw)
+    assert ops.conv_bias_deduce_layout(d) == want
+
+
+def _status(d):
+    oh, ow = C.c_uint32(), C.c_uint32()
+    return lib.lib().mi355_convbias_deduce_out(C.byref(d), C.byref(oh), C.byref(ow))
+
+
+def test_validation_errors():
+    # group conv channel mismatch (convolution.cpp:803-808)
+    assert _status(_abi.make_conv_desc("NCHW4", 1, 10, 8, 8, 8, 3)) == _abi.ERR_SHAPE
+    # oc % 4 (convolution.cpp:811)
+    assert _status(_abi.make_conv_desc("NCHW4", 1, 8, 8, 8, 6, 3)) == _abi.ERR_SHAPE
+    assert _status(_abi.make_conv_desc("NCHW32", 1, 32, 8, 8, 48, 3)) == _abi.ERR_SHAPE
+    # NCHWx dilation must be 1 (convolution.cpp:411-414)
+    assert _status(_abi.make_conv_desc("NCHW4", 1, 8, 8, 8, 8, 3, dilate=2)) == _abi.ERR_SHAPE
+    # quantized SIGMOID (naive/conv_bias/opr_impl.cpp:79-88)
+    assert _status(_abi.make_conv_desc("NCHW4", 1, 8, 8, 8, 8, 3, nonline="SIGMOID")) == _abi.ERR_UNSUPPORTED
+    # z with the 4<->32 formats (conv_bias.cpp:127-129)
+    assert _status(_abi.make_conv_desc("NCHW4_NCHW32", 1, 8, 8, 8, 32, 3, has_z=True)) == _abi.ERR_SHAPE
+    # unknown format
+    d = _abi.make_conv_desc("NCHW4", 1, 8, 8, 8, 8, 3)
+    d.format = 1  # NHWC
+    assert _status(d) == _abi.ERR_UNSUPPORTED
+    # filter larger than padded input
+    assert _status(_abi.make_conv_desc("NCHW4", 1, 8, 2, 2, 8, 5)) == _abi.ERR_SHAPE
+    # dense with group
+    d = _abi.make_conv_desc("NCHW4", 1, 8, 8, 8, 8, 3)
+    d.group = 2
+    assert _status(d) == _abi.ERR_SHAPE
+    assert b"group" in lib.lib().mi355_last_error()
+    # batch stride smaller than an image
+    assert _status(_abi.make_conv_desc("NCHW4", 2, 8, 8, 8, 8, 3, pad=1, src_stride_n=16)) == _abi.ERR_SHAPE
+    with pytest.raises(lib.Mi355Error):
+        ops.conv_bias_deduce_layout(_abi.make_conv_desc("NCHW4", 1, 10, 8, 8, 8, 3))
+
+
+def test_query_chooser_and_workspace():
+    igemm = lib.algo_names().index("MI355_IGEMM_MFMA_I8")
+    dw = lib.algo_names().index("MI355_DEPTHWISE_DOT4")
+    a, ws = ops.conv_bias_query(_abi.make_conv_desc("NCHW32", 64, 256, 56, 56, 64, 1, scale_bias=2e-4, scale_dst=0.05))
+    assert (a.id, ws) == (igemm, 0)
+    a, _ = ops.conv_bias_query(_abi.make_conv_desc("NCHW4", 1, 32, 8, 8, 32, 3, pad=1, group=32))
+    assert a.id == dw
+    # scales outside the fast epilogue's envelope: MFMA algo is not usable, direct kernel runs it
+    d = _abi.make_conv_desc("NCHW32", 1, 32, 8, 8, 32, 3, pad=1, scale_dst=1e-30)
+    a, _ = ops.conv_bias_query(d)
+    assert a.id == 0
+    with pytest.raises(lib.Mi355Error) as e:
+        ops.conv_bias_query(d, igemm)
+    assert e.value.status == _abi.ERR_ALGO
+    with pytest.raises(lib.Mi355Error):
+        ops.conv_bias_query(d, 42)
+    # asking for the depthwise kernel on a dense conv
+    assert lib.lib().mi355_convbias_algo_usable(C.byref(_abi.make_conv_desc("NCHW4", 1, 8, 8, 8, 8, 3)), dw) == _abi.ERR_ALGO
+
+
+def test_relayout_deduce():
+    assert ops.relayout_deduce_layout(ops.relayout_desc(_abi.RL_NCHW_NCHW4, (1, 6, 1, 2), group=2)) == (1, 2, 1, 2, 4)
+    assert ops.relayout_deduce_layout(ops.relayout_desc(_abi.RL_NCHW4_NCHW, (1, 2, 1, 2, 4), oc=7)) == (1, 7, 1, 2)
+    assert ops.relayout_deduce_layout(ops.relayout_desc(_abi.RL_NCHW_NCHW4_WEIGHT, (2, 2, 1, 2, 2))) == (2, 4, 1, 2, 2, 4)
+    assert ops.relayout_deduce_layout(ops.relayout_desc(_abi.RL_NCHW_NCHW32, (2, 40, 3, 3))) == (2, 2, 3, 3, 32)
+    assert ops.relayout_deduce_layout(ops.relayout_desc(_abi.RL_NCHW_NCHW4_IC_SMALL, (2, 3, 8, 8))) == (2, 1, 8, 8, 4)
+    with pytest.raises(lib.Mi355Error):
+        ops.relayout_deduce_layout(ops.relayout_desc(_abi.RL_NCHW_NCHW4_IC_SMALL, (2, 5, 8, 8)))
+    with pytest.raises(lib.Mi355Error):
+        ops.relayout_deduce_layout(ops.relayout_desc(99, (2, 5, 8, 8)))
+
+
+def test_exec_rejects_host_tensors():
+    import torch
+    d = _abi.make_conv_desc("NCHW4", 1, 8, 4, 4, 8, 1)
+    x = torch.zeros(1, 2, 4, 4, 4, dtype=torch.int8)
+    with pytest.raises(RuntimeError):
+        ops.conv_bias_exec(d, x, x, None, None)

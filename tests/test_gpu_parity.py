@@ -1,0 +1,198 @@
+"""Parity of the HIP kernels (through the C ABI) against the CPU checker: bit-exact int8.
+Every case prints what it is about to launch before touching the GPU."""
+import numpy as np
+import pytest
+import torch
+
+from megengine_amd import _abi, ops
+from tests import util
+from tests.gpu_util import check_case, run_gpu, say, to_dev
+
+pytestmark = pytest.mark.gpu
+
+DIRECT, IGEMM, DW = 0, 1, 2
+S = dict(scale_bias=2e-4, scale_z=0.05, scale_dst=0.05)
+
+
+# ---------------------------------------------------------------------------------------------
+# generic direct kernel: every format / mode on small shapes
+# ---------------------------------------------------------------------------------------------
+
+DIRECT_CASES = [
+    dict(fmt="NCHW", n=2, ic=3, ih=7, iw=9, oc=5, fh=3, pad=1),
+    dict(fmt="NCHW", n=1, ic=8, ih=8, iw=8, oc=12, fh=3, fw=2, group=4, pad=(1, 0), stride=(2, 1)),
+    dict(fmt="NCHW", n=2, ic=4, ih=11, iw=10, oc=6, fh=3, group=2, pad=2, stride=(1, 2), dilate=2),
+    dict(fmt="NCHW", n=1, ic=3, ih=8, iw=8, oc=4, fh=3, pad=1, mode=_abi.MODE_CONVOLUTION),
+    dict(fmt="NCHW", n=1, ic=6, ih=9, iw=9, oc=6, fh=5, group=6, pad=2),
+    dict(fmt="NCHW4", n=2, ic=8, ih=6, iw=5, oc=12, fh=3, pad=1),
+    dict(fmt="NCHW4", n=1, ic=60, ih=9, iw=9, oc=20, fh=3, group=5, pad=1),   # shape family of naive/convolution.cpp:215
+    dict(fmt="NCHW4", n=2, ic=16, ih=7, iw=7, oc=16, fh=3, group=16, pad=1),  # packed channel-wise
+    dict(fmt="NCHW32", n=2, ic=32, ih=4, iw=4, oc=32, fh=3, pad=1),           # naive/conv_bias.cpp:163
+    dict(fmt="NCHW32", n=1, ic=64, ih=5, iw=6, oc=64, fh=1, group=2),
+    dict(fmt="NCHW44", n=1, ic=8, ih=5, iw=5, oc=8, fh=3, pad=1),
+    dict(fmt="NCHW44", n=1, ic=16, ih=5, iw=5, oc=8, fh=3, group=2, pad=1),
+    dict(fmt="NCHW44", n=1, ic=8, ih=6, iw=6, oc=8, fh=3, group=8, pad=1, stride=2),
+    dict(fmt="NCHW4_NCHW32", n=1, ic=8, ih=6, iw=6, oc=32, fh=3, pad=1),
+    dict(fmt="NCHW32_NCHW4", n=1, ic=32, ih=6, iw=6, oc=8, fh=3, pad=1),
+]
+
+
+def mk(c, **extra):
+    kw = dict(c)
+    kw.update(extra)
+    fmt = kw.pop("fmt")
+    return _abi.make_conv_desc(fmt, kw.pop("n"), kw.pop("ic"), kw.pop("ih"), kw.pop("iw"), kw.pop("oc"),
+                               kw.pop("fh"), kw.pop("fw", None), **kw)
+
+
+@pytest.mark.parametrize("i", range(len(DIRECT_CASES)))
+def test_direct_all_formats(oracle, i):
+    c = DIRECT_CASES[i]
+    mixed = c["fmt"] in ("NCHW4_NCHW32", "NCHW32_NCHW4")
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        for has_z in ((False,) if mixed else (False, True)):
+            check_case(oracle, mk(c, nonline=nl, has_z=has_z, **S), seed=i + 1, algo=DIRECT, tag="direct%d" % i)
+
+
+def test_direct_s32_dst_and_full_bias(oracle, kats):
+    # the reference KAT itself, on the GPU (QuantizedS32 dst and z)
+    k = kats["conv_bias_quantized8x8x32"]
+    d = _abi.make_conv_desc("NCHW", 1, 1, 4, 4, 3, 3, has_z=True, dst_dtype=_abi.DT_QS32,
+                            scale_bias=float(np.float32(0.02)), scale_z=float(np.float32(0.3)),
+                            scale_dst=float(np.float32(0.1) * np.float32(0.2)))
+    say("case KAT conv_bias_quantized8x8x32 on GPU")
+    got = run_gpu(d, np.array(k["src"], np.int8).reshape(1, 1, 4, 4), np.array(k["filter"], np.int8).reshape(3, 1, 3, 3),
+                  np.array(k["bias"], np.int32).reshape(1, 3, 1, 1), np.array(k["z"], np.int32).reshape(1, 3, 2, 2),
+                  algo=DIRECT)
+    assert got.reshape(-1).tolist() == k["dst"]
+    check_case(oracle, _abi.make_conv_desc("NCHW4", 2, 8, 5, 5, 8, 3, pad=1, bias_mode=_abi.BIAS_FULL, **S), algo=DIRECT)
+    check_case(oracle, _abi.make_conv_desc("NCHW4", 2, 8, 5, 5, 8, 3, pad=1, bias_mode=_abi.BIAS_NONE, **S), algo=DIRECT)
+    check_case(oracle, _abi.make_conv_desc("NCHW32", 1, 32, 5, 5, 32, 3, pad=1, dst_dtype=_abi.DT_QS32,
+                                           scale_bias=2e-4, scale_dst=2e-4), algo=DIRECT)
+
+
+def test_direct_exact_epilogue_for_odd_scales(oracle):
+    """Scales outside the fast form's envelope take the literal IEEE-divide epilogue."""
+    for sd in (1e-20, 3e15):
+        d = _abi.make_conv_desc("NCHW4", 1, 8, 5, 5, 8, 3, pad=1, nonline="H_SWISH", has_z=True, scale_bias=2e-4,
+                                scale_z=0.05, scale_dst=sd)
+        check_case(oracle, d, algo=None, tag="oddscale")
+
+
+# ---------------------------------------------------------------------------------------------
+# MFMA implicit GEMM
+# ---------------------------------------------------------------------------------------------
+
+IGEMM_CASES = [
+    # fmt, n, ic, ih, iw, oc, f, pad, stride
+    ("NCHW32", 2, 64, 8, 8, 64, 1, 0, 1),
+    ("NCHW32", 3, 32, 7, 7, 96, 1, 0, 1),       # ragged pixels (147) and oc = 96
+    ("NCHW32", 2, 64, 9, 11, 64, 3, 1, 1),
+    ("NCHW32", 2, 96, 12, 12, 160, 3, 1, 2),
+    ("NCHW32", 1, 32, 14, 14, 32, 5, 2, 1),
+    ("NCHW32", 1, 32, 17, 15, 64, 7, 3, 2),
+    ("NCHW32", 2, 128, 6, 6, 256, 1, 0, 2),     # strided 1x1 (downsample)
+    ("NCHW32", 1, 256, 5, 5, 320, 3, 0, 1),     # no padding, long K
+    ("NCHW4", 2, 16, 9, 9, 32, 1, 0, 1),
+    ("NCHW4", 2, 64, 10, 10, 64, 3, 1, 1),      # cfg0 family
+    ("NCHW4", 1, 4, 30, 30, 64, 7, 3, 2),       # stem: K = 196 bytes, not a multiple of 32
+    ("NCHW4", 2, 24, 8, 8, 144, 1, 0, 1),       # MobileNetV2 expand
+    ("NCHW4", 2, 144, 8, 8, 24, 1, 0, 1),       # MobileNetV2 project (oc < 32)
+    ("NCHW4", 1, 12, 9, 7, 20, 3, 1, 2),        # oc % 32 != 0, K = 108
+    ("NCHW4_NCHW32", 2, 16, 8, 8, 64, 3, 1, 1),
+    ("NCHW32_NCHW4", 2, 64, 8, 8, 24, 3, 1, 1),
+]
+
+
+@pytest.mark.parametrize("i", range(len(IGEMM_CASES)))
+def test_igemm_formats_and_tiles(oracle, i):
+    fmt, n, ic, ih, iw, oc, f, pad, stride = IGEMM_CASES[i]
+    mixed = "_" in fmt
+    ntiles = 5
+    for tile in range(ntiles):
+        nl = ("IDENTITY", "RELU", "H_SWISH")[(tile + i) % 3]
+        has_z = (not mixed) and (tile % 2 == 0)
+        d = _abi.make_conv_desc(fmt, n, ic, ih, iw, oc, f, pad=pad, stride=stride, nonline=nl, has_z=has_z, **S)
+        check_case(oracle, d, seed=100 + i, algo=IGEMM, tile=tile, tag="igemm%d" % i)
+
+
+def test_igemm_nonlines_z_bias(oracle):
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        for has_z in (False, True):
+            for bm in (_abi.BIAS_BROADCAST_CHANNEL, _abi.BIAS_NONE):
+                d = _abi.make_conv_desc("NCHW32", 2, 64, 10, 10, 64, 3, pad=1, nonline=nl, has_z=has_z, bias_mode=bm, **S)
+                check_case(oracle, d, seed=7, algo=IGEMM, tag="nlzb")
+                d = _abi.make_conv_desc("NCHW4", 2, 32, 10, 10, 40, 3, pad=1, nonline=nl, has_z=has_z, bias_mode=bm, **S)
+                check_case(oracle, d, seed=8, algo=IGEMM, tag="nlzb4")
+
+
+def test_igemm_saturation_and_scales(oracle):
+    """Big accumulators (full-range int8 x long K) saturate both ways; random per-tensor scales."""
+    rng = np.random.RandomState(3)
+    for t in range(6):
+        sb = float(np.float32(np.exp(rng.uniform(np.log(1e-6), np.log(2.5e-3)))))
+        sz = float(np.float32(np.exp(rng.uniform(np.log(1e-3), np.log(5e-2)))))
+        sd = float(np.float32(np.exp(rng.uniform(np.log(1e-3), np.log(5e-2)))))
+        d = _abi.make_conv_desc("NCHW32", 1, 256, 6, 6, 64, 3, pad=1, nonline=("IDENTITY", "RELU", "H_SWISH")[t % 3],
+                                has_z=True, scale_bias=sb, scale_z=sz, scale_dst=sd)
+        check_case(oracle, d, seed=40 + t, algo=IGEMM, tag="scales")
+
+
+def test_igemm_strided_batch(oracle):
+    d0 = _abi.make_conv_desc("NCHW32", 3, 64, 6, 6, 64, 3, pad=1, nonline="RELU", has_z=True, **S)
+    per_src, per_dst = 64 * 36, 64 * 36
+    d = _abi.make_conv_desc("NCHW32", 3, 64, 6, 6, 64, 3, pad=1, nonline="RELU", has_z=True,
+                            src_stride_n=per_src + 64, z_stride_n=per_dst + 32, dst_stride_n=per_dst + 96, **S)
+    want = check_case(oracle, d, seed=5, algo=IGEMM, tag="strided")
+    assert np.array_equal(want, check_case(oracle, d0, seed=5, algo=IGEMM, tag="dense"))
+
+
+def test_config0_full_size(oracle):
+    """BASELINE config 0: NCHW4 N16 64->64 56x56 3x3 s1 p1, bias U[-1000,1000], RELU, scales .02*.01 -> .05."""
+    sb = float(np.float32(0.02) * np.float32(0.01))
+    d = _abi.make_conv_desc("NCHW4", 16, 64, 56, 56, 64, 3, pad=1, nonline="RELU", scale_bias=sb,
+                            scale_dst=float(np.float32(0.05)))
+    check_case(oracle, d, seed=2024, tag="config0")
+
+
+# ---------------------------------------------------------------------------------------------
+# depthwise
+# ---------------------------------------------------------------------------------------------
+
+DW_CASES = [
+    # fmt, n, c, ih, iw, f, pad, stride
+    ("NCHW4", 2, 32, 14, 14, 3, 1, 1),
+    ("NCHW4", 2, 24, 15, 13, 3, 1, 2),
+    ("NCHW4", 1, 96, 28, 28, 3, 1, 1),
+    ("NCHW4", 1, 96, 28, 28, 3, 1, 2),
+    ("NCHW44", 2, 16, 7, 7, 3, 1, 1),      # ow % 4 != 0
+    ("NCHW4", 1, 8, 12, 12, 5, 2, 1),      # generic filter size
+    ("NCHW4", 1, 8, 9, 16, 3, 0, 1),       # no padding
+    ("NCHW44", 1, 8, 11, 11, 3, 1, 3),     # generic stride
+]
+
+
+@pytest.mark.parametrize("i", range(len(DW_CASES)))
+def test_depthwise(oracle, i):
+    fmt, n, c, ih, iw, f, pad, stride = DW_CASES[i]
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        for has_z in (False, True):
+            d = _abi.make_conv_desc(fmt, n, c, ih, iw, c, f, group=c, pad=pad, stride=stride, nonline=nl, has_z=has_z, **S)
+            a, _ = ops.conv_bias_query(d)
+            assert a.id == DW
+            check_case(oracle, d, seed=200 + i, tag="dw%d" % i)
+
+
+# ---------------------------------------------------------------------------------------------
+# chooser + cross-algorithm agreement at larger sizes
+# ---------------------------------------------------------------------------------------------
+
+def test_heuristic_picks(oracle):
+    d = _abi.make_conv_desc("NCHW32", 64, 256, 56, 56, 64, 1)
+    assert ops.conv_bias_query(d)[0].id == IGEMM
+    d = _abi.make_conv_desc("NCHW", 1, 8, 8, 8, 8, 3, pad=1)
+    assert ops.conv_bias_query(d)[0].id == DIRECT
+    d = _abi.make_conv_desc("NCHW4", 1, 32, 8, 8, 32, 3, pad=1, group=32)
+    assert ops.conv_bias_query(d)[0].id == DW
+    d = _abi.make_conv_desc("NCHW32", 1, 64, 8, 8, 64, 3, pad=1, group=2)
+    assert ops.conv_bias_query(d)[0].id == DIRECT
