@@ -1,0 +1,314 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8 ConvBias hot path on one MI355X.
+
+A "step" is one pass over the 53 ConvBias layers of the ResNet-50 int8 conv stack at batch 64
+(BASELINE config 2) on synthetic, HBM-resident tensors; activations are requantised between
+layers and the residual z tensors are the real producer outputs.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+value      = images per second over the timed region (K steps, events on the launch stream)
+roofline   = algorithmic bytes of the stack / sum of per-launch kernel durations (second pass of
+             the same K steps with an event after every launch), against 8 TB/s HBM
+cpu_baseline = the CPU parity checker (a port of the reference's naive ConvBias) timed on this
+             host on a bounded sample (one image through the same 53 layers), scaled to images/s
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+INT8_PEAK_OPS = 5.0e15   # dense INT8 MFMA, MI355X
+HBM_PEAK = 8.0e12        # bytes/s
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_stack(layers, seed, torch, np, util, _abi):
+    """Allocates every tensor of a layer list on the GPU and returns launch closures."""
+    rng = np.random.RandomState(seed)
+
+    def scale():
+        return float(np.float32(np.exp(rng.uniform(np.log(1e-3), np.log(5e-2)))))
+
+    def rand_i8(shape, lo=-128, hi=127):
+        return torch.randint(lo, hi + 1, shape, dtype=torch.int8, device="cuda")
+
+    outs, out_scale, inputs = {}, {}, {}
+    plan = []
+    prev = None
+    for i, L in enumerate(layers):
+        d0 = L.desc(1.0, 1.0, 1.0)
+        src_s, flt_s, bias_s, dst_s = _abi.conv_shapes(d0)
+        # source tensor
+        sname = L.src if L.src is not None else prev
+        if sname is None or sname.startswith("input:") or sname not in outs or tuple(outs[sname].shape) != tuple(src_s):
+            key = "in:%s:%s" % (sname, src_s)
+            if key not in inputs:
+                inputs[key] = (rand_i8(src_s), scale())
+            src, s_src = inputs[key]
+        else:
+            src, s_src = outs[sname], out_scale[sname]
+        s_flt = scale()
+        s_bias = float(np.float32(s_src) * np.float32(s_flt))
+        s_dst = scale()
+        flt = rand_i8(flt_s, -127, 127)
+        bias = torch.randint(-1000, 1001, bias_s, dtype=torch.int32, device="cuda")
+        z, s_z = None, 1.0
+        if L.z is not None:
+            if L.z in outs and tuple(outs[L.z].shape) == tuple(dst_s):
+                z, s_z = outs[L.z], out_scale[L.z]
+            else:
+                key = "z:%s:%s" % (L.z, dst_s)
+                if key not in inputs:
+                    inputs[key] = (rand_i8(dst_s), scale())
+                z, s_z = inputs[key]
+        dst = torch.empty(dst_s, dtype=torch.int8, device="cuda")
+        desc = L.desc(s_bias, s_z, s_dst)
+        outs[L.name], out_scale[L.name] = dst, s_dst
+        prev = L.name
+        plan.append(dict(layer=L, desc=desc, src=src, flt=flt, bias=bias, z=z, dst=dst))
+    return plan
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-extras", action="store_true", help="skip the per-config side measurements")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--layers-out", default=None, help="write the per-layer table to this JSON file")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU (the path shards by batch with no exchange); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from megengine_amd import _abi, lib, ops, workloads
+    from tests import util
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    L = lib.lib()  # raises if the HIP extension is missing
+    info = lib.device_info(0)
+    log("device: %s %s, %d CUs, %.0f MHz" % (info.name.decode(), info.arch.decode(), info.compute_units,
+                                             info.clock_khz / 1e3))
+    torch.manual_seed(1234)
+    batch = 64
+    layers = workloads.resnet50(batch)
+    plan = build_stack(layers, 7, torch, np, util, _abi)
+    for p in plan:
+        p["algo"], _ = ops.conv_bias_query(p["desc"])
+    stream = torch.cuda.current_stream()
+
+    def launch(p):
+        ops.conv_bias_exec(p["desc"], p["src"], p["flt"], p["bias"], p["z"], dst=p["dst"], algo=p["algo"])
+
+    def step():
+        for p in plan:
+            launch(p)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(args.steps):
+        step()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    ms_total = e0.elapsed_time(e1)
+    ms_per_step = ms_total / args.steps
+    img_s = batch * 1000.0 / ms_per_step
+    tot_ops = sum(l.ops for l in layers)
+    tot_bytes = sum(l.bytes for l in layers)
+
+    # ---- second pass: an event after every launch -> per-layer kernel durations
+    nl = len(plan)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(nl + 1)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    for s in range(args.steps):
+        evs[s][0].record(stream)
+        for i, p in enumerate(plan):
+            launch(p)
+            evs[s][i + 1].record(stream)
+    torch.cuda.synchronize()
+    per_layer_ms = [sum(evs[s][i].elapsed_time(evs[s][i + 1]) for s in range(args.steps)) / args.steps
+                    for i in range(nl)]
+    kern_ms = sum(per_layer_ms)
+    table = []
+    for p, ms in zip(plan, per_layer_ms):
+        l = p["layer"]
+        t = ms * 1e-3
+        roof = max(l.ops / INT8_PEAK_OPS, l.bytes / HBM_PEAK)
+        table.append(dict(name=l.name, ic=l.ic, oc=l.oc, hw=l.ih, f=l.f, s=l.stride, z=l.z is not None,
+                          algo=lib.algo_names()[p["algo"].id], tile=lib.tile_names()[p["algo"].tile_cfg],
+                          us=round(ms * 1e3, 2), tops=round(l.ops / t / 1e12, 1), gbs=round(l.bytes / t / 1e9, 1),
+                          frac_roof=round(roof / t, 3)))
+    roofline = dict(bound="hbm", achieved=round(tot_bytes / (kern_ms * 1e-3) / 1e9, 1), peak=HBM_PEAK / 1e9,
+                    unit="GB/s", frac=round(tot_bytes / (kern_ms * 1e-3) / HBM_PEAK, 4), traffic=None,
+                    kernel="igemm_kernel (MI355_IGEMM_MFMA_I8), 53 launches per step",
+                    bytes_per_launch=round(tot_bytes / nl), avg_launch_us=round(kern_ms * 1e3 / nl, 2),
+                    kernel_ms_per_step=round(kern_ms, 4),
+                    mfma_tops=round(tot_ops / (kern_ms * 1e-3) / 1e12, 1),
+                    mfma_frac_of_int8_peak=round(tot_ops / (kern_ms * 1e-3) / INT8_PEAK_OPS, 4),
+                    frac_of_binding_roof=round(sum(max(l.ops / INT8_PEAK_OPS, l.bytes / HBM_PEAK) for l in layers)
+                                               / (kern_ms * 1e-3), 4))
+    tr = os.path.join(ROOT, "profiles", "traffic_resnet50_stack.json")
+    if os.path.exists(tr):
+        try:
+            roofline["traffic"] = json.load(open(tr))["hbm_bytes_per_launch"]
+        except Exception:
+            pass
+
+    out = dict(metric="ResNet-50 int8 conv-stack throughput @ bs64 (53 ConvBias layers)", value=round(img_s, 1),
+               unit="img/s", n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_per_step, 4),
+               higher_is_better=True, scaling="weak", vs_baseline=None, dtype="s8*s8->s32 accumulate, f32 requant",
+               data="synthetic",
+               config=dict(workload="BASELINE configs[2]: ResNet-50 v1.5 int8 conv stack, batch 64, 224x224, "
+                                    "NCHW4 stem + NCHW32, fused residual z + RELU, random per-tensor scales",
+                           batch=batch, layers=nl),
+               tops=round(tot_ops / (ms_per_step * 1e-3) / 1e12, 1),
+               pct_int8_peak=round(100 * tot_ops / (ms_per_step * 1e-3) / INT8_PEAK_OPS, 2),
+               roofline=roofline)
+
+    extras = {}
+    if not args.no_extras:
+        try:
+            extras = run_extras(torch, np, util, _abi, lib, ops, workloads)
+        except Exception as e:  # side measurements must not lose the headline
+            extras = dict(error=repr(e))
+        out["other_configs"] = extras
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(np, util, _abi, workloads)
+
+    if args.layers_out:
+        with open(args.layers_out, "w") as f:
+            json.dump(dict(layers=table, extras=extras), f, indent=1)
+    else:
+        for row in table:
+            log(row)
+    print(json.dumps(out), flush=True)
+
+
+def time_launches(torch, fn, iters=20, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    st = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(st)
+    for _ in range(iters):
+        fn()
+    e1.record(st)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters * 1e-3
+
+
+def run_extras(torch, np, util, _abi, lib, ops, workloads):
+    """Side measurements for the other BASELINE configs (not the headline value)."""
+    res = {}
+
+    def measure(layers, seed):
+        plan = build_stack(layers, seed, torch, np, util, _abi)
+        rows = []
+        for p in plan:
+            p["algo"], _ = ops.conv_bias_query(p["desc"])
+            t = time_launches(torch, lambda: ops.conv_bias_exec(p["desc"], p["src"], p["flt"], p["bias"], p["z"],
+                                                                dst=p["dst"], algo=p["algo"]))
+            l = p["layer"]
+            rows.append(dict(name=l.name, algo=lib.algo_names()[p["algo"].id], us=round(t * 1e6, 2),
+                             tops=round(l.ops / t / 1e12, 1), gbs=round(l.bytes / t / 1e9, 1),
+                             frac_roof=round(max(l.ops / INT8_PEAK_OPS, l.bytes / HBM_PEAK) / t, 3)))
+        return rows, plan
+
+    rows, _ = measure([workloads.config0()], 1)
+    res["config0"] = rows[0]
+    rows, _ = measure(workloads.pointwise_sweep(), 2)
+    res["config1_pointwise"] = rows
+    torch.cuda.empty_cache()
+    mb = workloads.mobilenet_v2()
+    rows, _ = measure(mb, 3)
+    dw = [(r, l) for r, l in zip(rows, mb) if l.group > 1]
+    pw = [(r, l) for r, l in zip(rows, mb) if l.group == 1]
+    t_dw = sum(r["us"] for r, _ in dw) * 1e-6
+    t_pw = sum(r["us"] for r, _ in pw) * 1e-6
+    res["config3_mobilenetv2"] = dict(
+        depthwise=dict(us=round(t_dw * 1e6, 1), gbs=round(sum(l.bytes for _, l in dw) / t_dw / 1e9, 1),
+                       frac_hbm=round(sum(l.bytes for _, l in dw) / t_dw / HBM_PEAK, 3)),
+        pointwise=dict(us=round(t_pw * 1e6, 1), gbs=round(sum(l.bytes for _, l in pw) / t_pw / 1e9, 1),
+                       tops=round(sum(l.ops for _, l in pw) / t_pw / 1e12, 1),
+                       frac_hbm=round(sum(l.bytes for _, l in pw) / t_pw / HBM_PEAK, 3)))
+    torch.cuda.empty_cache()
+    c4 = []
+    for l in workloads.large_hswish():
+        rows, plan = measure([l], 4)
+        p = plan[0]
+        # NCHW -> NCHW32 relayout of the input and NCHW32 -> NCHW of the output, timed with the conv
+        x_nchw = torch.randint(-128, 128, (l.n, l.ic, l.ih, l.iw), dtype=torch.int8, device="cuda")
+        y_nchw = torch.empty((l.n, l.oc, l.oh, l.ow), dtype=torch.int8, device="cuda")
+        d_in = ops.relayout_desc(_abi.RL_NCHW_NCHW32, tuple(x_nchw.shape))
+        d_out = ops.relayout_desc(_abi.RL_NCHW32_NCHW, tuple(p["dst"].shape))
+
+        def full():
+            ops.relayout_exec(d_in, x_nchw, p["src"])
+            ops.conv_bias_exec(p["desc"], p["src"], p["flt"], p["bias"], p["z"], dst=p["dst"], algo=p["algo"])
+            ops.relayout_exec(d_out, p["dst"], y_nchw)
+
+        t_full = time_launches(torch, full, iters=10)
+        t_in = time_launches(torch, lambda: ops.relayout_exec(d_in, x_nchw, p["src"]), iters=10)
+        t_out = time_launches(torch, lambda: ops.relayout_exec(d_out, p["dst"], y_nchw), iters=10)
+        rl_bytes_in, rl_bytes_out = 2 * x_nchw.numel(), 2 * y_nchw.numel()
+        c4.append(dict(conv=rows[0], total_us=round(t_full * 1e6, 1),
+                       relayout_in_gbs=round(rl_bytes_in / t_in / 1e9, 1),
+                       relayout_out_gbs=round(rl_bytes_out / t_out / 1e9, 1),
+                       relayout_frac_hbm=round((rl_bytes_in + rl_bytes_out) / (t_in + t_out) / HBM_PEAK, 3)))
+        del x_nchw, y_nchw, plan
+        torch.cuda.empty_cache()
+    res["config4_large_hswish"] = c4
+    return res
+
+
+def cpu_baseline(np, util, _abi, workloads):
+    """The CPU parity checker (port of the reference's naive ConvBias) on one image through the
+    same 53 layers, all host threads the process may use, scaled to images per second."""
+    from oracle import oracle
+    oracle.lib()
+    layers = workloads.resnet50(1)
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    os.environ["OMP_NUM_THREADS"] = str(cores)
+    t_tot, macs = 0.0, 0
+    budget = 25.0
+    done = 0
+    for i, l in enumerate(layers):
+        d = l.desc(2e-4, 0.05, 0.05)
+        src, flt, bias, z = util.make_tensors(d, seed=i + 1, flt_range=(-127, 127))
+        t0 = time.perf_counter()
+        oracle.conv_bias(d, src, flt, bias, z)
+        t_tot += time.perf_counter() - t0
+        macs += l.ops // 2
+        done += 1
+        if t_tot > budget:
+            break
+    total_macs = sum(l.ops // 2 for l in layers)
+    img_s = (macs / total_macs) / t_tot if t_tot > 0 else 0.0
+    return dict(value=round(img_s, 4), unit="img/s", cores=cores, kind="port",
+                sample="batch 1 through the first %d of 53 layers (%.2f of %.2f GMAC), %.1f s, scaled by MACs"
+                       % (done, macs / 1e9, total_macs / 1e9, t_tot))
+
+
+if __name__ == "__main__":
+    main()

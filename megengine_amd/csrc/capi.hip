@@ -266,8 +266,10 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
     if (!algo_usable(p, id)) return fail(MI355_ERR_ALGO, "%s cannot run this problem", kAlgoNames[id]);
     // the tiled kernels use 16-byte vector accesses; misaligned tensors take the generic kernel
     if (id != ALGO_DIRECT) {
+        // (pack-32 tensors move as 16-byte vectors, pack-4 tensors as dwords)
+        const int sa = p.pin == 32 ? 16 : 4, da = p.pout == 32 ? 16 : 4;
         bool al = aligned16(src) && aligned16(filter) && aligned16(dst) && (!bias || aligned16(bias)) &&
-                  (!z || aligned16(z)) && p.src_sn % 16 == 0 && p.dst_sn % 16 == 0 && p.z_sn % 16 == 0;
+                  (!z || aligned16(z)) && p.src_sn % sa == 0 && p.dst_sn % da == 0 && p.z_sn % da == 0;
         if (!al) {
             if (algo && algo->id != MI355_ALGO_HEURISTIC)
                 return fail(MI355_ERR_ALGO, "%s needs 16-byte aligned tensors", kAlgoNames[id]);

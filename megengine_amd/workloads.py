@@ -1,0 +1,104 @@
+"""The BASELINE workloads as lists of ConvBias descriptors (shapes only; no model code).
+
+config 2: the 53 ConvBias layers of ResNet-50 v1.5 at batch 64 (stem in NCHW4 with the input
+          padded to 4 channels, everything after the max-pool in NCHW32);
+config 1: the 1x1 NCHW32 sweep at N=64;
+config 3: MobileNetV2 (t=6, width 1.0) inverted-residual blocks at batch 64, NCHW4;
+config 4: large NCHW32 ConvBias + H_SWISH cases at batch 128 with relayouts on both sides.
+Work accounting follows the reference's own TOPS print (dnn/test/cuda/conv_test_utils.cpp:193,405):
+ops = 2*N*OC*OH*OW*(IC/group)*FH*FW; bytes = src + filter + 4*OC + (z ? dst : 0) + dst.
+"""
+from . import _abi
+
+
+class Layer:
+    def __init__(self, name, fmt, n, ic, ih, iw, oc, f, stride=1, pad=0, group=1, nonline="RELU", z=None,
+                 src=None):
+        self.name, self.fmt = name, fmt
+        self.n, self.ic, self.ih, self.iw, self.oc, self.f = n, ic, ih, iw, oc, f
+        self.stride, self.pad, self.group, self.nonline = stride, pad, group, nonline
+        self.z = z        # name of the layer whose output is added, or "input:<name>"
+        self.src = src    # name of the producing layer (None = the previous layer)
+        self.oh = _abi.out_size(ih, f, 1, stride, pad)
+        self.ow = _abi.out_size(iw, f, 1, stride, pad)
+
+    @property
+    def ops(self):
+        return 2 * self.n * self.oc * self.oh * self.ow * (self.ic // self.group) * self.f * self.f
+
+    @property
+    def bytes(self):
+        src = self.n * self.ic * self.ih * self.iw
+        flt = self.oc * (self.ic // self.group) * self.f * self.f
+        dst = self.n * self.oc * self.oh * self.ow
+        return src + flt + 4 * self.oc + (dst if self.z else 0) + dst
+
+    def desc(self, s_bias, s_z, s_dst):
+        return _abi.make_conv_desc(self.fmt, self.n, self.ic, self.ih, self.iw, self.oc, self.f, group=self.group,
+                                   pad=self.pad, stride=self.stride, nonline=self.nonline, has_z=self.z is not None,
+                                   scale_bias=s_bias, scale_z=s_z, scale_dst=s_dst)
+
+
+def resnet50(batch=64):
+    """53 layers.  The max-pool between the stem and stage 1 is not a ConvBias: stage 1 reads a
+    separate seeded tensor 'pool' of 64 channels at 56x56."""
+    L = [Layer("stem", "NCHW4", batch, 4, 224, 224, 64, 7, stride=2, pad=3)]
+    cin, h, prev = 64, 56, "input:pool"
+    for si, (mid, out, blocks, stride) in enumerate([(64, 256, 3, 1), (128, 512, 4, 2), (256, 1024, 6, 2),
+                                                      (512, 2048, 3, 2)]):
+        for b in range(blocks):
+            s = stride if b == 0 else 1
+            p = "s%db%d" % (si + 1, b)
+            L.append(Layer(p + "c1", "NCHW32", batch, cin, h, h, mid, 1, src=prev))
+            L.append(Layer(p + "c2", "NCHW32", batch, mid, h, h, mid, 3, stride=s, pad=1))
+            ho = h // s
+            if b == 0:
+                L.append(Layer(p + "ds", "NCHW32", batch, cin, h, h, out, 1, stride=s, nonline="IDENTITY", src=prev))
+                L.append(Layer(p + "c3", "NCHW32", batch, mid, ho, ho, out, 1, z=p + "ds", src=p + "c2"))
+            else:
+                L.append(Layer(p + "c3", "NCHW32", batch, mid, ho, ho, out, 1, z=prev, src=p + "c2"))
+            prev, cin, h = p + "c3", out, ho
+    assert len(L) == 53
+    return L
+
+
+def pointwise_sweep(batch=64):
+    shapes = [(256, 64, 56, False), (64, 256, 56, True), (512, 128, 28, False), (1024, 256, 14, False),
+              (2048, 512, 7, False)]
+    out = []
+    for ic, oc, hw, z in shapes:
+        for nl in ("IDENTITY", "RELU"):
+            out.append(Layer("pw%d_%d_%d_%s" % (ic, oc, hw, nl), "NCHW32", batch, ic, hw, hw, oc, 1, nonline=nl,
+                             z="input:z" if z else None))
+    return out
+
+
+def mobilenet_v2(batch=64):
+    """Inverted-residual blocks (expand 1x1, depthwise 3x3, project 1x1) from 16 channels at 112x112."""
+    L = []
+    cin, h = 16, 112
+    for c, n, s in [(24, 2, 2), (32, 3, 2), (64, 4, 2), (96, 3, 1), (160, 3, 2), (320, 1, 1)]:
+        for i in range(n):
+            stride = s if i == 0 else 1
+            hid = cin * 6
+            p = "c%d_%d" % (c, i)
+            L.append(Layer(p + "_expand", "NCHW4", batch, cin, h, h, hid, 1))
+            L.append(Layer(p + "_dw", "NCHW4", batch, hid, h, h, hid, 3, stride=stride, pad=1, group=hid))
+            ho = h // stride
+            res = stride == 1 and cin == c
+            L.append(Layer(p + "_project", "NCHW4", batch, hid, ho, ho, c, 1, nonline="IDENTITY",
+                           z="input:block" if res else None))
+            cin, h = c, ho
+    return L
+
+
+def large_hswish(batch=128):
+    return [
+        Layer("l3x3s1_256", "NCHW32", batch, 256, 64, 64, 256, 3, pad=1, nonline="H_SWISH", z="input:z"),
+        Layer("l3x3s2_512_1024", "NCHW32", batch, 512, 32, 32, 1024, 3, stride=2, pad=1, nonline="H_SWISH", z="input:z"),
+        Layer("l5x5s1_128", "NCHW32", batch, 128, 80, 80, 128, 5, pad=2, nonline="H_SWISH", z="input:z"),
+    ]
+
+
+def config0():
+    return Layer("cfg0", "NCHW4", 16, 64, 56, 56, 64, 3, pad=1, nonline="RELU")
