@@ -284,7 +284,7 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
             break;
         case ALGO_IGEMM_MFMA:
             if (cfg < 0 || cfg >= igemm_num_cfgs()) cfg = igemm_pick_cfg(p, cu_count());
-            rc = launch_conv_igemm(hs, p, cfg, src, filter, bias, z, reinterpret_cast<int8_t*>(dst));
+            rc = launch_conv_igemm(hs, p, cfg, cu_count(), src, filter, bias, z, reinterpret_cast<int8_t*>(dst));
             break;
         case ALGO_DEPTHWISE:
             rc = launch_conv_depthwise(hs, p, src, filter, bias, z, reinterpret_cast<int8_t*>(dst));

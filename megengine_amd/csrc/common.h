@@ -37,8 +37,8 @@ int igemm_num_cfgs();
 const char* igemm_cfg_name(int cfg);
 bool igemm_usable(const ConvProblem& p);
 int igemm_pick_cfg(const ConvProblem& p, int cu_count);
-int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int tile_cfg, const int8_t* src, const int8_t* flt,
-                      const int32_t* bias, const int8_t* z, int8_t* dst);
+int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int tile_cfg, int cu_count, const int8_t* src,
+                      const int8_t* flt, const int32_t* bias, const int8_t* z, int8_t* dst);
 
 bool depthwise_usable(const ConvProblem& p);
 int launch_conv_depthwise(hipStream_t st, const ConvProblem& p, const int8_t* src, const int8_t* flt,

@@ -6,12 +6,16 @@
 // requantised in registers by the fused epilogue (epilogue.h).  Activations and filters in the
 // reference's NCHW4 / NCHW32 layouts already hold the 16 consecutive k-bytes an MFMA lane needs
 // (NCHW32: one 16-byte run; NCHW4: four 4-byte runs), so the im2col matrix is never materialised:
-// each stage gathers a BN x BK activation tile and a BM x BK filter tile straight into LDS,
-// double-buffered against the MFMA loop, with an XOR swizzle on the 16-byte slots.
+// each stage gathers a BN x BK activation tile and a BM x BK filter tile straight into LDS.
 //
-// Data layout in LDS (per stage and operand): [row][BK bytes], BK = KCH * 32, 16-byte slot s of row r
-// stored at slot s ^ swz(r).  A k-chunk table {byte offset, fh, fw} for every 32-byte (NCHW32) or
-// 4-byte (NCHW4) k-unit is built once per workgroup, so the loaders do no divisions.
+// Schedule: persistent workgroups.  Each workgroup walks a list of output tiles and, inside a
+// tile, the k-stages; the two loops are flattened into one iteration space so that the global
+// loads of the next TWO iterations (registers R0/R1) are always in flight -- across tile
+// boundaries too, i.e. under the epilogue of the previous tile.  LDS is double buffered.
+//
+// Data layout in LDS (per buffer and operand): [row][BK bytes], BK = KCH * 32, 16-byte slot s of
+// row r stored at slot s ^ swz(r).  A k-unit table {byte offset, fh, fw} for every 32-byte (NCHW32)
+// or 4-byte (NCHW4) k-unit is built once per workgroup, so the loaders do no divisions.
 //
 // Accumulator layout of the 32x32 MFMA (lane l, register v): pixel = l % 32,
 // oc = 8*(v/4) + 4*(l/32) + v%4.  NCHW4 output stores one dword (4 channels) per register quad;
@@ -27,7 +31,32 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int IG_THREADS = 256;
-constexpr int IG_MAX_ENTRIES = 2048;  // k-chunk table capacity (entries of 8 bytes)
+constexpr int IG_MAX_ENTRIES = 2048;  // k-unit table capacity (entries of 8 bytes)
+
+// unsigned division by a runtime constant: q = (t + ((x - t) >> s1)) >> s2, t = mulhi(x, m)
+struct FastDiv {
+    uint32_t m, s1, s2, d;
+};
+
+FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d;
+    if (d <= 1) {
+        f.m = 0; f.s1 = 0; f.s2 = 0;
+        return f;
+    }
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    f.m = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    f.s1 = 1;
+    f.s2 = l - 1;
+    return f;
+}
+
+__device__ __forceinline__ uint32_t fdiv(uint32_t x, const FastDiv& f) {
+    uint32_t t = __umulhi(x, f.m);
+    return (t + ((x - t) >> f.s1)) >> f.s2;
+}
 
 struct IgemmArgs {
     const int8_t* src;
@@ -39,7 +68,6 @@ struct IgemmArgs {
     int IH, IW, OH, OW, OHW;
     int FH, FW, T;
     int sh, sw, ph, pw;
-    int CBI;          // input channel blocks (ic / PIN)
     int OC;
     int M;            // n * oh * ow
     int kbytes;       // filter bytes per output channel
@@ -49,8 +77,9 @@ struct IgemmArgs {
     int src_sn, src_scb;      // bytes: per image, per channel block
     int dst_sn, dst_scb;      // bytes: per image, per output channel block
     int z_sn;
-    int tiles_m, tiles_n;
+    int tiles_m, tiles_n, tiles;
     int has_bias;
+    FastDiv div_ohw, div_ow, div_t, div_fw;
     EpiParams epi;
 };
 
@@ -59,12 +88,18 @@ struct KEntry {
     int fhfw;   // fh | fw << 16 ; fh = 0x4000 marks a padding entry (never valid)
 };
 
-// 16-byte slot swizzle.  S = slots per row.  Rows r..r+15 read the same logical slot in one
-// ds_read_b128 wavefront pass and must land in distinct 4-bank groups of the 64 banks.
+// 16-byte slot swizzle (S = slots per row), derived from how gfx950 serves 128-bit LDS accesses
+// (measured with SQ_LDS_BANK_CONFLICT on single-wave probes):
+//   ds_read_b128 : 64 banks; 4 passes over all 64 lanes; in pass k lane l reads dword (k + l/16) % 4
+//   ds_write_b128: behaves as 32 banks; half-wave at a time, 4 passes; lane l writes dword (k + l/8) % 4
+// MFMA fragment reads (lane -> row l%32, slot-half l/32) need, per row class (row mod 256/ROWB rows),
+// distinct slots for the rows of one 16-lane group; loader writes (lane -> row l/2, half l%2) need
+// disjoint slot pairs for the rows of one 8-lane group.  With r_i = bit i of the row:
 template <int S>
 __device__ __forceinline__ int swz(int row) {
-    if (S == 4) return ((row >> 2) & 1) * 2 + ((row >> 3) & 1);
-    if (S == 8) return (((row >> 1) & 3) << 1) | ((row >> 3) & 1);
+    const int r0 = row & 1, r1 = (row >> 1) & 1, r2 = (row >> 2) & 1, r3 = (row >> 3) & 1;
+    if (S == 4) return ((r1 ^ r2) << 1) | r3;
+    if (S == 8) return (r1 << 2) | ((r0 ^ r2) << 1) | r3;
     return 0;
 }
 
@@ -81,45 +116,169 @@ struct IgemmKernel {
     static constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB;
     static constexpr int UA = BM * S / IG_THREADS;  // 16-byte units per thread per stage
     static constexpr int UB = BN * S / IG_THREADS;
-    static constexpr int LDS_BYTES = 2 * (A_BYTES + B_BYTES) + IG_MAX_ENTRIES * 8;
+    static constexpr int RB = BN >= 128 ? BN / 128 : 1;  // distinct pixel rows a loader thread serves
+    static constexpr int BIAS_BYTES = 2 * BM * 4;          // bias of the current / next tile's channels
+    static constexpr int STAGE_BYTES = 2 * (A_BYTES + B_BYTES) + BIAS_BYTES;
     static_assert(WM * WN * 64 == IG_THREADS, "4 waves");
     static_assert(UA >= 1 && UB >= 1, "tile too small for 256 loader threads");
     static_assert(MT >= 1 && NT >= 1, "wave tile");
 
-    // unit u of an operand with R rows: half = u & 1, row = (u >> 1) % R, chunk = (u >> 1) / R
+    struct Regs {
+        v4i a[UA];
+        v4i b[UB];
+    };
+    // loader-side state: which (tile, stage) the next issue() fetches, and the pixel rows of that tile
+    struct Loader {
+        int tile, stage;      // position in this workgroup's sequence
+        int oc0;
+        int base[RB], ih0[RB], iw0[RB];
+    };
+
+    __device__ static __forceinline__ void tile_coords(const IgemmArgs& a, int tile, int& oc0, int& pix0) {
+        const int tn = tile / a.tiles_m, tm = tile - tn * a.tiles_m;
+        oc0 = tm * BM;
+        pix0 = tn * BN;
+    }
+
+    __device__ static __forceinline__ void loader_enter_tile(const IgemmArgs& a, Loader& L, int tile, int t) {
+        int pix0;
+        tile_coords(a, tile, L.oc0, pix0);
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            const int row = ((t >> 1) % BN) + 128 * r;
+            const int m = pix0 + row;
+            const bool ok = m < a.M;
+            const uint32_t mm = ok ? m : 0;
+            const uint32_t n = fdiv(mm, a.div_ohw), rem = mm - n * a.OHW;
+            const uint32_t oh = fdiv(rem, a.div_ow), ow = rem - oh * a.OW;
+            const int ih0 = (int)oh * a.sh - a.ph, iw0 = (int)ow * a.sw - a.pw;
+            L.ih0[r] = ok ? ih0 : -0x8000;  // makes every tap fail the bounds test
+            L.iw0[r] = iw0;
+            L.base[r] = (int)n * a.src_sn + (ih0 * a.IW + iw0) * PIN;
+        }
+    }
+
+    __device__ static __forceinline__ void issue(const IgemmArgs& a, const Loader& L, const KEntry* tab,
+                                                 const __amdgpu_buffer_rsrc_t& rs_src,
+                                                 const __amdgpu_buffer_rsrc_t& rs_flt, Regs& R, int t) {
+        const int kc0 = L.stage * KCH;
+#pragma unroll
+        for (int j = 0; j < UA; ++j) {
+            const int v = (t >> 1) + 128 * j;
+            const int row = v % BM, chunk = v / BM;
+            const int oc = L.oc0 + row;
+            const int off = oc * a.kbytes + (kc0 + chunk) * 32 + (t & 1) * 16;
+            const bool ok = oc < a.OC && (kc0 + chunk) < a.KC;
+            R.a[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_flt, ok ? off : -1, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < UB; ++j) {
+            const int v = (t >> 1) + 128 * j;
+            const int r = BN >= 128 ? (j % RB) : 0;
+            const int chunk = v / BN;
+            if (PIN == 32) {
+                const KEntry k = tab[kc0 + chunk];
+                const int ih = L.ih0[r] + (k.fhfw & 0xffff), iw = L.iw0[r] + (k.fhfw >> 16);
+                const bool ok = (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
+                const int off = L.base[r] + k.off + (t & 1) * 16;
+                R.b[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_src, ok ? off : -1, 0, 0);
+            } else {
+                const int e0 = (kc0 + chunk) * 8 + (t & 1) * 4;
+                v4i x;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const KEntry k = tab[e0 + i];
+                    const int ih = L.ih0[r] + (k.fhfw & 0xffff), iw = L.iw0[r] + (k.fhfw >> 16);
+                    const bool ok = (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
+                    const int off = L.base[r] + k.off;
+                    x[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_src, ok ? off : -1, 0, 0);
+                }
+                R.b[j] = x;
+            }
+        }
+    }
+
+    __device__ static __forceinline__ void stash(int8_t* sA, int8_t* sB, const Regs& R, int t) {
+#pragma unroll
+        for (int j = 0; j < UA; ++j) {
+            const int v = (t >> 1) + 128 * j;
+            const int row = v % BM, chunk = v / BM;
+            const int slot = (chunk * 2 + (t & 1)) ^ swz<S>(row);
+            *reinterpret_cast<v4i*>(sA + row * ROWB + slot * 16) = R.a[j];
+        }
+#pragma unroll
+        for (int j = 0; j < UB; ++j) {
+            const int v = (t >> 1) + 128 * j;
+            const int row = v % BN, chunk = v / BN;
+            const int slot = (chunk * 2 + (t & 1)) ^ swz<S>(row);
+            *reinterpret_cast<v4i*>(sB + row * ROWB + slot * 16) = R.b[j];
+        }
+    }
+
+    // accumulators start from the bias of their output channel (held in LDS per tile)
+    __device__ static __forceinline__ void init_acc(v16i (&acc)[MT][NT], const int* sBias, int wm, int lh) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            v16i init;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const v4i b = *reinterpret_cast<const v4i*>(sBias + wm * WTM + i * 32 + 8 * q + 4 * lh);
+                init[4 * q + 0] = b[0]; init[4 * q + 1] = b[1]; init[4 * q + 2] = b[2]; init[4 * q + 3] = b[3];
+            }
+#pragma unroll
+            for (int j = 0; j < NT; ++j) acc[i][j] = init;
+        }
+    }
+
+    __device__ static __forceinline__ int fetch_bias(const IgemmArgs& a, int oc0, int t) {
+        const int oc = oc0 + t;
+        return (a.has_bias && t < BM && oc < a.OC) ? a.bias[oc] : 0;
+    }
+
     __device__ static __forceinline__ void run(const IgemmArgs& a) {
         extern __shared__ __attribute__((aligned(16))) int8_t lds[];
-        int8_t* sA = lds;
-        int8_t* sB = lds + 2 * A_BYTES;
-        KEntry* tab = reinterpret_cast<KEntry*>(lds + 2 * (A_BYTES + B_BYTES));
+        int8_t* sA = lds;                  // 2 buffers of A_BYTES
+        int8_t* sB = lds + 2 * A_BYTES;    // 2 buffers of B_BYTES
+        int* sBias = reinterpret_cast<int*>(lds + 2 * (A_BYTES + B_BYTES));  // 2 x BM
+        KEntry* tab = reinterpret_cast<KEntry*>(lds + STAGE_BYTES);
 
         const int t = threadIdx.x;
         const int lane = t & 63, wave = t >> 6;
         const int l32 = lane & 31, lh = lane >> 5;
         const int wm = wave / WN, wn = wave % WN;
 
-        // ---- workgroup -> tile, XCD aware: workgroups are dealt round-robin to the 8 XCDs, so give
-        // each XCD a contiguous run of tiles (neighbouring tiles share activations in that XCD's L2)
-        int logical;
+        // ---- this workgroup's tile sequence: first, first + step, ... (< last).
+        // Workgroups are dealt round-robin to the 8 XCDs; when the grid is a multiple of 8 every XCD
+        // owns a contiguous range of tiles (neighbouring tiles share activations and halos in that
+        // XCD's L2) and its workgroups stride through the range.
+        int first, step, last;
         {
-            const int nb = gridDim.x, bid = blockIdx.x;
-            const int per = nb >> 3, rem = nb & 7, x = bid & 7, i = bid >> 3;
-            logical = x < rem ? x * (per + 1) + i : rem * (per + 1) + (x - rem) * per + i;
+            const int G = gridDim.x, b = blockIdx.x;
+            if ((G & 7) == 0) {
+                const int x = b & 7, j = b >> 3, gx = G >> 3;
+                const int per = a.tiles >> 3, rem = a.tiles & 7;
+                const int t0 = x * per + (x < rem ? x : rem);
+                last = t0 + per + (x < rem ? 1 : 0);
+                first = t0 + j;
+                step = gx;
+            } else {
+                first = b; step = G; last = a.tiles;
+            }
         }
-        const int tile_n = logical / a.tiles_m, tile_m = logical - tile_n * a.tiles_m;
-        const int oc0 = tile_m * BM, pix0 = tile_n * BN;
+        const int my_tiles = first < last ? (last - first + step - 1) / step : 0;
+        const int total = my_tiles * a.nstages;
 
         // ---- k-unit table
         {
-            constexpr int UNIT = PIN == 32 ? 32 : 4;
-            const int cap = a.nstages * KCH * (32 / UNIT);
+            constexpr int UPC = PIN == 32 ? 1 : 8;  // units per 32-byte chunk
+            const int cap = a.nstages * KCH * UPC;
             for (int e = t; e < cap; e += IG_THREADS) {
                 KEntry k;
                 if (e < a.entries) {
-                    int cb = e / a.T, tap = e - cb * a.T;
-                    int fh = tap / a.FW, fw = tap - fh * a.FW;
-                    k.off = cb * a.src_scb + (fh * a.IW + fw) * PIN;
-                    k.fhfw = fh | (fw << 16);
+                    const uint32_t cb = fdiv(e, a.div_t), tap = e - cb * a.T;
+                    const uint32_t fh = fdiv(tap, a.div_fw), fw = tap - fh * a.FW;
+                    k.off = (int)cb * a.src_scb + ((int)fh * a.IW + (int)fw) * PIN;
+                    k.fhfw = (int)(fh | (fw << 16));
                 } else {
                     k.off = 0;
                     k.fhfw = 0x4000;
@@ -127,150 +286,125 @@ struct IgemmKernel {
                 tab[e] = k;
             }
         }
+        if (total == 0) return;
 
-        // ---- per-thread loader state
-        // B rows handled by this thread (RB of them), fixed for the whole K loop
-        constexpr int RB = BN >= 128 ? BN / 128 : 1;
-        int b_base[RB], b_ih0[RB], b_iw0[RB];
-#pragma unroll
-        for (int r = 0; r < RB; ++r) {
-            int row = ((t >> 1) % BN) + 128 * r;
-            int m = pix0 + row;
-            bool ok = m < a.M;
-            int mm = ok ? m : 0;
-            int n = mm / a.OHW, rem = mm - n * a.OHW;
-            int oh = rem / a.OW, ow = rem - oh * a.OW;
-            int ih0 = oh * a.sh - a.ph, iw0 = ow * a.sw - a.pw;
-            b_ih0[r] = ok ? ih0 : -0x8000;  // makes every tap fail the bounds test
-            b_iw0[r] = iw0;
-            b_base[r] = n * a.src_sn + (ih0 * a.IW + iw0) * PIN;
-        }
         const __amdgpu_buffer_rsrc_t rs_src = make_rsrc(a.src, a.src_bytes);
         const __amdgpu_buffer_rsrc_t rs_flt = make_rsrc(a.flt, a.flt_bytes);
 
-        v4i ra[UA], rb[UB];
-
-        auto load_stage = [&](int s) {
-            const int kc0 = s * KCH;
-            // filter units
-#pragma unroll
-            for (int j = 0; j < UA; ++j) {
-                int v = (t >> 1) + 128 * j;
-                int row = v % BM, chunk = v / BM;
-                int oc = oc0 + row;
-                int off = oc * a.kbytes + (kc0 + chunk) * 32 + (t & 1) * 16;
-                bool ok = oc < a.OC && (kc0 + chunk) < a.KC;
-                ra[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_flt, ok ? off : -1, 0, 0);
+        Loader L;
+        L.tile = first;
+        L.stage = 0;
+        loader_enter_tile(a, L, first, t);
+        int issued = 0;  // iterations whose loads have been issued
+        auto advance = [&]() __attribute__((always_inline)) {
+            ++issued;
+            if (++L.stage == a.nstages) {
+                L.stage = 0;
+                L.tile += step;
+                if (issued < total) loader_enter_tile(a, L, L.tile, t);
             }
-            // activation units
+            if (issued >= total) {
+                // past the end of this workgroup's work: every further load is out of range (returns 0,
+                // moves no data), which keeps issue/stash unconditional in the steady-state loop
+                L.oc0 = 0x40000000;
 #pragma unroll
-            for (int j = 0; j < UB; ++j) {
-                int v = (t >> 1) + 128 * j;
-                int r = BN >= 128 ? (j % RB) : 0;
-                int chunk = v / BN;
-                if (PIN == 32) {
-                    KEntry k = tab[kc0 + chunk];
-                    int ih = b_ih0[r] + (k.fhfw & 0xffff), iw = b_iw0[r] + (k.fhfw >> 16);
-                    bool ok = (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
-                    int off = b_base[r] + k.off + (t & 1) * 16;
-                    rb[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_src, ok ? off : -1, 0, 0);
-                } else {
-                    const int e0 = (kc0 + chunk) * 8 + (t & 1) * 4;
-                    v4i x;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        KEntry k = tab[e0 + i];
-                        int ih = b_ih0[r] + (k.fhfw & 0xffff), iw = b_iw0[r] + (k.fhfw >> 16);
-                        bool ok = (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
-                        int off = b_base[r] + k.off;
-                        x[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_src, ok ? off : -1, 0, 0);
-                    }
-                    rb[j] = x;
-                }
+                for (int r = 0; r < RB; ++r) L.ih0[r] = -0x8000;
             }
         };
 
-        auto store_stage = [&](int buf) {
-#pragma unroll
-            for (int j = 0; j < UA; ++j) {
-                int v = (t >> 1) + 128 * j;
-                int row = v % BM, chunk = v / BM;
-                int slot = (chunk * 2 + (t & 1)) ^ swz<S>(row);
-                *reinterpret_cast<v4i*>(sA + buf * A_BYTES + row * ROWB + slot * 16) = ra[j];
-            }
-#pragma unroll
-            for (int j = 0; j < UB; ++j) {
-                int v = (t >> 1) + 128 * j;
-                int row = v % BN, chunk = v / BN;
-                int slot = (chunk * 2 + (t & 1)) ^ swz<S>(row);
-                *reinterpret_cast<v4i*>(sB + buf * B_BYTES + row * ROWB + slot * 16) = rb[j];
-            }
-        };
-
-        // ---- accumulators, initialised with the bias of their output channel
-        v16i acc[MT][NT];
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            v16i init;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                int oc = oc0 + wm * WTM + i * 32 + 8 * q + 4 * lh;
-                v4i b = {0, 0, 0, 0};
-                if (a.has_bias && oc < a.OC) b = *reinterpret_cast<const v4i*>(a.bias + oc);
-                init[4 * q + 0] = b[0]; init[4 * q + 1] = b[1]; init[4 * q + 2] = b[2]; init[4 * q + 3] = b[3];
-            }
-#pragma unroll
-            for (int j = 0; j < NT; ++j) acc[i][j] = init;
-        }
-
+        Regs R0, R1;
         __syncthreads();  // table ready
-        load_stage(0);
-        store_stage(0);
+        issue(a, L, tab, rs_src, rs_flt, R0, t);
+        advance();
+        issue(a, L, tab, rs_src, rs_flt, R1, t);
+        advance();
+
+        // consumer-side state
+        int c_tile = first, c_stage = 0, c_oc0, c_pix0;
+        tile_coords(a, c_tile, c_oc0, c_pix0);
+        int c_par = 0;          // which half of sBias the current tile uses
+        int bias_next = 0;      // prefetched bias word of the next tile (threads < BM)
+        if (t < BM) sBias[t] = fetch_bias(a, c_oc0, t);
+        v16i acc[MT][NT];
+
+        stash(sA, sB, R0, t);
         __syncthreads();
 
-        for (int s = 0; s < a.nstages; ++s) {
-            const int buf = s & 1;
-            const bool more = s + 1 < a.nstages;
-            if (more) load_stage(s + 1);
+        auto phase = [&](int it, int buf, Regs& Rfree, Regs& Rnext) __attribute__((always_inline)) {
+            // Rfree was stashed into LDS in the previous phase; Rnext holds iteration it + 1
+            if (c_stage == 0) init_acc(acc, sBias + c_par * BM, wm, lh);
+            const bool last_stage = it < total && c_stage + 1 == a.nstages;
+            int n_oc0 = c_oc0, n_pix0 = c_pix0;
+            if (last_stage && it + 1 < total) {
+                tile_coords(a, c_tile + step, n_oc0, n_pix0);
+                if (a.tiles_m > 1) bias_next = fetch_bias(a, n_oc0, t);  // lands during the MFMAs + epilogue
+            }
+            issue(a, L, tab, rs_src, rs_flt, Rfree, t);  // iteration it + 2
+            advance();
             const int8_t* pA = sA + buf * A_BYTES;
             const int8_t* pB = sB + buf * B_BYTES;
-#pragma unroll
-            for (int c = 0; c < KCH; ++c) {
-                v4i fa[MT], fb[NT];
+            // LDS fragment reads run one k-chunk ahead of the MFMAs
+            v4i fa[2][MT], fb[2][NT];
+            auto frags = [&](int c, v4i (&xa)[MT], v4i (&xb)[NT]) __attribute__((always_inline)) {
 #pragma unroll
                 for (int i = 0; i < MT; ++i) {
-                    int row = wm * WTM + i * 32 + l32;
-                    int slot = (c * 2 + lh) ^ swz<S>(row);
-                    fa[i] = *reinterpret_cast<const v4i*>(pA + row * ROWB + slot * 16);
+                    const int row = wm * WTM + i * 32 + l32;
+                    const int slot = (c * 2 + lh) ^ swz<S>(row);
+                    xa[i] = *reinterpret_cast<const v4i*>(pA + row * ROWB + slot * 16);
                 }
 #pragma unroll
                 for (int j = 0; j < NT; ++j) {
-                    int row = wn * WTN + j * 32 + l32;
-                    int slot = (c * 2 + lh) ^ swz<S>(row);
-                    fb[j] = *reinterpret_cast<const v4i*>(pB + row * ROWB + slot * 16);
+                    const int row = wn * WTN + j * 32 + l32;
+                    const int slot = (c * 2 + lh) ^ swz<S>(row);
+                    xb[j] = *reinterpret_cast<const v4i*>(pB + row * ROWB + slot * 16);
                 }
+            };
+            frags(0, fa[0], fb[0]);
+#pragma unroll
+            for (int c = 0; c < KCH; ++c) {
+                if (c + 1 < KCH) frags(c + 1, fa[(c + 1) & 1], fb[(c + 1) & 1]);
 #pragma unroll
                 for (int i = 0; i < MT; ++i)
 #pragma unroll
                     for (int j = 0; j < NT; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[c & 1][i], fb[c & 1][j], acc[i][j], 0, 0, 0);
             }
-            if (more) store_stage(buf ^ 1);
+            if (last_stage) {
+                run_epilogue(a, acc, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh);
+                c_stage = 0;
+                c_tile += step;
+                if (a.tiles_m > 1) {
+                    c_par ^= 1;
+                    if (t < BM) sBias[c_par * BM + t] = bias_next;
+                }
+                c_oc0 = n_oc0;
+                c_pix0 = n_pix0;
+            } else {
+                ++c_stage;
+            }
+            stash(sA + (buf ^ 1) * A_BYTES, sB + (buf ^ 1) * B_BYTES, Rnext, t);
             __syncthreads();
-        }
+        };
 
-        // ---- epilogue
+        for (int it = 0; it < total; it += 2) {
+            phase(it, 0, R0, R1);
+            phase(it + 1, 1, R1, R0);  // when it + 1 == total this is a dead phase on zero-filled LDS
+        }
+    }
+
+    __device__ static __forceinline__ void run_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w,
+                                                        int l32, int lh) {
         if (a.epi.has_z) {
             switch (a.epi.nonline) {
-                case NL_RELU: epilogue<NL_RELU, true>(a, acc, oc0 + wm * WTM, pix0 + wn * WTN, l32, lh); break;
-                case NL_H_SWISH: epilogue<NL_H_SWISH, true>(a, acc, oc0 + wm * WTM, pix0 + wn * WTN, l32, lh); break;
-                default: epilogue<NL_IDENTITY, true>(a, acc, oc0 + wm * WTM, pix0 + wn * WTN, l32, lh); break;
+                case NL_RELU: epilogue<NL_RELU, true>(a, acc, oc_w, pix_w, l32, lh); break;
+                case NL_H_SWISH: epilogue<NL_H_SWISH, true>(a, acc, oc_w, pix_w, l32, lh); break;
+                default: epilogue<NL_IDENTITY, true>(a, acc, oc_w, pix_w, l32, lh); break;
             }
         } else {
             switch (a.epi.nonline) {
-                case NL_RELU: epilogue<NL_RELU, false>(a, acc, oc0 + wm * WTM, pix0 + wn * WTN, l32, lh); break;
-                case NL_H_SWISH: epilogue<NL_H_SWISH, false>(a, acc, oc0 + wm * WTM, pix0 + wn * WTN, l32, lh); break;
-                default: epilogue<NL_IDENTITY, false>(a, acc, oc0 + wm * WTM, pix0 + wn * WTN, l32, lh); break;
+                case NL_RELU: epilogue<NL_RELU, false>(a, acc, oc_w, pix_w, l32, lh); break;
+                case NL_H_SWISH: epilogue<NL_H_SWISH, false>(a, acc, oc_w, pix_w, l32, lh); break;
+                default: epilogue<NL_IDENTITY, false>(a, acc, oc_w, pix_w, l32, lh); break;
             }
         }
     }
@@ -283,10 +417,10 @@ struct IgemmKernel {
         for (int j = 0; j < NT; ++j) {
             const int m = pix_w + j * 32 + l32;
             const bool pok = m < a.M;
-            const int mm = pok ? m : 0;
-            const int n = mm / a.OHW, rem = mm - n * a.OHW;
-            const int d_pix = n * a.dst_sn + rem * POUT;
-            const int z_pix = n * a.z_sn + rem * POUT;
+            const uint32_t mm = pok ? m : 0;
+            const uint32_t n = fdiv(mm, a.div_ohw), rem = mm - n * a.OHW;
+            const int d_pix = (int)n * a.dst_sn + (int)rem * POUT;
+            const int z_pix = (int)n * a.z_sn + (int)rem * POUT;
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
                 const int ocb = oc_w + i * 32;  // first channel of this 32-channel block
@@ -328,55 +462,80 @@ struct IgemmKernel {
     }
 };
 
-template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH>
-__global__ __launch_bounds__(IG_THREADS) void igemm_kernel(IgemmArgs a) {
+template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH, int MINW>
+__global__ __launch_bounds__(IG_THREADS, MINW) void igemm_kernel(IgemmArgs a) {
     IgemmKernel<PIN, POUT, BM, BN, WM, WN, KCH>::run(a);
 }
 
 struct TileCfg {
     const char* name;
-    int bm, bn;
+    int bm, bn, kch;
 };
 // index = tile_cfg of mi355_algo
 const TileCfg kCfgs[] = {
-        {"128x128", 128, 128},
-        {"64x256", 64, 256},
-        {"256x128", 256, 128},
-        {"64x64", 64, 64},
-        {"32x256", 32, 256},
+        {"128x128x64", 128, 128, 2},
+        {"64x256x64", 64, 256, 2},
+        {"256x128x64", 256, 128, 2},
+        {"64x64x128", 64, 64, 4},
+        {"32x256x128", 32, 256, 4},
+        {"128x128x128", 128, 128, 4},
+        {"64x128x128", 64, 128, 4},
+        {"128x64x128", 128, 64, 4},
 };
 constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
 
-template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH>
-int launch_one(hipStream_t st, IgemmArgs& a) {
+template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH, int MINW>
+int launch_one(hipStream_t st, IgemmArgs& a, int cu_count) {
     using K = IgemmKernel<PIN, POUT, BM, BN, WM, WN, KCH>;
     a.tiles_m = (a.OC + BM - 1) / BM;
     a.tiles_n = (a.M + BN - 1) / BN;
+    const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
+    if (tiles <= 0 || tiles > 0x3fffffff) return (int)hipErrorInvalidValue;
+    a.tiles = (int)tiles;
     a.nstages = (a.KC + KCH - 1) / KCH;
-    auto kern = igemm_kernel<PIN, POUT, BM, BN, WM, WN, KCH>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, K::LDS_BYTES);
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
-    const int64_t grid = (int64_t)a.tiles_m * a.tiles_n;
-    if (grid <= 0 || grid > 0x7fffffff) return (int)hipErrorInvalidValue;
     const int tab_entries = a.nstages * KCH * (PIN == 32 ? 1 : 8);
-    const int lds = 2 * (K::A_BYTES + K::B_BYTES) + tab_entries * 8;
+    const int lds = K::STAGE_BYTES + tab_entries * 8;
+    auto kern = igemm_kernel<PIN, POUT, BM, BN, WM, WN, KCH, MINW>;
+    static int max_lds_set = 0;
+    if (lds > max_lds_set) {
+        const int want = K::STAGE_BYTES + IG_MAX_ENTRIES * 8;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, want);
+        if (e != hipSuccess) return (int)e;
+        max_lds_set = want;
+    }
+    // persistent grid: as many workgroups as fit on the device at once
+    static int occ_lds = -1, occ_val = 0;  // last query of this instantiation
+    int occ = occ_val;
+    if (occ_lds != lds) {
+        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(kern),
+                                                                    IG_THREADS, (size_t)lds);
+        if (e != hipSuccess || occ < 1) {
+            (void)hipGetLastError();
+            occ = 1;
+        }
+        occ_lds = lds;
+        occ_val = occ;
+    }
+    if (cu_count <= 0) cu_count = 256;
+    int64_t grid = (int64_t)occ * cu_count;
+    if (grid > tiles) grid = tiles;
+    if (grid >= 8) grid &= ~(int64_t)7;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(IG_THREADS), lds, st, a);
     return (int)hipGetLastError();
 }
 
 template <int PIN, int POUT>
-int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg) {
+int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
     switch (cfg) {
-        case 0: return launch_one<PIN, POUT, 128, 128, 2, 2, 2>(st, a);
-        case 1: return launch_one<PIN, POUT, 64, 256, 1, 4, 2>(st, a);
-        case 2: return launch_one<PIN, POUT, 256, 128, 2, 2, 2>(st, a);
-        case 3: return launch_one<PIN, POUT, 64, 64, 2, 2, 4>(st, a);
-        case 4: return launch_one<PIN, POUT, 32, 256, 1, 4, 4>(st, a);
+        case 0: return launch_one<PIN, POUT, 128, 128, 2, 2, 2, 2>(st, a, cu);
+        case 1: return launch_one<PIN, POUT, 64, 256, 1, 4, 2, 2>(st, a, cu);
+        case 2: return launch_one<PIN, POUT, 256, 128, 2, 2, 2, 1>(st, a, cu);
+        case 3: return launch_one<PIN, POUT, 64, 64, 2, 2, 4, 3>(st, a, cu);
+        case 4: return launch_one<PIN, POUT, 32, 256, 1, 4, 4, 2>(st, a, cu);
+        case 5: return launch_one<PIN, POUT, 128, 128, 2, 2, 4, 2>(st, a, cu);
+        case 6: return launch_one<PIN, POUT, 64, 128, 2, 2, 4, 3>(st, a, cu);
+        case 7: return launch_one<PIN, POUT, 128, 64, 2, 2, 4, 3>(st, a, cu);
         default: return (int)hipErrorInvalidValue;
     }
 }
@@ -416,22 +575,23 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
     const int OC = d.oc;
     if (cu_count <= 0) cu_count = 256;
     auto tiles = [&](int cfg) { return ((OC + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm) * ((M + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn); };
+    const int kbytes = d.ic * d.fh * d.fw;
+    const bool long_k = kbytes >= 256;
     if (OC <= 32) return 4;
     if (OC <= 64) return tiles(1) >= cu_count ? 1 : 3;
-    if (OC % 256 == 0 && tiles(2) >= 2 * cu_count) return 2;
-    if (tiles(0) >= cu_count) return 0;
+    if (tiles(0) >= 2 * cu_count) return long_k ? 5 : 0;
+    if (tiles(6) >= cu_count) return 6;
     return 3;
 }
 
-int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, const int8_t* src, const int8_t* flt,
-                      const int32_t* bias, const int8_t* z, int8_t* dst) {
+int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_count, const int8_t* src,
+                      const int8_t* flt, const int32_t* bias, const int8_t* z, int8_t* dst) {
     const mi355_conv_desc& d = p.d;
     IgemmArgs a;
     a.src = src; a.flt = flt; a.bias = bias; a.z = z; a.dst = dst;
     a.IH = d.ih; a.IW = d.iw; a.OH = p.oh; a.OW = p.ow; a.OHW = p.oh * p.ow;
     a.FH = d.fh; a.FW = d.fw; a.T = d.fh * d.fw;
     a.sh = d.stride_h; a.sw = d.stride_w; a.ph = d.pad_h; a.pw = d.pad_w;
-    a.CBI = d.ic / p.pin;
     a.OC = d.oc;
     a.M = d.n * p.oh * p.ow;
     a.kbytes = d.ic * d.fh * d.fw;
@@ -447,12 +607,16 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, const int8_
     a.dst_bytes = (uint32_t)((int64_t)(d.n - 1) * p.dst_sn + (int64_t)d.oc * a.OHW);
     a.z_bytes = d.has_z ? (uint32_t)((int64_t)(d.n - 1) * p.z_sn + (int64_t)d.oc * a.OHW) : 0;
     a.has_bias = d.bias_mode == MI355_BIAS_BROADCAST_CHANNEL;
+    a.div_ohw = make_fastdiv(a.OHW);
+    a.div_ow = make_fastdiv(a.OW);
+    a.div_t = make_fastdiv(a.T);
+    a.div_fw = make_fastdiv(a.FW);
     a.epi = p.epi;
     if (a.M == 0 || a.OC == 0) return 0;
-    if (p.pin == 32 && p.pout == 32) return launch_fmt<32, 32>(st, a, cfg);
-    if (p.pin == 4 && p.pout == 4) return launch_fmt<4, 4>(st, a, cfg);
-    if (p.pin == 4 && p.pout == 32) return launch_fmt<4, 32>(st, a, cfg);
-    return launch_fmt<32, 4>(st, a, cfg);
+    if (p.pin == 32 && p.pout == 32) return launch_fmt<32, 32>(st, a, cfg, cu_count);
+    if (p.pin == 4 && p.pout == 4) return launch_fmt<4, 4>(st, a, cfg, cu_count);
+    if (p.pin == 4 && p.pout == 32) return launch_fmt<4, 32>(st, a, cfg, cu_count);
+    return launch_fmt<32, 4>(st, a, cfg, cu_count);
 }
 
 }  // namespace mi355

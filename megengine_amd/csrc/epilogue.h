@@ -94,10 +94,10 @@ __device__ __forceinline__ int requant_s8_fast(int sfb, int z, const EpiParams& 
     float q = __builtin_fmaf(res, e.y_hi, q0);
     int out;
     if (NL == NL_RELU) {
-        q = fminf(fmaxf(q, 0.f), 127.f);
+        q = __builtin_amdgcn_fmed3f(q, 0.f, 127.f);  // q is finite here: same as min(max(q, 0), 127)
         out = (int)(q + 0.49999997f);
     } else {
-        q = fminf(fmaxf(q, -128.f), 127.f);
+        q = __builtin_amdgcn_fmed3f(q, -128.f, 127.f);
         out = (int)(q + __builtin_copysignf(0.49999997f, q));
     }
     return out;
