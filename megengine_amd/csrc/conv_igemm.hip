@@ -100,6 +100,7 @@ __device__ __forceinline__ int swz(int row) {
     const int r0 = row & 1, r1 = (row >> 1) & 1, r2 = (row >> 2) & 1, r3 = (row >> 3) & 1;
     if (S == 4) return ((r1 ^ r2) << 1) | r3;
     if (S == 8) return (r1 << 2) | ((r0 ^ r2) << 1) | r3;
+    if (S == 16) return r2 | (r0 << 1) | (r1 << 2) | (r3 << 3);
     return 0;
 }
 
@@ -107,7 +108,11 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
 
-template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH>
+constexpr int SENT = (int)0x80000000;  // byte offset that is out of range for every buffer (< 2 GiB)
+
+// PW = pointwise fast path: 1x1 filter, no padding, K a multiple of the stage depth.  Its loaders need no
+// bounds tests and no k-unit table: every address is a per-row base plus a wave-uniform term.
+template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH, bool PW>
 struct IgemmKernel {
     static constexpr int WTM = BM / WM, WTN = BN / WN;
     static constexpr int MT = WTM / 32, NT = WTN / 32;
@@ -116,7 +121,13 @@ struct IgemmKernel {
     static constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB;
     static constexpr int UA = BM * S / IG_THREADS;  // 16-byte units per thread per stage
     static constexpr int UB = BN * S / IG_THREADS;
-    static constexpr int RB = BN >= 128 ? BN / 128 : 1;  // distinct pixel rows a loader thread serves
+    // Activation unit j: row pass j % RB (rows (t/2) + 128 * pass), k-chunk csel + CSB * (j / RB): lanes run along
+    // pixels, which are contiguous in memory for one channel block.
+    // Filter unit j: slot t % S of row t / S + RPA * j: lanes run along k, so that every filter row contributes one
+    // whole contiguous BK-byte run (full cache lines) per load instruction.
+    static constexpr int RB = BN >= 128 ? BN / 128 : 1;
+    static constexpr int CSB = BN >= 128 ? 1 : 128 / BN;
+    static constexpr int RPA = IG_THREADS / S;  // filter rows per loader pass
     static constexpr int BIAS_BYTES = 2 * BM * 4;          // bias of the current / next tile's channels
     static constexpr int STAGE_BYTES = 2 * (A_BYTES + B_BYTES) + BIAS_BYTES;
     static_assert(WM * WN * 64 == IG_THREADS, "4 waves");
@@ -127,12 +138,18 @@ struct IgemmKernel {
         v4i a[UA];
         v4i b[UB];
     };
-    // loader-side state: which (tile, stage) the next issue() fetches, and the pixel rows of that tile
+    // loader-side state: which (tile, stage) the next issue() fetches, and the rows of that tile
     struct Loader {
-        int tile, stage;      // position in this workgroup's sequence
-        int oc0;
-        int base[RB], ih0[RB], iw0[RB];
+        int tile, stage, kc0;   // position in this workgroup's sequence; kc0 = stage * KCH
+        int a_base[UA];         // filter row byte offset (+ lane slot), SENT for rows past OC
+        int b_base[RB];         // pixel byte offset (+ lane half); PW: SENT for rows past M
+        int ih0[RB], iw0[RB];   // table path: top-left input coordinate (ih0 = -0x8000 for rows past M)
     };
+
+    __device__ static __forceinline__ int rowA(int t, int j) { return t / S + RPA * j; }
+    __device__ static __forceinline__ int rowB(int t, int j) { return BN >= 128 ? (t >> 1) + 128 * (j % RB) : (t >> 1) % BN; }
+    // wave-uniform first chunk of this thread's units (non-zero only for tiles with fewer than 128 rows)
+    __device__ static __forceinline__ int cselB(int t) { return BN >= 128 ? 0 : __builtin_amdgcn_readfirstlane((t >> 1) / BN); }
 
     __device__ static __forceinline__ void tile_coords(const IgemmArgs& a, int tile, int& oc0, int& pix0) {
         const int tn = tile / a.tiles_m, tm = tile - tn * a.tiles_m;
@@ -141,57 +158,82 @@ struct IgemmKernel {
     }
 
     __device__ static __forceinline__ void loader_enter_tile(const IgemmArgs& a, Loader& L, int tile, int t) {
-        int pix0;
-        tile_coords(a, tile, L.oc0, pix0);
+        int oc0, pix0;
+        tile_coords(a, tile, oc0, pix0);
+#pragma unroll
+        for (int r = 0; r < UA; ++r) {
+            const int oc = oc0 + rowA(t, r);
+            L.a_base[r] = oc < a.OC ? oc * a.kbytes + (t % S) * 16 : SENT;
+        }
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
-            const int row = ((t >> 1) % BN) + 128 * r;
-            const int m = pix0 + row;
+            const int m = pix0 + rowB(t, r);
             const bool ok = m < a.M;
             const uint32_t mm = ok ? m : 0;
             const uint32_t n = fdiv(mm, a.div_ohw), rem = mm - n * a.OHW;
             const uint32_t oh = fdiv(rem, a.div_ow), ow = rem - oh * a.OW;
             const int ih0 = (int)oh * a.sh - a.ph, iw0 = (int)ow * a.sw - a.pw;
+            const int lane_part = PIN == 32 ? (t & 1) * 16 : (PW ? (t & 1) * 4 * a.src_scb : 0);
+            const int base = (int)n * a.src_sn + (ih0 * a.IW + iw0) * PIN + lane_part;
+            L.b_base[r] = (PW && !ok) ? SENT : base;
             L.ih0[r] = ok ? ih0 : -0x8000;  // makes every tap fail the bounds test
             L.iw0[r] = iw0;
-            L.base[r] = (int)n * a.src_sn + (ih0 * a.IW + iw0) * PIN;
         }
     }
 
+    __device__ static __forceinline__ void loader_kill(Loader& L) {
+        // past the end of this workgroup's work: every further load is out of range (returns 0, moves no
+        // data), which keeps issue/stash unconditional in the steady-state loop
+#pragma unroll
+        for (int r = 0; r < UA; ++r) L.a_base[r] = SENT;
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            L.b_base[r] = SENT;
+            L.ih0[r] = -0x8000;
+        }
+        L.kc0 = 0;
+    }
+
+    // Global loads of one stage into registers.  Straight-line code: every offset is fully bounds-checked
+    // by the buffer descriptor, invalid rows/taps use the SENT offset and return zeros.
     __device__ static __forceinline__ void issue(const IgemmArgs& a, const Loader& L, const KEntry* tab,
                                                  const __amdgpu_buffer_rsrc_t& rs_src,
                                                  const __amdgpu_buffer_rsrc_t& rs_flt, Regs& R, int t) {
-        const int kc0 = L.stage * KCH;
+        const int cb = cselB(t);
+        // bytes past the end of a filter row (last stage of a K that is not a multiple of BK) belong to the next
+        // row or are out of range (zeros): either way they meet zero activations
 #pragma unroll
-        for (int j = 0; j < UA; ++j) {
-            const int v = (t >> 1) + 128 * j;
-            const int row = v % BM, chunk = v / BM;
-            const int oc = L.oc0 + row;
-            const int off = oc * a.kbytes + (kc0 + chunk) * 32 + (t & 1) * 16;
-            const bool ok = oc < a.OC && (kc0 + chunk) < a.KC;
-            R.a[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_flt, ok ? off : -1, 0, 0);
-        }
+        for (int j = 0; j < UA; ++j)
+            R.a[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_flt, L.a_base[j] + L.kc0 * 32, 0, 0);
 #pragma unroll
         for (int j = 0; j < UB; ++j) {
-            const int v = (t >> 1) + 128 * j;
-            const int r = BN >= 128 ? (j % RB) : 0;
-            const int chunk = v / BN;
-            if (PIN == 32) {
-                const KEntry k = tab[kc0 + chunk];
-                const int ih = L.ih0[r] + (k.fhfw & 0xffff), iw = L.iw0[r] + (k.fhfw >> 16);
+            const int r = j % RB;
+            const int kc = L.kc0 + cb + CSB * (j / RB);  // wave-uniform
+            if (PW) {
+                if (PIN == 32) {
+                    R.b[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_src, L.b_base[r] + kc * a.src_scb, 0, 0);
+                } else {
+                    v4i x;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        x[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_src, L.b_base[r] + (kc * 8 + i) * a.src_scb, 0, 0);
+                    R.b[j] = x;
+                }
+            } else if (PIN == 32) {
+                const KEntry k = tab[kc];
+                const int k_off = __builtin_amdgcn_readfirstlane(k.off), k_fhfw = __builtin_amdgcn_readfirstlane(k.fhfw);
+                const int ih = L.ih0[r] + (k_fhfw & 0xffff), iw = L.iw0[r] + (k_fhfw >> 16);
                 const bool ok = (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
-                const int off = L.base[r] + k.off + (t & 1) * 16;
-                R.b[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_src, ok ? off : -1, 0, 0);
+                R.b[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_src, ok ? L.b_base[r] + k_off : SENT, 0, 0);
             } else {
-                const int e0 = (kc0 + chunk) * 8 + (t & 1) * 4;
+                const int e0 = kc * 8 + (t & 1) * 4;
                 v4i x;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const KEntry k = tab[e0 + i];
                     const int ih = L.ih0[r] + (k.fhfw & 0xffff), iw = L.iw0[r] + (k.fhfw >> 16);
                     const bool ok = (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
-                    const int off = L.base[r] + k.off;
-                    x[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_src, ok ? off : -1, 0, 0);
+                    x[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_src, ok ? L.b_base[r] + k.off : SENT, 0, 0);
                 }
                 R.b[j] = x;
             }
@@ -199,17 +241,16 @@ struct IgemmKernel {
     }
 
     __device__ static __forceinline__ void stash(int8_t* sA, int8_t* sB, const Regs& R, int t) {
+        const int cb = cselB(t);
 #pragma unroll
         for (int j = 0; j < UA; ++j) {
-            const int v = (t >> 1) + 128 * j;
-            const int row = v % BM, chunk = v / BM;
-            const int slot = (chunk * 2 + (t & 1)) ^ swz<S>(row);
+            const int row = rowA(t, j);
+            const int slot = (t % S) ^ swz<S>(row);
             *reinterpret_cast<v4i*>(sA + row * ROWB + slot * 16) = R.a[j];
         }
 #pragma unroll
         for (int j = 0; j < UB; ++j) {
-            const int v = (t >> 1) + 128 * j;
-            const int row = v % BN, chunk = v / BN;
+            const int row = rowB(t, j), chunk = cb + CSB * (j / RB);
             const int slot = (chunk * 2 + (t & 1)) ^ swz<S>(row);
             *reinterpret_cast<v4i*>(sB + row * ROWB + slot * 16) = R.b[j];
         }
@@ -268,8 +309,8 @@ struct IgemmKernel {
         const int my_tiles = first < last ? (last - first + step - 1) / step : 0;
         const int total = my_tiles * a.nstages;
 
-        // ---- k-unit table
-        {
+        // ---- k-unit table (not needed by the pointwise path)
+        if (!PW) {
             constexpr int UPC = PIN == 32 ? 1 : 8;  // units per 32-byte chunk
             const int cap = a.nstages * KCH * UPC;
             for (int e = t; e < cap; e += IG_THREADS) {
@@ -294,22 +335,19 @@ struct IgemmKernel {
         Loader L;
         L.tile = first;
         L.stage = 0;
+        L.kc0 = 0;
         loader_enter_tile(a, L, first, t);
         int issued = 0;  // iterations whose loads have been issued
         auto advance = [&]() __attribute__((always_inline)) {
             ++issued;
+            L.kc0 += KCH;
             if (++L.stage == a.nstages) {
                 L.stage = 0;
+                L.kc0 = 0;
                 L.tile += step;
                 if (issued < total) loader_enter_tile(a, L, L.tile, t);
             }
-            if (issued >= total) {
-                // past the end of this workgroup's work: every further load is out of range (returns 0,
-                // moves no data), which keeps issue/stash unconditional in the steady-state loop
-                L.oc0 = 0x40000000;
-#pragma unroll
-                for (int r = 0; r < RB; ++r) L.ih0[r] = -0x8000;
-            }
+            if (issued >= total) loader_kill(L);
         };
 
         Regs R0, R1;
@@ -326,25 +364,35 @@ struct IgemmKernel {
         int bias_next = 0;      // prefetched bias word of the next tile (threads < BM)
         if (t < BM) sBias[t] = fetch_bias(a, c_oc0, t);
         v16i acc[MT][NT];
+        // a wave with a single 32x32 tile alternates two accumulators so that consecutive MFMAs are independent
+        constexpr bool DUAL = MT * NT == 1;
+        v16i alt;
 
         stash(sA, sB, R0, t);
         __syncthreads();
 
         auto phase = [&](int it, int buf, Regs& Rfree, Regs& Rnext) __attribute__((always_inline)) {
             // Rfree was stashed into LDS in the previous phase; Rnext holds iteration it + 1
-            if (c_stage == 0) init_acc(acc, sBias + c_par * BM, wm, lh);
+            if (c_stage == 0) {
+                init_acc(acc, sBias + c_par * BM, wm, lh);
+                if (DUAL) alt = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            }
             const bool last_stage = it < total && c_stage + 1 == a.nstages;
             int n_oc0 = c_oc0, n_pix0 = c_pix0;
             if (last_stage && it + 1 < total) {
                 tile_coords(a, c_tile + step, n_oc0, n_pix0);
                 if (a.tiles_m > 1) bias_next = fetch_bias(a, n_oc0, t);  // lands during the MFMAs + epilogue
             }
-            issue(a, L, tab, rs_src, rs_flt, Rfree, t);  // iteration it + 2
-            advance();
+            // ---- one straight-line block: loads of iteration it + 2, MFMAs of iteration it with their
+            // LDS fragment reads running one k-chunk ahead, then iteration it + 1 goes to the other buffer
+            issue(a, L, tab, rs_src, rs_flt, Rfree, t);
             const int8_t* pA = sA + buf * A_BYTES;
             const int8_t* pB = sB + buf * B_BYTES;
-            // LDS fragment reads run one k-chunk ahead of the MFMAs
-            v4i fa[2][MT], fb[2][NT];
+            // Fragment reads run ahead of the MFMAs: the whole stage when it fits in registers, else one
+            // k-chunk ahead.  The LDS writes of iteration it + 1 are issued before the MFMAs so that their
+            // latency hides under the matrix pipeline.
+            constexpr int FD = KCH * (MT + NT) <= 12 ? KCH : 2;
+            v4i fa[FD][MT], fb[FD][NT];
             auto frags = [&](int c, v4i (&xa)[MT], v4i (&xb)[NT]) __attribute__((always_inline)) {
 #pragma unroll
                 for (int i = 0; i < MT; ++i) {
@@ -359,17 +407,37 @@ struct IgemmKernel {
                     xb[j] = *reinterpret_cast<const v4i*>(pB + row * ROWB + slot * 16);
                 }
             };
-            frags(0, fa[0], fb[0]);
-#pragma unroll
-            for (int c = 0; c < KCH; ++c) {
-                if (c + 1 < KCH) frags(c + 1, fa[(c + 1) & 1], fb[(c + 1) & 1]);
+            auto mfmas = [&](int c, const v4i (&xa)[MT], const v4i (&xb)[NT]) __attribute__((always_inline)) {
 #pragma unroll
                 for (int i = 0; i < MT; ++i)
 #pragma unroll
-                    for (int j = 0; j < NT; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[c & 1][i], fb[c & 1][j], acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < NT; ++j) {
+                        if (DUAL && (c & 1))
+                            alt = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa[i], xb[j], alt, 0, 0, 0);
+                        else
+                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa[i], xb[j], acc[i][j], 0, 0, 0);
+                    }
+            };
+            if (FD == KCH) {
+#pragma unroll
+                for (int c = 0; c < KCH; ++c) frags(c, fa[c], fb[c]);
+                __builtin_amdgcn_sched_barrier(0);
+                stash(sA + (buf ^ 1) * A_BYTES, sB + (buf ^ 1) * B_BYTES, Rnext, t);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int c = 0; c < KCH; ++c) mfmas(c, fa[c], fb[c]);
+            } else {
+                frags(0, fa[0], fb[0]);
+                stash(sA + (buf ^ 1) * A_BYTES, sB + (buf ^ 1) * B_BYTES, Rnext, t);
+#pragma unroll
+                for (int c = 0; c < KCH; ++c) {
+                    if (c + 1 < KCH) frags(c + 1, fa[(c + 1) & 1], fb[(c + 1) & 1]);
+                    mfmas(c, fa[c & 1], fb[c & 1]);
+                }
             }
+            // ---- bookkeeping
             if (last_stage) {
+                if (DUAL) acc[0][0] += alt;
                 run_epilogue(a, acc, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh);
                 c_stage = 0;
                 c_tile += step;
@@ -382,7 +450,7 @@ struct IgemmKernel {
             } else {
                 ++c_stage;
             }
-            stash(sA + (buf ^ 1) * A_BYTES, sB + (buf ^ 1) * B_BYTES, Rnext, t);
+            advance();
             __syncthreads();
         };
 
@@ -462,9 +530,9 @@ struct IgemmKernel {
     }
 };
 
-template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH, int MINW>
+template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH, int MINW, bool PW>
 __global__ __launch_bounds__(IG_THREADS, MINW) void igemm_kernel(IgemmArgs a) {
-    IgemmKernel<PIN, POUT, BM, BN, WM, WN, KCH>::run(a);
+    IgemmKernel<PIN, POUT, BM, BN, WM, WN, KCH, PW>::run(a);
 }
 
 struct TileCfg {
@@ -484,18 +552,18 @@ const TileCfg kCfgs[] = {
 };
 constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
 
-template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH, int MINW>
-int launch_one(hipStream_t st, IgemmArgs& a, int cu_count) {
-    using K = IgemmKernel<PIN, POUT, BM, BN, WM, WN, KCH>;
+template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH, int MINW, bool PW>
+int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
+    using K = IgemmKernel<PIN, POUT, BM, BN, WM, WN, KCH, PW>;
     a.tiles_m = (a.OC + BM - 1) / BM;
     a.tiles_n = (a.M + BN - 1) / BN;
     const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
     if (tiles <= 0 || tiles > 0x3fffffff) return (int)hipErrorInvalidValue;
     a.tiles = (int)tiles;
     a.nstages = (a.KC + KCH - 1) / KCH;
-    const int tab_entries = a.nstages * KCH * (PIN == 32 ? 1 : 8);
+    const int tab_entries = PW ? 0 : a.nstages * KCH * (PIN == 32 ? 1 : 8);
     const int lds = K::STAGE_BYTES + tab_entries * 8;
-    auto kern = igemm_kernel<PIN, POUT, BM, BN, WM, WN, KCH, MINW>;
+    auto kern = igemm_kernel<PIN, POUT, BM, BN, WM, WN, KCH, MINW, PW>;
     static int max_lds_set = 0;
     if (lds > max_lds_set) {
         const int want = K::STAGE_BYTES + IG_MAX_ENTRIES * 8;
@@ -525,6 +593,14 @@ int launch_one(hipStream_t st, IgemmArgs& a, int cu_count) {
     return (int)hipGetLastError();
 }
 
+template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH, int MINW>
+int launch_one(hipStream_t st, IgemmArgs& a, int cu_count) {
+    // pointwise fast path: 1x1, no padding, whole stages of K
+    const bool pw = a.T == 1 && a.ph == 0 && a.pw == 0 && a.kbytes % (32 * KCH) == 0;
+    if (pw) return launch_pw<PIN, POUT, BM, BN, WM, WN, KCH, MINW, true>(st, a, cu_count);
+    return launch_pw<PIN, POUT, BM, BN, WM, WN, KCH, MINW, false>(st, a, cu_count);
+}
+
 template <int PIN, int POUT>
 int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
     switch (cfg) {
@@ -535,7 +611,7 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
         case 4: return launch_one<PIN, POUT, 32, 256, 1, 4, 4, 2>(st, a, cu);
         case 5: return launch_one<PIN, POUT, 128, 128, 2, 2, 4, 2>(st, a, cu);
         case 6: return launch_one<PIN, POUT, 64, 128, 2, 2, 4, 3>(st, a, cu);
-        case 7: return launch_one<PIN, POUT, 128, 64, 2, 2, 4, 3>(st, a, cu);
+        case 7: return launch_one<PIN, POUT, 128, 64, 2, 2, 4, 2>(st, a, cu);
         default: return (int)hipErrorInvalidValue;
     }
 }
@@ -564,8 +640,8 @@ bool igemm_usable(const ConvProblem& p) {
     if (src_b >= lim || dst_b >= lim || z_b >= lim || flt_b >= lim) return false;
     if ((int64_t)d.n * p.oh * p.ow >= lim) return false;
     const int64_t entries = p.pin == 32 ? (int64_t)(d.ic / 32) * d.fh * d.fw : (int64_t)(d.ic / 4) * d.fh * d.fw;
-    // table capacity incl. the padding entries of the last stage (<= 4 chunks of 8 units)
-    if (entries + 32 > IG_MAX_ENTRIES) return false;
+    // table capacity incl. the padding entries of the last stage (<= 8 chunks of 8 units)
+    if (entries + 64 > IG_MAX_ENTRIES) return false;
     return true;
 }
 
