@@ -8,8 +8,9 @@ layers and the residual z tensors are the real producer outputs.  Prints ONE JSO
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
 
 value      = images per second over the timed region (K steps, events on the launch stream)
-roofline   = algorithmic bytes of the stack / sum of per-launch kernel durations (second pass of
-             the same K steps with an event after every launch), against 8 TB/s HBM
+roofline   = algorithmic bytes per launch / average launch duration over the timed region (HIP events
+             on the launch stream around K x 53 back-to-back launches), against 8 TB/s HBM; a second
+             pass with an event after every launch gives the per-layer table
 cpu_baseline = the CPU parity checker (a port of the reference's naive ConvBias) timed on this
              host on a bounded sample (one image through the same 53 layers), scaled to images/s
 """
@@ -84,6 +85,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-extras", action="store_true", help="skip the per-config side measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches only")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also launch one plain 256 MiB streaming kernel (counter calibration for profilers)")
     ap.add_argument("--layers-out", default=None, help="write the per-layer table to this JSON file")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -110,42 +114,80 @@ def main():
     plan = build_stack(layers, 7, torch, np, util, _abi)
     for p in plan:
         p["algo"], _ = ops.conv_bias_query(p["desc"])
+    side = torch.cuda.Stream()          # default priority; every launch of the bench goes here
+    torch.cuda.set_stream(side)
     stream = torch.cuda.current_stream()
-
-    def launch(p):
-        ops.conv_bias_exec(p["desc"], p["src"], p["flt"], p["bias"], p["z"], dst=p["dst"], algo=p["algo"])
+    raw_stream = stream.cuda_stream
+    calls = [ops.conv_bias_bind(p["desc"], p["src"], p["flt"], p["bias"], p["z"], p["dst"], p["algo"]) for p in plan]
 
     def step():
-        for p in plan:
-            launch(p)
+        for c in calls:
+            c()
 
-    for _ in range(args.warmup):
+    for _ in range(max(1, args.warmup)):
         step()
     torch.cuda.synchronize()
+    want = [p["dst"].clone() for p in plan]
+
+    # ---- timed region, eager launches through the C ABI
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
     for _ in range(args.steps):
         step()
     e1.record(stream)
     torch.cuda.synchronize()
-    ms_total = e0.elapsed_time(e1)
-    ms_per_step = ms_total / args.steps
+    eager_ms = e0.elapsed_time(e1) / args.steps
+
+    # ---- the same K steps as replays of one captured HIP graph of the 53 launches (kernel nodes only)
+    graph_ms, graph_note = None, "not attempted"
+    if not args.no_graph:
+        try:
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=side):
+                step()
+            ok = True
+            for rep in range(3):            # replays separated by eager work and synchronisation
+                for p in plan:
+                    p["dst"].fill_(rep)
+                torch.cuda.synchronize()
+                g.replay()
+                torch.cuda.synchronize()
+                ok = ok and all(torch.equal(p["dst"], w) for p, w in zip(plan, want))
+            if ok:
+                for _ in range(args.warmup):
+                    g.replay()
+                torch.cuda.synchronize()
+                e0.record(stream)
+                for _ in range(args.steps):
+                    g.replay()
+                e1.record(stream)
+                torch.cuda.synchronize()
+                graph_ms = e0.elapsed_time(e1) / args.steps
+                graph_note = "replays bit-identical to eager launches (3 checked)"
+            else:
+                graph_note = "replay differed from eager launches; not used"
+        except Exception as e:  # capture is an optimisation of the launch path only
+            graph_note = "capture failed: %r" % (e,)
+    log("eager %.4f ms/step, graph %s ms/step (%s)" % (eager_ms, graph_ms, graph_note))
+    ms_per_step = graph_ms if graph_ms is not None else eager_ms
+    launch_mode = "hipGraph replay" if graph_ms is not None else "eager"
     img_s = batch * 1000.0 / ms_per_step
     tot_ops = sum(l.ops for l in layers)
     tot_bytes = sum(l.bytes for l in layers)
 
-    # ---- second pass: an event after every launch -> per-layer kernel durations
+    # ---- second pass over the same K steps: a HIP event after every launch, on the launch stream
     nl = len(plan)
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(nl + 1)] for _ in range(args.steps)]
+    timer = EventTimer(torch, raw_stream, args.steps * (nl + 1))
     torch.cuda.synchronize()
     for s in range(args.steps):
-        evs[s][0].record(stream)
-        for i, p in enumerate(plan):
-            launch(p)
-            evs[s][i + 1].record(stream)
+        timer.record()
+        for c in calls:
+            c()
+            timer.record()
     torch.cuda.synchronize()
-    per_layer_ms = [sum(evs[s][i].elapsed_time(evs[s][i + 1]) for s in range(args.steps)) / args.steps
+    per_layer_ms = [sum(timer.elapsed(s * (nl + 1) + i, s * (nl + 1) + i + 1) for s in range(args.steps)) / args.steps
                     for i in range(nl)]
+    assert all(torch.equal(p["dst"], w) for p, w in zip(plan, want)), "outputs changed between passes"
     kern_ms = sum(per_layer_ms)
     table = []
     for p, ms in zip(plan, per_layer_ms):
@@ -156,15 +198,19 @@ def main():
                           algo=lib.algo_names()[p["algo"].id], tile=lib.tile_names()[p["algo"].tile_cfg],
                           us=round(ms * 1e3, 2), tops=round(l.ops / t / 1e12, 1), gbs=round(l.bytes / t / 1e9, 1),
                           frac_roof=round(roof / t, 3)))
-    roofline = dict(bound="hbm", achieved=round(tot_bytes / (kern_ms * 1e-3) / 1e9, 1), peak=HBM_PEAK / 1e9,
-                    unit="GB/s", frac=round(tot_bytes / (kern_ms * 1e-3) / HBM_PEAK, 4), traffic=None,
+    # dominant kernel = the implicit-GEMM kernel (all 53 launches).  Average launch duration = the
+    # timed region of K steps (two HIP events on the launch stream) / (K * 53): the launches run
+    # back to back, so this is the kernel duration plus the sub-microsecond gap between launches.
+    t_launch = ms_per_step * 1e-3 / nl
+    roofline = dict(bound="hbm", achieved=round(tot_bytes / nl / t_launch / 1e9, 1), peak=HBM_PEAK / 1e9,
+                    unit="GB/s", frac=round(tot_bytes / nl / t_launch / HBM_PEAK, 4), traffic=None,
                     kernel="igemm_kernel (MI355_IGEMM_MFMA_I8), 53 launches per step",
-                    bytes_per_launch=round(tot_bytes / nl), avg_launch_us=round(kern_ms * 1e3 / nl, 2),
-                    kernel_ms_per_step=round(kern_ms, 4),
-                    mfma_tops=round(tot_ops / (kern_ms * 1e-3) / 1e12, 1),
-                    mfma_frac_of_int8_peak=round(tot_ops / (kern_ms * 1e-3) / INT8_PEAK_OPS, 4),
+                    bytes_per_launch=round(tot_bytes / nl), avg_launch_us=round(t_launch * 1e6, 2),
+                    per_launch_event_sum_ms=round(kern_ms, 4),
+                    mfma_tops=round(tot_ops / (ms_per_step * 1e-3) / 1e12, 1),
+                    mfma_frac_of_int8_peak=round(tot_ops / (ms_per_step * 1e-3) / INT8_PEAK_OPS, 4),
                     frac_of_binding_roof=round(sum(max(l.ops / INT8_PEAK_OPS, l.bytes / HBM_PEAK) for l in layers)
-                                               / (kern_ms * 1e-3), 4))
+                                               / (ms_per_step * 1e-3), 4))
     tr = os.path.join(ROOT, "profiles", "traffic_resnet50_stack.json")
     if os.path.exists(tr):
         try:
@@ -178,10 +224,19 @@ def main():
                data="synthetic",
                config=dict(workload="BASELINE configs[2]: ResNet-50 v1.5 int8 conv stack, batch 64, 224x224, "
                                     "NCHW4 stem + NCHW32, fused residual z + RELU, random per-tensor scales",
-                           batch=batch, layers=nl),
+                           batch=batch, layers=nl, launch=launch_mode, graph=graph_note),
+               eager_ms_per_step=round(eager_ms, 4),
                tops=round(tot_ops / (ms_per_step * 1e-3) / 1e12, 1),
                pct_int8_peak=round(100 * tot_ops / (ms_per_step * 1e-3) / INT8_PEAK_OPS, 2),
                roofline=roofline)
+
+    if args.calib_copy:
+        a = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device="cuda")
+        b = torch.empty_like(a)
+        torch.cuda.synchronize()
+        torch.bitwise_not(a, out=b)     # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del a, b
 
     extras = {}
     if not args.no_extras:
@@ -201,6 +256,43 @@ def main():
         for row in table:
             log(row)
     print(json.dumps(out), flush=True)
+
+
+class EventTimer:
+    """HIP events recorded straight on a raw stream (cheaper than torch's wrappers, so the host
+    stays ahead of the GPU and an interval between two events is the kernel between them)."""
+
+    def __init__(self, torch, raw_stream, n):
+        import ctypes as C
+        self.C = C
+        self.torch = torch
+        self.stream = C.c_void_p(raw_stream)
+        self.n = 0
+        try:
+            self.hip = C.CDLL("libamdhip64.so")
+            self.ev = (C.c_void_p * n)()
+            for i in range(n):
+                if self.hip.hipEventCreate(C.byref(self.ev, i * C.sizeof(C.c_void_p))):
+                    raise OSError("hipEventCreate failed")
+        except OSError:
+            self.hip = None
+            self.ev = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+    def record(self):
+        if self.hip is not None:
+            if self.hip.hipEventRecord(self.C.c_void_p(self.ev[self.n]), self.stream):
+                raise RuntimeError("hipEventRecord failed")
+        else:
+            self.ev[self.n].record(self.torch.cuda.current_stream())
+        self.n += 1
+
+    def elapsed(self, i, j):
+        if self.hip is None:
+            return self.ev[i].elapsed_time(self.ev[j])
+        ms = self.C.c_float()
+        if self.hip.hipEventElapsedTime(self.C.byref(ms), self.C.c_void_p(self.ev[i]), self.C.c_void_p(self.ev[j])):
+            raise RuntimeError("hipEventElapsedTime failed")
+        return ms.value
 
 
 def time_launches(torch, fn, iters=20, warm=3):
@@ -282,32 +374,38 @@ def run_extras(torch, np, util, _abi, lib, ops, workloads):
 
 
 def cpu_baseline(np, util, _abi, workloads):
-    """The CPU parity checker (port of the reference's naive ConvBias) on one image through the
-    same 53 layers, all host threads the process may use, scaled to images per second."""
+    """The CPU parity checker (a port of the reference's naive ConvBias, OpenMP over output rows)
+    on a bounded sample of the same workload: the same 53 layers at a batch chosen so that the
+    whole leg is 10-30 s of CPU work on this host, scaled to images per second."""
     from oracle import oracle
     oracle.lib()
-    layers = workloads.resnet50(1)
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     os.environ["OMP_NUM_THREADS"] = str(cores)
-    t_tot, macs = 0.0, 0
-    budget = 25.0
-    done = 0
-    for i, l in enumerate(layers):
-        d = l.desc(2e-4, 0.05, 0.05)
-        src, flt, bias, z = util.make_tensors(d, seed=i + 1, flt_range=(-127, 127))
-        t0 = time.perf_counter()
-        oracle.conv_bias(d, src, flt, bias, z)
-        t_tot += time.perf_counter() - t0
-        macs += l.ops // 2
-        done += 1
-        if t_tot > budget:
-            break
-    total_macs = sum(l.ops // 2 for l in layers)
-    img_s = (macs / total_macs) / t_tot if t_tot > 0 else 0.0
-    return dict(value=round(img_s, 4), unit="img/s", cores=cores, kind="port",
-                sample="batch 1 through the first %d of 53 layers (%.2f of %.2f GMAC), %.1f s, scaled by MACs"
-                       % (done, macs / 1e9, total_macs / 1e9, t_tot))
+
+    def run(batch, budget):
+        t_tot, macs, done = 0.0, 0, 0
+        layers = workloads.resnet50(batch)
+        for i, l in enumerate(layers):
+            d = l.desc(2e-4, 0.05, 0.05)
+            src, flt, bias, z = util.make_tensors(d, seed=i + 1, flt_range=(-127, 127))
+            t0 = time.perf_counter()
+            oracle.conv_bias(d, src, flt, bias, z)
+            t_tot += time.perf_counter() - t0
+            macs += l.ops // 2
+            done += 1
+            if t_tot > budget:
+                break
+        return t_tot, macs, done, sum(l.ops // 2 for l in layers)
+
+    t1, m1, _, tm1 = run(1, 10.0)                 # probe: one image
+    est = t1 * tm1 / max(m1, 1)
+    batch = int(max(1, min(64, round(15.0 / max(est, 1e-3)))))
+    t_tot, macs, done, total_macs = run(batch, 30.0)
+    img_s = batch * (macs / total_macs) / t_tot if t_tot > 0 else 0.0
+    return dict(value=round(img_s, 3), unit="img/s", cores=cores, kind="port",
+                sample="batch %d through the first %d of 53 layers (%.1f of %.1f GMAC) in %.1f s on %d threads, "
+                       "scaled by MACs" % (batch, done, macs / 1e9, total_macs / 1e9, t_tot, cores))
 
 
 if __name__ == "__main__":

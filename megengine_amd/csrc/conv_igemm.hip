@@ -456,7 +456,8 @@ struct IgemmKernel {
 
         for (int it = 0; it < total; it += 2) {
             phase(it, 0, R0, R1);
-            phase(it + 1, 1, R1, R0);  // when it + 1 == total this is a dead phase on zero-filled LDS
+            if (it + 1 >= total) break;  // leaving the loop here keeps the loads inside both phases unconditional
+            phase(it + 1, 1, R1, R0);
         }
     }
 
@@ -652,10 +653,13 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
     if (cu_count <= 0) cu_count = 256;
     auto tiles = [&](int cfg) { return ((OC + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm) * ((M + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn); };
     const int kbytes = d.ic * d.fh * d.fw;
-    const bool long_k = kbytes >= 256;
     if (OC <= 32) return 4;
     if (OC <= 64) return tiles(1) >= cu_count ? 1 : 3;
-    if (tiles(0) >= 2 * cu_count) return long_k ? 5 : 0;
+    // 128x128 tiles as soon as they give every CU 1.5 tiles; the deeper k stage pays once the
+    // reduction is long enough to amortise its larger prologue
+    if (tiles(0) >= 2 * cu_count) return kbytes >= 512 ? 5 : 0;
+    if (2 * tiles(0) >= 3 * cu_count) return kbytes >= 1024 ? 5 : 0;
+    if (OC >= 256 && tiles(7) >= cu_count) return 7;
     if (tiles(6) >= cu_count) return 6;
     return 3;
 }

@@ -72,6 +72,25 @@ def conv_bias_exec(desc, src, flt, bias=None, z=None, dst=None, algo=None, works
     return dst
 
 
+def conv_bias_bind(desc, src, flt, bias, z, dst, algo, workspace=None, stream=None):
+    """Pre-marshals one exec call; the returned callable launches it on the CURRENT torch stream
+    when `stream` is None, else on that raw stream handle, and raises on a non-zero status.
+    Keeps the tensors alive.  For callers that replay the same launch many times."""
+    fn = lib().mi355_convbias_s8_exec
+    wsn = workspace.numel() if workspace is not None else 0
+    tail = (C.byref(desc), C.byref(algo), _ptr(src), _ptr(flt), _ptr(bias), _ptr(z), _ptr(dst), _ptr(workspace), wsn)
+    keep = (desc, algo, src, flt, bias, z, dst, workspace)
+    fixed = None if stream is None else C.c_void_p(stream)
+
+    def call(_keep=keep):
+        st = fixed if fixed is not None else C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = fn(st, *tail)
+        if rc:
+            check(rc)
+
+    return call
+
+
 def relayout_desc(mode, shape, group=1, oc=0, elem_bytes=1, scale_src=1.0, scale_dst=1.0):
     d = _abi.RelayoutDesc(mode=mode, ndim=len(shape), group=group, oc=oc, elem_bytes=elem_bytes,
                           scale_src=scale_src, scale_dst=scale_dst)
