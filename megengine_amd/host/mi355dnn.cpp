@@ -1,0 +1,382 @@
+// Implementation of the host-side operator classes over the C ABI.  Shape and dtype rules
+// follow the reference's common layer; each block cites the rule it restates.
+#include "mi355dnn.h"
+
+#include <math.h>
+#include <stdio.h>
+
+#include "../../include/mi355_convbias.h"
+
+namespace mi355dnn {
+
+namespace {
+
+[[noreturn]] void fail(int status, const std::string& msg) {
+    throw Error(status, std::string(mi355_status_string(status)) + ": " + msg);
+}
+
+void check_abi(int status) {
+    if (status != MI355_OK) {
+        const char* m = mi355_last_error();
+        throw Error(status, std::string(mi355_status_string(status)) + ": " + (m ? m : ""));
+    }
+}
+
+#define HOST_ASSERT(cond, status, ...)                       \
+    do {                                                     \
+        if (!(cond)) {                                       \
+            char buf_[512];                                  \
+            snprintf(buf_, sizeof(buf_), __VA_ARGS__);       \
+            fail(status, std::string(buf_) + " (" #cond ")"); \
+        }                                                    \
+    } while (0)
+
+using Format = param::ConvBias::Format;
+
+bool format_supported(Format f) {
+    switch (f) {
+        case Format::NCHW: case Format::NCHW4: case Format::NCHW32: case Format::NCHW44:
+        case Format::NCHW4_NCHW32: case Format::NCHW32_NCHW4:
+            return true;
+        default:
+            return false;
+    }
+}
+size_t in_pack(Format f) {
+    switch (f) {
+        case Format::NCHW: return 1;
+        case Format::NCHW32: case Format::NCHW32_NCHW4: return 32;
+        default: return 4;
+    }
+}
+size_t out_pack(Format f) {
+    switch (f) {
+        case Format::NCHW: return 1;
+        case Format::NCHW32: case Format::NCHW4_NCHW32: return 32;
+        default: return 4;
+    }
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------- shapes / layouts
+TensorShape::TensorShape(std::initializer_list<size_t> s) {
+    if (s.size() > MAX_NDIM) fail(MI355_ERR_BAD_ARG, "too many dimensions");
+    ndim = 0;
+    for (size_t v : s) shape[ndim++] = v;
+}
+size_t TensorShape::total_nr_elems() const {
+    if (!ndim) return 0;
+    size_t r = 1;
+    for (size_t i = 0; i < ndim; ++i) r *= shape[i];
+    return r;
+}
+bool TensorShape::eq_shape(const TensorShape& o) const {
+    if (ndim != o.ndim) return false;
+    for (size_t i = 0; i < ndim; ++i)
+        if (shape[i] != o.shape[i]) return false;
+    return true;
+}
+std::string TensorShape::to_string() const {
+    std::string s = "{";
+    for (size_t i = 0; i < ndim; ++i) s += (i ? "," : "") + std::to_string(shape[i]);
+    return s + "}";
+}
+TensorLayout::TensorLayout(const TensorShape& sh, DType dt) : TensorShape(sh), dtype(dt) { init_contiguous_stride(); }
+void TensorLayout::init_contiguous_stride() {
+    ptrdiff_t s = 1;
+    for (size_t i = ndim; i-- > 0;) {
+        stride[i] = s;
+        s *= (ptrdiff_t)shape[i];
+    }
+}
+bool TensorLayout::is_contiguous() const {
+    ptrdiff_t s = 1;
+    for (size_t i = ndim; i-- > 0;) {
+        if (shape[i] != 1 && stride[i] != s) return false;
+        s *= (ptrdiff_t)shape[i];
+    }
+    return true;
+}
+bool TensorLayout::is_batch_strided() const {
+    ptrdiff_t s = 1;
+    for (size_t i = ndim; i-- > 1;) {
+        if (shape[i] != 1 && stride[i] != s) return false;
+        s *= (ptrdiff_t)shape[i];
+    }
+    return ndim == 0 || shape[0] == 1 || stride[0] >= s;
+}
+size_t TensorLayout::span_bytes() const {
+    if (!ndim) return 0;
+    size_t last = 0;
+    for (size_t i = 0; i < ndim; ++i) last += (shape[i] - 1) * (size_t)stride[i];
+    return (last + 1) * dtype.size();
+}
+
+// ---------------------------------------------------------------- handle
+std::unique_ptr<Handle> Handle::make(void* stream, int device) {
+    return std::unique_ptr<Handle>(new Handle(stream, device));
+}
+int Handle::abi_version() { return mi355_abi_version(); }
+void Handle::check_device() const {
+    mi355_device_info info;
+    check_abi(mi355_get_device_info(m_device, &info));
+}
+
+// ---------------------------------------------------------------- ConvBias
+struct ConvBiasForward::Canon {
+    mi355_conv_desc d;
+    TensorShape dst_shape;
+};
+
+ConvBiasForward::BiasMode ConvBiasForward::bias_mode_of(const TensorLayout& bias, const TensorLayout& dst) {
+    if (bias.ndim == 0) return BiasMode::NO_BIAS;
+    if (bias.eq_shape(dst)) return BiasMode::BIAS;
+    return BiasMode::BROADCAST_CHANNEL_BIAS;
+}
+
+void ConvBiasForward::deduce_dtype(DType src, DType filter, DType, DType, DType& dst) const {
+    // dnn/src/common/convolution.cpp:545-631: s8 x s8 gives QuantizedS32(s_src * s_flt) by default and
+    // accepts a caller-named QuantizedS8 of any scale
+    HOST_ASSERT(src.enumv == DTypeEnum::QuantizedS8 && filter.enumv == DTypeEnum::QuantizedS8, MI355_ERR_UNSUPPORTED,
+                "this backend implements QuantizedS8 x QuantizedS8 ConvBias only");
+    if (dst.enumv == DTypeEnum::QuantizedS8) return;
+    dst = dtype::QuantizedS32(src.scale * filter.scale);
+}
+
+void ConvBiasForward::canonize(const TensorLayout& src, const TensorLayout& filter, const TensorLayout& bias,
+                               const TensorLayout& z, const TensorLayout& dst, Canon& out, bool need_dst) const {
+    const Param& p = m_param;
+    HOST_ASSERT(format_supported(p.format), MI355_ERR_UNSUPPORTED, "format %u is not implemented", (unsigned)p.format);
+    HOST_ASSERT(p.nonlineMode != Param::NonlineMode::SIGMOID, MI355_ERR_UNSUPPORTED,
+                "SIGMOID is not defined for quantized ConvBias");  // naive/conv_bias/opr_impl.cpp:79-88
+    HOST_ASSERT(src.dtype.enumv == DTypeEnum::QuantizedS8 && filter.dtype.enumv == DTypeEnum::QuantizedS8,
+                MI355_ERR_UNSUPPORTED, "src and filter must be QuantizedS8");
+    const size_t pi = in_pack(p.format), po = out_pack(p.format);
+    const bool packed = p.format != Format::NCHW;
+    HOST_ASSERT(src.ndim == (packed ? 5u : 4u), MI355_ERR_SHAPE, "src %s has the wrong rank for the format",
+                src.to_string().c_str());
+    if (packed) HOST_ASSERT(src[4] == pi, MI355_ERR_SHAPE, "src %s: innermost axis must be %zu", src.to_string().c_str(), pi);
+    HOST_ASSERT(src.is_batch_strided() && filter.is_contiguous(), MI355_ERR_UNSUPPORTED,
+                "src must be contiguous within an image and filter contiguous");
+
+    mi355_conv_desc& d = out.d;
+    d = mi355_conv_desc();
+    d.format = (uint32_t)p.format;
+    d.sparse = (uint32_t)p.sparse;
+    d.nonline = (uint32_t)p.nonlineMode;
+    d.mode = (uint32_t)p.mode;
+    d.pad_h = p.pad_h; d.pad_w = p.pad_w; d.stride_h = p.stride_h; d.stride_w = p.stride_w;
+    d.dilate_h = p.dilate_h; d.dilate_w = p.dilate_w;
+    d.n = (uint32_t)src[0];
+    d.ic = (uint32_t)(src[1] * pi);
+    d.ih = (uint32_t)src[2];
+    d.iw = (uint32_t)src[3];
+
+    // filter meta: dnn/src/common/convolution.cpp:33-94 (NCHW), :357-418 (NCHW4/NCHW32), :241-310 (NCHW44)
+    const bool grp = p.sparse == Param::Sparse::GROUP;
+    size_t g = 1, ocpg, icpg, fh, fw;
+    if (p.format == Format::NCHW) {
+        HOST_ASSERT(filter.ndim == (grp ? 5u : 4u), MI355_ERR_SHAPE, "filter %s: bad rank", filter.to_string().c_str());
+        const size_t o = grp ? 1 : 0;
+        if (grp) g = filter[0];
+        ocpg = filter[o]; icpg = filter[o + 1]; fh = filter[o + 2]; fw = filter[o + 3];
+    } else if (p.format == Format::NCHW44) {
+        if (grp && filter.ndim == 6) {  // channel-wise: (G/4, 1, 1, FH, FW, 4)
+            HOST_ASSERT(filter[1] == 1 && filter[2] == 1 && filter[5] == 4, MI355_ERR_SHAPE,
+                        "filter %s is not a channel-wise NCHW44 filter", filter.to_string().c_str());
+            g = filter[0] * 4; ocpg = icpg = 1; fh = filter[3]; fw = filter[4];
+        } else {
+            HOST_ASSERT(filter.ndim == (grp ? 7u : 6u), MI355_ERR_SHAPE, "filter %s: bad rank", filter.to_string().c_str());
+            const size_t o = grp ? 1 : 0;
+            if (grp) g = filter[0];
+            HOST_ASSERT(filter[o + 4] == 4 && filter[o + 5] == 4, MI355_ERR_SHAPE, "filter %s: inner axes must be 4,4",
+                        filter.to_string().c_str());
+            ocpg = filter[o] * 4; icpg = filter[o + 1] * 4; fh = filter[o + 2]; fw = filter[o + 3];
+        }
+    } else {
+        HOST_ASSERT(filter.ndim == (grp ? 6u : 5u), MI355_ERR_SHAPE, "filter %s: bad rank", filter.to_string().c_str());
+        const size_t o = grp ? 1 : 0;
+        if (grp) g = filter[0];
+        HOST_ASSERT(filter[o + 4] == pi, MI355_ERR_SHAPE, "filter %s: innermost axis must be %zu",
+                    filter.to_string().c_str(), pi);
+        ocpg = filter[o]; icpg = filter[o + 1] * pi; fh = filter[o + 2]; fw = filter[o + 3];
+        HOST_ASSERT(p.dilate_h == 1 && p.dilate_w == 1, MI355_ERR_UNSUPPORTED,
+                    "dilation must be 1 for channel-packed formats");  // convolution.cpp:411-414
+    }
+    HOST_ASSERT(icpg * g == d.ic, MI355_ERR_SHAPE, "group %zu x icpg %zu does not match %u input channels", g, icpg, d.ic);
+    d.group = (uint32_t)g;
+    d.oc = (uint32_t)(ocpg * g);
+    d.fh = (uint32_t)fh;
+    d.fw = (uint32_t)fw;
+    HOST_ASSERT(d.oc % po == 0, MI355_ERR_SHAPE, "%u output channels are not a multiple of %zu", d.oc, po);
+
+    uint32_t oh = 0, ow = 0;
+    check_abi(mi355_convbias_deduce_out(&d, &oh, &ow));
+    out.dst_shape = packed ? TensorShape{d.n, d.oc / po, oh, ow, po} : TensorShape{d.n, d.oc, oh, ow};
+
+    // dtypes and the bias / z rules of dnn/src/common/conv_bias.cpp:8-133
+    const float s_acc = src.dtype.scale * filter.dtype.scale;
+    d.scale_bias = s_acc;
+    if (bias.dtype.enumv == DTypeEnum::QuantizedS32) {
+        HOST_ASSERT(fabsf(s_acc - bias.dtype.scale) < 1e-6f, MI355_ERR_BAD_ARG,
+                    "bias scale %g differs from src scale * filter scale = %g", bias.dtype.scale, s_acc);
+        d.scale_bias = bias.dtype.scale;
+    } else {
+        HOST_ASSERT(bias.ndim == 0, MI355_ERR_BAD_ARG, "bias must be QuantizedS32");
+    }
+    if (!need_dst) return;
+
+    HOST_ASSERT(dst.eq_shape(out.dst_shape), MI355_ERR_SHAPE, "dst %s, expected %s", dst.to_string().c_str(),
+                out.dst_shape.to_string().c_str());
+    HOST_ASSERT(dst.dtype.enumv == DTypeEnum::QuantizedS8 || dst.dtype.enumv == DTypeEnum::QuantizedS32,
+                MI355_ERR_UNSUPPORTED, "dst must be QuantizedS8 or QuantizedS32");
+    HOST_ASSERT(dst.is_batch_strided(), MI355_ERR_UNSUPPORTED, "dst must be contiguous within an image");
+    d.dst_dtype = dst.dtype.enumv == DTypeEnum::QuantizedS8 ? MI355_DT_QS8 : MI355_DT_QS32;
+    d.scale_dst = dst.dtype.scale;
+    switch (bias_mode_of(bias, dst)) {
+        case BiasMode::NO_BIAS: d.bias_mode = MI355_BIAS_NONE; break;
+        case BiasMode::BIAS: d.bias_mode = MI355_BIAS_FULL; break;
+        default: {
+            TensorShape want = packed ? TensorShape{1, d.oc / po, 1, 1, po} : TensorShape{1, d.oc, 1, 1};
+            HOST_ASSERT(bias.eq_shape(want), MI355_ERR_SHAPE, "bias %s, expected %s or the dst shape",
+                        bias.to_string().c_str(), want.to_string().c_str());
+            d.bias_mode = MI355_BIAS_BROADCAST_CHANNEL;
+        }
+    }
+    if (bias.ndim) HOST_ASSERT(bias.is_contiguous(), MI355_ERR_UNSUPPORTED, "bias must be contiguous");
+    d.has_z = z.ndim != 0;
+    d.scale_z = 1.f;
+    if (d.has_z) {
+        HOST_ASSERT(z.dtype.enumv == dst.dtype.enumv, MI355_ERR_BAD_ARG, "z and dst must have the same dtype kind");
+        HOST_ASSERT(z.eq_shape(dst), MI355_ERR_SHAPE, "z %s must have the dst shape %s", z.to_string().c_str(),
+                    dst.to_string().c_str());
+        HOST_ASSERT(z.is_batch_strided(), MI355_ERR_UNSUPPORTED, "z must be contiguous within an image");
+        d.scale_z = z.dtype.scale;
+        d.z_stride_n = z.stride[0];
+    }
+    d.src_stride_n = src.is_contiguous() ? 0 : src.stride[0];
+    d.dst_stride_n = dst.is_contiguous() ? 0 : dst.stride[0];
+    if (d.has_z && z.is_contiguous()) d.z_stride_n = 0;
+}
+
+void ConvBiasForward::deduce_layout(const TensorLayout& src, const TensorLayout& filter, const TensorLayout& bias,
+                                    const TensorLayout& z, TensorLayout& dst) const {
+    Canon c;
+    canonize(src, filter, bias, z, dst, c, false);
+    DType dt = dst.dtype;
+    deduce_dtype(src.dtype, filter.dtype, bias.dtype, z.dtype, dt);
+    dst = TensorLayout(c.dst_shape, dt);
+}
+
+static mi355_algo resolve_algo(const mi355_conv_desc& d, const ExecutionPolicy& pol, size_t* ws) {
+    mi355_algo a;
+    check_abi(mi355_convbias_s8_query(&d, pol.valid() ? pol.algo.id : MI355_ALGO_HEURISTIC, &a, ws));
+    if (pol.valid() && pol.algo.tile_cfg >= 0) {
+        if (pol.algo.tile_cfg >= mi355_igemm_tile_count()) fail(MI355_ERR_ALGO, "unknown tile configuration");
+        a.tile_cfg = pol.algo.tile_cfg;
+    }
+    return a;
+}
+
+size_t ConvBiasForward::get_workspace_in_bytes(const TensorLayout& src, const TensorLayout& filter,
+                                               const TensorLayout& bias, const TensorLayout& z,
+                                               const TensorLayout& dst, const PreprocessedFilter*) const {
+    Canon c;
+    canonize(src, filter, bias, z, dst, c, true);
+    size_t ws = 0;
+    resolve_algo(c.d, m_policy, &ws);
+    return ws;
+}
+
+void ConvBiasForward::exec(const TensorND& src, const TensorND& filter, const TensorND& bias, const TensorND& z,
+                           const TensorND& dst, const PreprocessedFilter*, const Workspace& workspace) {
+    Canon c;
+    canonize(src.layout, filter.layout, bias.layout, z.layout, dst.layout, c, true);
+    size_t ws = 0;
+    mi355_algo a = resolve_algo(c.d, m_policy, &ws);
+    HOST_ASSERT(workspace.size >= ws, MI355_ERR_WORKSPACE, "workspace of %zu bytes, %zu needed", workspace.size, ws);
+    HOST_ASSERT(src.raw_ptr && filter.raw_ptr && dst.raw_ptr, MI355_ERR_BAD_ARG, "null tensor pointer");
+    check_abi(mi355_convbias_s8_exec(m_handle->stream(), &c.d, &a, (const int8_t*)src.raw_ptr,
+                                     (const int8_t*)filter.raw_ptr,
+                                     bias.layout.ndim ? (const int32_t*)bias.raw_ptr : nullptr,
+                                     z.layout.ndim ? (const int8_t*)z.raw_ptr : nullptr, dst.raw_ptr,
+                                     workspace.raw_ptr, workspace.size));
+}
+
+std::vector<AlgorithmInfo> ConvBiasForward::get_all_algorithms_info(const TensorLayout& src, const TensorLayout& filter,
+                                                                    const TensorLayout& bias, const TensorLayout& z,
+                                                                    const TensorLayout& dst) const {
+    Canon c;
+    canonize(src, filter, bias, z, dst, c, true);
+    std::vector<AlgorithmInfo> r;
+    for (int id = 0; id < mi355_convbias_algo_count(); ++id) {
+        if (mi355_convbias_algo_usable(&c.d, id) != MI355_OK) continue;
+        const std::string base = mi355_convbias_algo_name(id);
+        r.push_back(AlgorithmInfo{AlgorithmDesc{id, -1}, base, true});
+        if (base.find("IGEMM") != std::string::npos)
+            for (int t = 0; t < mi355_igemm_tile_count(); ++t)
+                r.push_back(AlgorithmInfo{AlgorithmDesc{id, t}, base + ":" + mi355_igemm_tile_name(t), true});
+    }
+    return r;
+}
+
+AlgorithmInfo ConvBiasForward::get_algorithm_info_heuristic(const TensorLayout& src, const TensorLayout& filter,
+                                                            const TensorLayout& bias, const TensorLayout& z,
+                                                            const TensorLayout& dst, size_t workspace_limit) const {
+    Canon c;
+    canonize(src, filter, bias, z, dst, c, true);
+    size_t ws = 0;
+    mi355_algo a;
+    check_abi(mi355_convbias_s8_query(&c.d, MI355_ALGO_HEURISTIC, &a, &ws));
+    HOST_ASSERT(ws <= workspace_limit, MI355_ERR_WORKSPACE, "no algorithm within the workspace limit of %zu bytes",
+                workspace_limit);
+    std::string name = mi355_convbias_algo_name(a.id);
+    if (name.find("IGEMM") != std::string::npos && a.tile_cfg >= 0) name += std::string(":") + mi355_igemm_tile_name(a.tile_cfg);
+    return AlgorithmInfo{AlgorithmDesc{a.id, a.tile_cfg}, name, true};
+}
+
+// ---------------------------------------------------------------- RelayoutFormat
+static mi355_relayout_desc relayout_desc(const param::RelayoutFormat& p, const TensorLayout& src, const DType& dst_dt) {
+    mi355_relayout_desc d = mi355_relayout_desc();
+    d.mode = (uint32_t)p.mode;
+    d.ndim = (uint32_t)src.ndim;
+    for (size_t i = 0; i < src.ndim; ++i) d.shape[i] = (uint32_t)src[i];
+    d.group = p.group ? p.group : 1;
+    d.oc = p.oc;
+    d.elem_bytes = (uint32_t)src.dtype.size();
+    d.scale_src = src.dtype.enumv == DTypeEnum::QuantizedS8 ? src.dtype.scale : 1.f;
+    d.scale_dst = dst_dt.enumv == DTypeEnum::QuantizedS8 ? dst_dt.scale : d.scale_src;
+    return d;
+}
+
+void RelayoutFormat::deduce_layout(const TensorLayout& src, TensorLayout& dst) const {
+    mi355_relayout_desc d = relayout_desc(m_param, src, src.dtype);
+    uint32_t nd = 0, sh[7];
+    check_abi(mi355_relayout_deduce(&d, &nd, sh));
+    TensorShape s;
+    s.ndim = nd;
+    for (uint32_t i = 0; i < nd; ++i) s.shape[i] = sh[i];
+    // an unset dst dtype inherits the src dtype (relayout_format.cpp deduce_layout)
+    DType dt = (dst.ndim == 0 && dst.dtype == DType()) ? src.dtype : dst.dtype;
+    if (dt.size() != src.dtype.size()) dt = src.dtype;
+    dst = TensorLayout(s, dt);
+}
+
+void RelayoutFormat::exec(const TensorND& src, const TensorND& dst, const Workspace&) {
+    HOST_ASSERT(src.layout.is_contiguous() && dst.layout.is_contiguous(), MI355_ERR_UNSUPPORTED,
+                "relayout takes contiguous tensors");
+    HOST_ASSERT(src.layout.dtype.size() == dst.layout.dtype.size(), MI355_ERR_BAD_ARG, "element sizes differ");
+    mi355_relayout_desc d = relayout_desc(m_param, src.layout, dst.layout.dtype);
+    uint32_t nd = 0, sh[7];
+    check_abi(mi355_relayout_deduce(&d, &nd, sh));
+    TensorShape want;
+    want.ndim = nd;
+    for (uint32_t i = 0; i < nd; ++i) want.shape[i] = sh[i];
+    HOST_ASSERT(dst.layout.eq_shape(want), MI355_ERR_SHAPE, "dst %s, expected %s", dst.layout.to_string().c_str(),
+                want.to_string().c_str());
+    HOST_ASSERT(src.raw_ptr && dst.raw_ptr, MI355_ERR_BAD_ARG, "null tensor pointer");
+    check_abi(mi355_relayout_exec(m_handle->stream(), &d, src.raw_ptr, dst.raw_ptr));
+}
+
+}  // namespace mi355dnn

@@ -1,0 +1,363 @@
+// Test driver for the host-side C++ operator classes (megengine_amd/host), in the manner of the
+// reference's Checker<ConvBias> (dnn/test/common/checker.h, dnn/test/common/conv_bias.cpp): build
+// layouts, let the operator deduce dst, run exec on the device, compare every element with the CPU
+// parity checker fed from an independently written descriptor.
+//
+//   host_checker --cpu     layout deduction, validation errors, algorithm listing (no device needed)
+//   host_checker --gpu     the above + exec cases on device 0
+//
+// Prints one line per case and "ALL OK" at the end; exit status 0 only when everything passed.
+#include <hip/hip_runtime_api.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <functional>
+#include <string>
+#include <vector>
+
+#include "../../include/mi355_convbias.h"
+#include "../../megengine_amd/host/mi355dnn.h"
+
+extern "C" {
+int oracle_convbias_s8(const mi355_conv_desc* d, const int8_t* src, const int8_t* flt, const int32_t* bias,
+                       const void* z, void* dst);
+int oracle_relayout_deduce(const mi355_relayout_desc* d, uint32_t* ndim, uint32_t shape[7]);
+int oracle_relayout(const mi355_relayout_desc* d, const void* src, void* dst);
+}
+
+using namespace mi355dnn;
+using CB = param::ConvBias;
+
+static int g_fail = 0;
+#define EXPECT(cond, ...)                        \
+    do {                                         \
+        if (!(cond)) {                           \
+            printf("  FAIL %s:%d: ", __FILE__, __LINE__); \
+            printf(__VA_ARGS__);                 \
+            printf("\n");                        \
+            ++g_fail;                            \
+        }                                        \
+    } while (0)
+
+static uint64_t splitmix(uint64_t& s) {
+    uint64_t z = (s += 0x9E3779B97F4A7C15ull);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+static void fill_s8(std::vector<int8_t>& v, uint64_t seed, int lo, int hi) {
+    for (auto& x : v) x = (int8_t)(lo + (int)(splitmix(seed) % (uint64_t)(hi - lo + 1)));
+}
+static void fill_s32(std::vector<int32_t>& v, uint64_t seed, int lo, int hi) {
+    for (auto& x : v) x = lo + (int)(splitmix(seed) % (uint64_t)(hi - lo + 1));
+}
+
+#define HIP_OK(x)                                                        \
+    do {                                                                 \
+        hipError_t e_ = (x);                                             \
+        if (e_ != hipSuccess) {                                          \
+            printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+            exit(3);                                                     \
+        }                                                                \
+    } while (0)
+
+struct DevBuf {
+    void* p = nullptr;
+    explicit DevBuf(size_t bytes) { HIP_OK(hipMalloc(&p, bytes ? bytes : 16)); }
+    ~DevBuf() { (void)hipFree(p); }
+};
+
+static bool throws(const std::function<void()>& f, int status) {
+    try {
+        f();
+    } catch (const Error& e) {
+        if (e.status() != status) printf("  (threw status %d: %s)\n", e.status(), e.what());
+        return e.status() == status;
+    }
+    return false;
+}
+
+// ------------------------------------------------------------------ a ConvBias case
+struct Case {
+    const char* name;
+    CB::Format fmt;
+    CB::Sparse sparse;
+    CB::NonlineMode nl;
+    TensorShape src, flt;
+    uint32_t pad, stride;
+    bool has_bias, has_z;
+    bool dst_s32;
+    // the descriptor the CPU checker is given, written by hand for each case
+    uint32_t n, ic, ih, iw, oc, fh, fw, group;
+};
+
+static std::vector<Case> cases() {
+    using F = CB::Format;
+    using S = CB::Sparse;
+    using N = CB::NonlineMode;
+    return {
+        {"nchw4 dense 3x3 relu", F::NCHW4, S::DENSE, N::RELU, {2, 4, 9, 11, 4}, {24, 4, 3, 3, 4}, 1, 1, true, false, false,
+         2, 16, 9, 11, 24, 3, 3, 1},
+        {"nchw4 dense 1x1 z identity", F::NCHW4, S::DENSE, N::IDENTITY, {3, 8, 7, 7, 4}, {32, 8, 1, 1, 4}, 0, 1, true, true,
+         false, 3, 32, 7, 7, 32, 1, 1, 1},
+        {"nchw4 group 2", F::NCHW4, S::GROUP, N::RELU, {2, 4, 8, 8, 4}, {2, 8, 2, 3, 3, 4}, 1, 2, true, false, false,
+         2, 16, 8, 8, 16, 3, 3, 2},
+        {"nchw32 dense 3x3 hswish z", F::NCHW32, S::DENSE, N::H_SWISH, {2, 2, 10, 10, 32}, {64, 2, 3, 3, 32}, 1, 1, true,
+         true, false, 2, 64, 10, 10, 64, 3, 3, 1},
+        {"nchw32 1x1 s2 no bias", F::NCHW32, S::DENSE, N::IDENTITY, {2, 4, 12, 12, 32}, {32, 4, 1, 1, 32}, 0, 2, false, false,
+         false, 2, 128, 12, 12, 32, 1, 1, 1},
+        {"nchw32 s32 dst", F::NCHW32, S::DENSE, N::IDENTITY, {1, 1, 6, 6, 32}, {32, 1, 3, 3, 32}, 1, 1, true, false, true,
+         1, 32, 6, 6, 32, 3, 3, 1},
+        {"nchw4->nchw32", F::NCHW4_NCHW32, S::DENSE, N::RELU, {2, 4, 8, 8, 4}, {32, 4, 3, 3, 4}, 1, 1, true, false, false,
+         2, 16, 8, 8, 32, 3, 3, 1},
+        {"nchw32->nchw4", F::NCHW32_NCHW4, S::DENSE, N::RELU, {2, 1, 8, 8, 32}, {12, 1, 3, 3, 32}, 1, 1, true, false, false,
+         2, 32, 8, 8, 12, 3, 3, 1},
+        {"nchw dense", F::NCHW, S::DENSE, N::RELU, {2, 5, 9, 9}, {7, 5, 3, 3}, 1, 1, true, true, false,
+         2, 5, 9, 9, 7, 3, 3, 1},
+        {"nchw depthwise", F::NCHW, S::GROUP, N::RELU, {2, 6, 9, 9}, {6, 1, 1, 3, 3}, 1, 2, true, false, false,
+         2, 6, 9, 9, 6, 3, 3, 6},
+        {"nchw44 channel-wise", F::NCHW44, S::GROUP, N::RELU, {2, 3, 9, 9, 4}, {3, 1, 1, 3, 3, 4}, 1, 1, true, false, false,
+         2, 12, 9, 9, 12, 3, 3, 12},
+        {"nchw44 dense", F::NCHW44, S::DENSE, N::IDENTITY, {1, 2, 6, 6, 4}, {2, 2, 3, 3, 4, 4}, 1, 1, true, false, false,
+         1, 8, 6, 6, 8, 3, 3, 1},
+    };
+}
+
+static TensorShape bias_shape(const Case& c, const TensorShape& dst) {
+    if (c.fmt == CB::Format::NCHW) return {1, dst[1], 1, 1};
+    return {1, dst[1], 1, 1, dst[4]};
+}
+
+static void run_conv_case(Handle* h, const Case& c, bool on_gpu) {
+    printf("case: %s\n", c.name);
+    fflush(stdout);
+    const float s_src = 0.02f, s_flt = 0.01f, s_dst = 0.05f, s_z = 0.04f;
+    auto opr = h->create_operator<ConvBiasForward>();
+    opr->param().format = c.fmt;
+    opr->param().sparse = c.sparse;
+    opr->param().nonlineMode = c.nl;
+    opr->param().pad_h = opr->param().pad_w = c.pad;
+    opr->param().stride_h = opr->param().stride_w = c.stride;
+    TensorLayout src(c.src, dtype::QuantizedS8(s_src)), flt(c.flt, dtype::QuantizedS8(s_flt));
+    TensorLayout dst;
+    dst.dtype = c.dst_s32 ? dtype::QuantizedS32(s_src * s_flt) : dtype::QuantizedS8(s_dst);
+    TensorLayout none_b, none_z;
+    none_b.dtype = dtype::QuantizedS32(s_src * s_flt);
+    none_z.dtype = dst.dtype;
+    opr->deduce_layout(src, flt, none_b, none_z, dst);
+
+    // independent expectation of the dst shape
+    mi355_conv_desc d = mi355_conv_desc();
+    d.format = (uint32_t)c.fmt; d.sparse = (uint32_t)c.sparse; d.nonline = (uint32_t)c.nl; d.mode = 0;
+    d.n = c.n; d.ic = c.ic; d.ih = c.ih; d.iw = c.iw; d.oc = c.oc; d.fh = c.fh; d.fw = c.fw; d.group = c.group;
+    d.pad_h = d.pad_w = c.pad; d.stride_h = d.stride_w = c.stride; d.dilate_h = d.dilate_w = 1;
+    d.dst_dtype = c.dst_s32 ? MI355_DT_QS32 : MI355_DT_QS8;
+    d.bias_mode = c.has_bias ? MI355_BIAS_BROADCAST_CHANNEL : MI355_BIAS_NONE;
+    d.has_z = c.has_z;
+    d.scale_bias = s_src * s_flt; d.scale_z = c.dst_s32 ? s_src * s_flt : s_z; d.scale_dst = c.dst_s32 ? s_src * s_flt : s_dst;
+    const uint32_t oh = (c.ih + 2 * c.pad - c.fh) / c.stride + 1, ow = (c.iw + 2 * c.pad - c.fw) / c.stride + 1;
+    const bool plain = c.fmt == CB::Format::NCHW;
+    const uint32_t po = plain ? 1 : (c.fmt == CB::Format::NCHW32 || c.fmt == CB::Format::NCHW4_NCHW32) ? 32 : 4;
+    TensorShape want = plain ? TensorShape{c.n, c.oc, oh, ow} : TensorShape{c.n, c.oc / po, oh, ow, po};
+    EXPECT(dst.eq_shape(want), "deduced dst %s, expected %s", dst.to_string().c_str(), want.to_string().c_str());
+    EXPECT(dst.is_contiguous(), "deduced dst must be contiguous");
+    if (!c.dst_s32) EXPECT(dst.dtype == dtype::QuantizedS8(s_dst), "a named QuantizedS8 dst dtype must be kept");
+    else EXPECT(dst.dtype == dtype::QuantizedS32(s_src * s_flt), "default dst dtype is QuantizedS32(s_src*s_flt)");
+
+    TensorLayout bias = none_b, z = none_z;
+    if (c.has_bias) bias = TensorLayout(bias_shape(c, dst), dtype::QuantizedS32(s_src * s_flt));
+    if (c.has_z) z = TensorLayout(dst, c.dst_s32 ? dst.dtype : dtype::QuantizedS8(s_z));
+    if (c.dst_s32 && c.has_z) return;  // not in the table
+
+    size_t ws = opr->get_workspace_in_bytes(src, flt, bias, z, dst);
+    auto algos = opr->get_all_algorithms_info(src, flt, bias, z, dst);
+    EXPECT(!algos.empty(), "no usable algorithm");
+    auto heur = opr->get_algorithm_info_heuristic(src, flt, bias, z, dst);
+    bool listed = false;
+    for (auto& a : algos) listed = listed || a.desc.id == heur.desc.id;
+    EXPECT(listed, "heuristic algorithm %s is not in the list", heur.name.c_str());
+    if (!on_gpu) return;
+
+    std::vector<int8_t> hsrc(src.total_nr_elems()), hflt(flt.total_nr_elems()), hz(z.total_nr_elems());
+    std::vector<int32_t> hbias(bias.total_nr_elems());
+    fill_s8(hsrc, 11, -128, 127);
+    fill_s8(hflt, 12, -127, 127);
+    fill_s8(hz, 13, -128, 127);
+    fill_s32(hbias, 14, -1000, 1000);
+    const size_t dst_bytes = dst.total_nr_elems() * dst.dtype.size();
+    std::vector<uint8_t> expect(dst_bytes), got(dst_bytes);
+    int st = oracle_convbias_s8(&d, hsrc.data(), hflt.data(), c.has_bias ? hbias.data() : nullptr,
+                                c.has_z ? hz.data() : nullptr, expect.data());
+    EXPECT(st == 0, "CPU checker refused the case: %d", st);
+
+    DevBuf dsrc(hsrc.size()), dflt(hflt.size()), dbias(hbias.size() * 4), dz(hz.size()), ddst(dst_bytes), dws(ws);
+    HIP_OK(hipMemcpy(dsrc.p, hsrc.data(), hsrc.size(), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dflt.p, hflt.data(), hflt.size(), hipMemcpyHostToDevice));
+    if (c.has_bias) HIP_OK(hipMemcpy(dbias.p, hbias.data(), hbias.size() * 4, hipMemcpyHostToDevice));
+    if (c.has_z) HIP_OK(hipMemcpy(dz.p, hz.data(), hz.size(), hipMemcpyHostToDevice));
+
+    // every listed algorithm must reproduce the checker bit for bit
+    for (auto& a : algos) {
+        HIP_OK(hipMemset(ddst.p, 0x5a, dst_bytes));
+        opr->execution_policy().algo = a.desc;
+        size_t need = opr->get_workspace_in_bytes(src, flt, bias, z, dst);
+        EXPECT(need <= ws || need == 0, "algorithm %s wants a larger workspace", a.name.c_str());
+        opr->exec(TensorND(dsrc.p, src), TensorND(dflt.p, flt), TensorND(dbias.p, bias), TensorND(dz.p, z),
+                  TensorND(ddst.p, dst), nullptr, Workspace(dws.p, ws));
+        HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
+        HIP_OK(hipMemcpy(got.data(), ddst.p, dst_bytes, hipMemcpyDeviceToHost));
+        size_t bad = 0;
+        for (size_t i = 0; i < dst_bytes; ++i) bad += got[i] != expect[i];
+        EXPECT(bad == 0, "%s: %zu of %zu bytes differ from the CPU checker", a.name.c_str(), bad, dst_bytes);
+    }
+    printf("  %zu algorithms bit-exact (heuristic: %s)\n", algos.size(), heur.name.c_str());
+}
+
+// ------------------------------------------------------------------ validation (no device)
+static void run_validation(Handle* h) {
+    printf("case: validation errors\n");
+    auto opr = h->create_operator<ConvBiasForward>();
+    opr->param().format = CB::Format::NCHW4;
+    TensorLayout src({2, 4, 8, 8, 4}, dtype::QuantizedS8(0.02f)), flt({16, 4, 3, 3, 4}, dtype::QuantizedS8(0.01f));
+    TensorLayout nb, nz, dst;
+    nb.dtype = dtype::QuantizedS32(0.02f * 0.01f);
+    dst.dtype = dtype::QuantizedS8(0.1f);
+    opr->deduce_layout(src, flt, nb, nz, dst);
+    EXPECT(dst.eq_shape(TensorShape{2, 4, 6, 6, 4}), "pad 0 dst %s", dst.to_string().c_str());
+
+    // bias scale must equal src scale * filter scale within 1e-6
+    TensorLayout bad_bias({1, 4, 1, 1, 4}, dtype::QuantizedS32(0.5f));
+    EXPECT(throws([&] { opr->get_workspace_in_bytes(src, flt, bad_bias, nz, dst); }, MI355_ERR_BAD_ARG),
+           "bias scale mismatch must be rejected");
+    // wrong bias shape
+    TensorLayout bias5({1, 5, 1, 1, 4}, dtype::QuantizedS32(0.02f * 0.01f));
+    EXPECT(throws([&] { opr->get_workspace_in_bytes(src, flt, bias5, nz, dst); }, MI355_ERR_SHAPE),
+           "bias of the wrong shape must be rejected");
+    // z must have the dst shape
+    TensorLayout zbad({2, 4, 6, 5, 4}, dtype::QuantizedS8(0.1f));
+    EXPECT(throws([&] { opr->get_workspace_in_bytes(src, flt, nb, zbad, dst); }, MI355_ERR_SHAPE), "z shape");
+    // channel mismatch between src and filter
+    TensorLayout flt_bad({16, 3, 3, 3, 4}, dtype::QuantizedS8(0.01f));
+    TensorLayout d2 = dst;
+    EXPECT(throws([&] { opr->deduce_layout(src, flt_bad, nb, nz, d2); }, MI355_ERR_SHAPE), "channel mismatch");
+    // SIGMOID has no quantized definition
+    opr->param().nonlineMode = CB::NonlineMode::SIGMOID;
+    EXPECT(throws([&] { opr->deduce_layout(src, flt, nb, nz, d2); }, MI355_ERR_UNSUPPORTED), "SIGMOID");
+    opr->param().nonlineMode = CB::NonlineMode::RELU;
+    // dilation in a packed format
+    opr->param().dilate_h = 2;
+    EXPECT(throws([&] { opr->deduce_layout(src, flt, nb, nz, d2); }, MI355_ERR_UNSUPPORTED), "dilation in NCHW4");
+    opr->param().dilate_h = 1;
+    // unsupported format
+    opr->param().format = CB::Format::NHWC;
+    EXPECT(throws([&] { opr->deduce_layout(src, flt, nb, nz, d2); }, MI355_ERR_UNSUPPORTED), "NHWC");
+    opr->param().format = CB::Format::NCHW4;
+    // non-contiguous rows
+    TensorLayout src_nc = src;
+    src_nc.stride[2] += 4;
+    EXPECT(throws([&] { opr->deduce_layout(src_nc, flt, nb, nz, d2); }, MI355_ERR_UNSUPPORTED), "row-strided src");
+    // batch-strided src is fine
+    TensorLayout src_bs = src;
+    src_bs.stride[0] += 64;
+    opr->deduce_layout(src_bs, flt, nb, nz, d2);
+    EXPECT(d2.eq_shape(dst), "batch-strided src");
+    // undersized workspace is only checked at exec; a null tensor pointer is rejected before any launch
+    EXPECT(throws([&] {
+               opr->exec(TensorND(nullptr, src), TensorND(nullptr, flt), TensorND(nullptr, nb), TensorND(nullptr, nz),
+                         TensorND(nullptr, dst), nullptr, Workspace());
+           }, MI355_ERR_BAD_ARG),
+           "null pointers");
+    EXPECT(std::string(opr->get_algorithm_set_name()) == "MI355_CONV_BIAS", "set name");
+    EXPECT(Handle::abi_version() == MI355_CONVBIAS_ABI_VERSION, "abi version");
+
+    // RelayoutFormat deduction against the CPU checker's rule
+    auto rl = h->create_operator<RelayoutFormat>();
+    struct { param::RelayoutFormat::Mode m; TensorShape s; uint32_t oc, group; } rc[] = {
+        {param::RelayoutFormat::Mode::NCHW_NCHW4, {2, 7, 5, 6}, 0, 1},
+        {param::RelayoutFormat::Mode::NCHW_NCHW4, {2, 12, 5, 6}, 0, 4},
+        {param::RelayoutFormat::Mode::NCHW4_NCHW, {2, 2, 5, 6, 4}, 7, 1},
+        {param::RelayoutFormat::Mode::NCHW_NCHW4_WEIGHT, {6, 7, 3, 3}, 0, 1},
+        {param::RelayoutFormat::Mode::NCHW_NCHW4_IC_SMALL, {2, 3, 8, 8}, 0, 1},
+        {param::RelayoutFormat::Mode::NCHW_NCHW32, {2, 40, 5, 6}, 0, 1},
+        {param::RelayoutFormat::Mode::NCHW32_NCHW, {2, 2, 5, 6, 32}, 40, 1},
+    };
+    for (auto& r : rc) {
+        rl->param().mode = r.m; rl->param().oc = r.oc; rl->param().group = r.group;
+        TensorLayout s(r.s, dtype::QuantizedS8(1.f)), o;
+        rl->deduce_layout(s, o);
+        mi355_relayout_desc rd = mi355_relayout_desc();
+        rd.mode = (uint32_t)r.m; rd.ndim = (uint32_t)r.s.ndim; rd.group = r.group; rd.oc = r.oc; rd.elem_bytes = 1;
+        rd.scale_src = rd.scale_dst = 1.f;
+        for (size_t i = 0; i < r.s.ndim; ++i) rd.shape[i] = (uint32_t)r.s[i];
+        uint32_t nd, sh[7];
+        int st = oracle_relayout_deduce(&rd, &nd, sh);
+        bool same = st == 0 && nd == o.ndim;
+        for (uint32_t i = 0; same && i < nd; ++i) same = sh[i] == o[i];
+        EXPECT(same, "relayout mode %u: deduced %s", (unsigned)r.m, o.to_string().c_str());
+    }
+}
+
+static void run_relayout_gpu(Handle* h) {
+    printf("case: relayout exec\n");
+    fflush(stdout);
+    auto rl = h->create_operator<RelayoutFormat>();
+    struct { param::RelayoutFormat::Mode m; TensorShape s; uint32_t oc, group; float ss, sd; } rc[] = {
+        {param::RelayoutFormat::Mode::NCHW_NCHW4, {3, 7, 9, 10}, 0, 1, 1.f, 1.f},
+        {param::RelayoutFormat::Mode::NCHW_NCHW4, {3, 7, 9, 10}, 0, 1, 1.f, 2.f},
+        {param::RelayoutFormat::Mode::NCHW4_NCHW, {2, 2, 5, 6, 4}, 7, 1, 1.f, 1.f},
+        {param::RelayoutFormat::Mode::NCHW_NCHW32, {2, 40, 15, 16}, 0, 1, 1.f, 1.f},
+        {param::RelayoutFormat::Mode::NCHW32_NCHW, {2, 2, 15, 16, 32}, 40, 1, 1.f, 1.f},
+    };
+    for (auto& r : rc) {
+        rl->param().mode = r.m; rl->param().oc = r.oc; rl->param().group = r.group;
+        TensorLayout s(r.s, dtype::QuantizedS8(r.ss)), o;
+        o.dtype = dtype::QuantizedS8(r.sd);
+        rl->deduce_layout(s, o);
+        mi355_relayout_desc rd = mi355_relayout_desc();
+        rd.mode = (uint32_t)r.m; rd.ndim = (uint32_t)r.s.ndim; rd.group = r.group; rd.oc = r.oc; rd.elem_bytes = 1;
+        rd.scale_src = r.ss; rd.scale_dst = r.sd;
+        for (size_t i = 0; i < r.s.ndim; ++i) rd.shape[i] = (uint32_t)r.s[i];
+        std::vector<int8_t> hs(s.total_nr_elems()), want(o.total_nr_elems()), got(o.total_nr_elems());
+        fill_s8(hs, 21, -128, 127);
+        EXPECT(oracle_relayout(&rd, hs.data(), want.data()) == 0, "checker refused relayout");
+        DevBuf ds(hs.size()), dd(want.size());
+        HIP_OK(hipMemcpy(ds.p, hs.data(), hs.size(), hipMemcpyHostToDevice));
+        HIP_OK(hipMemset(dd.p, 0x5a, want.size()));
+        rl->exec(TensorND(ds.p, s), TensorND(dd.p, o), Workspace());
+        HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
+        HIP_OK(hipMemcpy(got.data(), dd.p, got.size(), hipMemcpyDeviceToHost));
+        EXPECT(got == want, "relayout mode %u differs from the CPU checker", (unsigned)r.m);
+    }
+}
+
+int main(int argc, char** argv) {
+    bool gpu = argc > 1 && !strcmp(argv[1], "--gpu");
+    bool cpu = argc > 1 && !strcmp(argv[1], "--cpu");
+    if (!gpu && !cpu) {
+        printf("usage: host_checker --cpu | --gpu\n");
+        return 2;
+    }
+    hipStream_t stream = nullptr;
+    if (gpu) {
+        HIP_OK(hipSetDevice(0));
+        HIP_OK(hipStreamCreate(&stream));
+    }
+    try {
+        auto handle = Handle::make(stream, 0);
+        if (gpu) handle->check_device();
+        run_validation(handle.get());
+        for (auto& c : cases()) run_conv_case(handle.get(), c, gpu);
+        if (gpu) run_relayout_gpu(handle.get());
+    } catch (const Error& e) {
+        printf("unexpected mi355dnn::Error %d: %s\n", e.status(), e.what());
+        return 1;
+    }
+    if (gpu) HIP_OK(hipStreamDestroy(stream));
+    if (g_fail) {
+        printf("%d FAILURES\n", g_fail);
+        return 1;
+    }
+    printf("ALL OK\n");
+    return 0;
+}
