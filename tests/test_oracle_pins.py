@@ -326,3 +326,55 @@ def test_fastdiv_matches_true_division(oracle):
         for k in (0, 1, 2, 63, 100, 126):
             centre = bits(np.float32((k + 0.5) * b))
             assert L.oracle_fastdiv_sweep(b, centre - 50000, 1, 100000, C.byref(bad)) == 0, (b, k, bad.value)
+
+
+# ----------------------------------------------------------------------------------------
+# relayout: requantising copy and the NCHW32 extension modes
+# ----------------------------------------------------------------------------------------
+
+def test_relayout_requantises_between_scales(oracle):
+    """QuantizedS8{1.f} -> QuantizedS8{2.f} is legal for RelayoutFormat (dnn/test/cuda/relayout_format.cpp:83-87):
+    every byte becomes quantize_dst(dequantize_src(x)) = round-half-away(x / 2), a closed form in integers."""
+    x = np.arange(-128, 128, dtype=np.int8).reshape(1, 4, 8, 8)
+    d = oracle.relayout_desc(_abi.RL_NCHW_NCHW4, x.shape, scale_src=1.0, scale_dst=2.0)
+    got = oracle.relayout(d, x)
+    xi = x.astype(np.int64)
+    half_away = np.sign(xi) * ((np.abs(xi) + 1) // 2)
+    want = half_away.reshape(1, 1, 4, 8, 8).transpose(0, 1, 3, 4, 2).astype(np.int8)
+    assert np.array_equal(got, want)
+    # up-scaling saturates: x * 4 clamps to [-128, 127]
+    d = oracle.relayout_desc(_abi.RL_NCHW_NCHW4, x.shape, scale_src=4.0, scale_dst=1.0)
+    want = np.clip(xi * 4, -128, 127).reshape(1, 1, 4, 8, 8).transpose(0, 1, 3, 4, 2).astype(np.int8)
+    assert np.array_equal(oracle.relayout(d, x), want)
+
+
+def _pack(x, p):
+    n, c, h, w = x.shape
+    cp = -(-c // p) * p
+    y = np.zeros((n, cp, h, w), x.dtype)
+    y[:, :c] = x
+    return y.reshape(n, cp // p, p, h, w).transpose(0, 1, 3, 4, 2)
+
+
+def test_relayout_nchw32_extension_modes(oracle):
+    """Modes 32-35 have no reference enumerator; they are the permutation dst[n][c/32][h][w][c%32] =
+    src[n][c][h][w] with zero padding (the map the reference's test helper from_nchw4_to_nchw32 states,
+    dnn/test/naive/conv_bias.cpp:222-269).  Checked against a direct numpy statement and against the
+    composition with the reference modes 24 / 25."""
+    rng = np.random.RandomState(3)
+    for (n, c, h, w) in ((2, 40, 3, 5), (1, 64, 4, 4), (3, 7, 2, 9), (2, 96, 3, 3)):
+        x = rng.randint(-128, 128, (n, c, h, w)).astype(np.int8)
+        d32 = oracle.relayout_desc(_abi.RL_NCHW_NCHW32, x.shape)
+        y32 = oracle.relayout(d32, x)
+        assert np.array_equal(y32, _pack(x, 32))
+        back = oracle.relayout(oracle.relayout_desc(_abi.RL_NCHW32_NCHW, y32.shape, oc=c), y32)
+        assert np.array_equal(back, x)
+        # through NCHW4: mode 24 then 34 equals mode 32; mode 35 then 25 equals mode 33
+        y4 = oracle.relayout(oracle.relayout_desc(_abi.RL_NCHW_NCHW4, x.shape), x)
+        assert np.array_equal(y4, _pack(x, 4))
+        if y4.shape[1] % 8 == 0:   # mode 34 regroups whole blocks of eight 4-packs
+            assert np.array_equal(oracle.relayout(oracle.relayout_desc(_abi.RL_NCHW4_NCHW32, y4.shape), y4), y32)
+        z4 = oracle.relayout(oracle.relayout_desc(_abi.RL_NCHW32_NCHW4, y32.shape), y32)
+        assert np.array_equal(z4, _pack(_pack(x, 32).transpose(0, 1, 4, 2, 3).reshape(n, -1, h, w), 4))
+        z4c = np.ascontiguousarray(z4[:, :-(-c // 4)])   # mode 25 crops inside the last 4-pack only
+        assert np.array_equal(oracle.relayout(oracle.relayout_desc(_abi.RL_NCHW4_NCHW, z4c.shape, oc=c), z4c), x)
