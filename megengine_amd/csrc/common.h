@@ -52,4 +52,29 @@ static inline uint32_t conv_out_size(uint32_t i, uint32_t f, uint32_t dil, uint3
     return (i + 2 * p - df) / s + 1;
 }
 
+// unsigned division by a runtime constant: q = (t + ((x - t) >> s1)) >> s2, t = mulhi(x, m)
+struct FastDiv {
+    uint32_t m, s1, s2, d;
+};
+
+static inline FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d;
+    if (d <= 1) {
+        f.m = 0; f.s1 = 0; f.s2 = 0;
+        return f;
+    }
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    f.m = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    f.s1 = 1;
+    f.s2 = l - 1;
+    return f;
+}
+
+__device__ __forceinline__ uint32_t fdiv(uint32_t x, const FastDiv& f) {
+    uint32_t t = __umulhi(x, f.m);
+    return (t + ((x - t) >> f.s1)) >> f.s2;
+}
+
 }  // namespace mi355

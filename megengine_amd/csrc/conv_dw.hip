@@ -10,6 +10,8 @@
 //   * consecutive lanes own consecutive pixel quads: loads are coalesced dwords, the store is a
 //     16-byte vector per lane (1 KiB per wavefront);
 //   * all threads of a workgroup share (n, c/4), so filter and bias loads are scalar.
+// That form (dw4_kernel) serves every filter size / stride.  The 3x3, stride 1 or 2 case -- every
+// channel-wise layer of the MobileNet family -- has its own kernel, dw3x3_kernel, below.
 #include "common.h"
 
 namespace mi355 {
@@ -127,6 +129,232 @@ __global__ __launch_bounds__(256) void dw4_kernel(DwArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// 3x3, stride S in {1, 2}: one thread = 4 consecutive output pixels x R output rows x 4 channels.
+//
+//   * work items (image, channel quad, row strip, pixel quad) are flattened over the whole launch,
+//     so 7x7 planes fill wavefronts as well as 112x112 ones; lanes run along a row, so the 16-byte
+//     loads and stores of neighbouring lanes are contiguous;
+//   * an input row is read once per thread as 16-byte vectors and serves up to three output rows;
+//   * the 4 pixels x 4 channels block is transposed in registers (8 v_perm) so that one dword holds
+//     4 consecutive pixels of ONE channel; a filter row [w0 w1 w2 0] (or shifted, [0 w0 w1 w2]) then
+//     multiplies three horizontally adjacent taps with a single v_dot4: 3 dot products per output
+//     instead of 9.
+// ---------------------------------------------------------------------------------------------
+struct Dw3Args {
+    const int8_t* src;
+    const int8_t* flt;
+    const int32_t* bias;
+    const int8_t* z;
+    int8_t* dst;
+    int CG, IH, IW, OH, OW, QW, OHS;  // QW = pixel quads per output row, OHS = row strips per plane
+    int ph, pw;
+    uint32_t items;
+    int64_t src_sn, dst_sn, z_sn;
+    int has_bias;
+    FastDiv div_qw, div_ohs, div_cg;
+    EpiParams epi;
+};
+
+__device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) {
+    return __builtin_amdgcn_perm(hi, lo, sel);
+}
+
+// pixels (dwords of 4 channels) p[0..3]  ->  t[c] = {p0.c, p1.c, p2.c, p3.c}
+__device__ __forceinline__ void transpose4(const uint32_t p[4], uint32_t t[4]) {
+    const uint32_t a = perm(p[1], p[0], 0x05010400u), b = perm(p[1], p[0], 0x07030602u);
+    const uint32_t c = perm(p[3], p[2], 0x05010400u), d = perm(p[3], p[2], 0x07030602u);
+    t[0] = perm(c, a, 0x05040100u);
+    t[1] = perm(c, a, 0x07060302u);
+    t[2] = perm(d, b, 0x05040100u);
+    t[3] = perm(d, b, 0x07060302u);
+}
+
+// 4 consecutive pixels of one input row starting at column c0 (any of them may fall outside the row)
+__device__ __forceinline__ void load_px4(const uint32_t* row, int c0, int IW, bool rok, uint32_t p[4]) {
+    if (rok && c0 >= 0 && c0 + 3 < IW) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(row + c0);  // needs 4-byte alignment only
+        p[0] = v[0]; p[1] = v[1]; p[2] = v[2]; p[3] = v[3];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) p[i] = (rok && (unsigned)(c0 + i) < (unsigned)IW) ? row[c0 + i] : 0u;
+    }
+}
+
+template <int R, int NL, bool HZ, bool FAST>
+__device__ __forceinline__ void dw3_store(const Dw3Args& a, const int (&acc)[R][4][4], int n, int cg, int oh0, int ow0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int oh = oh0 + r;
+        if (oh >= a.OH) break;
+        const int64_t off = (((int64_t)cg * a.OH + oh) * a.OW + ow0) * 4;
+        uint32_t* dp = reinterpret_cast<uint32_t*>(a.dst + n * a.dst_sn + off);
+        const uint32_t* zp = reinterpret_cast<const uint32_t*>(a.z + n * a.z_sn + off);
+        const bool full = ow0 + 3 < a.OW;
+        uint32_t zw[4] = {0u, 0u, 0u, 0u};
+        if (FAST ? HZ : a.epi.has_z != 0) {
+            if (full) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(zp);
+                zw[0] = v[0]; zw[1] = v[1]; zw[2] = v[2]; zw[3] = v[3];
+            } else {
+#pragma unroll
+                for (int x = 0; x < 4; ++x) zw[x] = ow0 + x < a.OW ? zp[x] : 0u;
+            }
+        }
+        u32x4 o;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            if (FAST)
+                o[x] = requant4_fast<NL, HZ>(acc[r][x][0], acc[r][x][1], acc[r][x][2], acc[r][x][3], zw[x], a.epi);
+            else
+                o[x] = requant4_exact(acc[r][x][0], acc[r][x][1], acc[r][x][2], acc[r][x][3], zw[x], a.epi);
+        }
+        if (full) {
+            *reinterpret_cast<u32x4*>(dp) = o;
+        } else {
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+                if (ow0 + x < a.OW) dp[x] = o[x];
+        }
+    }
+}
+
+template <int S, int R>
+__global__ __launch_bounds__(256) void dw3x3_kernel(Dw3Args a) {
+    const uint32_t item = blockIdx.x * 256u + threadIdx.x;
+    if (item >= a.items) return;
+    // item = ((n * CG + cg) * OHS + strip) * QW + quad
+    const uint32_t i1 = fdiv(item, a.div_qw), q = item - i1 * a.QW;
+    const uint32_t i2 = fdiv(i1, a.div_ohs), strip = i1 - i2 * a.OHS;
+    const uint32_t n = fdiv(i2, a.div_cg), cg = i2 - n * a.CG;
+    const int oh0 = (int)strip * R, ow0 = (int)q * 4;
+
+    // filter rows per channel: wlo = {w(fh,0), w(fh,1), w(fh,2), 0}, whi = the same one byte up
+    uint32_t wlo[3][4], whi[3][4];
+    {
+        const uint32_t* wp = reinterpret_cast<const uint32_t*>(a.flt) + cg * 9;
+#pragma unroll
+        for (int fh = 0; fh < 3; ++fh) {
+            const uint32_t w0 = wp[fh * 3], w1 = wp[fh * 3 + 1], w2 = wp[fh * 3 + 2];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t t = perm(w1, w0, 0x0c0c0000u | ((4u + c) << 8) | (uint32_t)c);
+                wlo[fh][c] = perm(w2, t, 0x0c000100u | ((4u + c) << 16));
+                whi[fh][c] = wlo[fh][c] << 8;
+            }
+        }
+    }
+    v4i bias4 = {0, 0, 0, 0};
+    if (a.has_bias) bias4 = *reinterpret_cast<const v4i*>(a.bias + cg * 4);
+    int acc[R][4][4];
+
+    const uint32_t* sp = reinterpret_cast<const uint32_t*>(a.src + n * a.src_sn) + (int64_t)cg * a.IH * a.IW;
+    const int c0 = ow0 * S - a.pw;              // leftmost input column of this thread's window
+    constexpr int ROWS = (R - 1) * S + 3;       // input rows touched by R output rows
+    // window columns: L = c0, block T = c0+1 .. c0+4, then (S = 1) Rt = c0+5 or (S = 2) block U = c0+5 .. c0+8
+    uint32_t L[ROWS], Rt[ROWS], pt[ROWS][4], pu[ROWS][4];
+    const bool interior = c0 + 1 >= 0 && c0 + (S == 1 ? 4 : 8) < a.IW;
+    if (interior) {
+        // every vector load is in range: rows are clamped and masked afterwards, so all loads of the thread are
+        // independent of any branch and go out back to back
+        const bool lok = c0 >= 0, rtok = c0 + 5 < a.IW;
+        const int cl = lok ? c0 : 0, cr = rtok ? c0 + 5 : 0;
+#pragma unroll
+        for (int ir = 0; ir < ROWS; ++ir) {
+            const int ih = oh0 * S + ir - a.ph;
+            const int ihc = min(max(ih, 0), a.IH - 1);
+            const uint32_t* row = sp + ihc * a.IW;
+            L[ir] = row[cl];
+            const u32x4 v = *reinterpret_cast<const u32x4*>(row + c0 + 1);  // needs 4-byte alignment only
+            pt[ir][0] = v[0]; pt[ir][1] = v[1]; pt[ir][2] = v[2]; pt[ir][3] = v[3];
+            if (S == 1) {
+                Rt[ir] = row[cr];
+            } else {
+                const u32x4 u = *reinterpret_cast<const u32x4*>(row + c0 + 5);
+                pu[ir][0] = u[0]; pu[ir][1] = u[1]; pu[ir][2] = u[2]; pu[ir][3] = u[3];
+            }
+        }
+#pragma unroll
+        for (int ir = 0; ir < ROWS; ++ir) {
+            const int ih = oh0 * S + ir - a.ph;
+            const bool rok = (unsigned)ih < (unsigned)a.IH;
+            L[ir] = (rok && lok) ? L[ir] : 0u;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pt[ir][i] = rok ? pt[ir][i] : 0u;
+            if (S == 1) {
+                Rt[ir] = (rok && rtok) ? Rt[ir] : 0u;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) pu[ir][i] = rok ? pu[ir][i] : 0u;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int ir = 0; ir < ROWS; ++ir) {
+            const int ih = oh0 * S + ir - a.ph;
+            const bool rok = (unsigned)ih < (unsigned)a.IH;
+            const uint32_t* row = sp + (int64_t)ih * a.IW;
+            L[ir] = (rok && (unsigned)c0 < (unsigned)a.IW) ? row[c0] : 0u;
+            load_px4(row, c0 + 1, a.IW, rok, pt[ir]);
+            if (S == 1)
+                Rt[ir] = (rok && (unsigned)(c0 + 5) < (unsigned)a.IW) ? row[c0 + 5] : 0u;
+            else
+                load_px4(row, c0 + 5, a.IW, rok, pu[ir]);
+        }
+    }
+
+#pragma unroll
+    for (int ir = 0; ir < ROWS; ++ir) {
+        uint32_t T[4], U[4] = {0u, 0u, 0u, 0u};
+        transpose4(pt[ir], T);
+        if (S == 2) transpose4(pu[ir], U);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            // three-tap windows of the 4 outputs, one channel: e[x] holds the taps in the bytes its filter row expects
+            uint32_t e0, e1, e2, e3;
+            e0 = perm(T[c], L[ir], 0x0c050400u | (uint32_t)c);               // {L.c, T0, T1, -}   -> wlo
+            if (S == 1) {
+                e1 = T[c];                                                     // {T0, T1, T2, -}    -> wlo
+                e2 = T[c];                                                     // {-, T1, T2, T3}    -> whi
+                e3 = perm(Rt[ir], T[c], 0x0003020cu | ((4u + c) << 24));       // {-, T2, T3, Rt.c}  -> whi
+            } else {
+                e1 = T[c];                                                     // {-, T1, T2, T3}    -> whi
+                e2 = perm(U[c], T[c], 0x0c050403u);                            // {T3, U0, U1, -}    -> wlo
+                e3 = U[c];                                                     // {-, U1, U2, U3}    -> whi
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int fh = ir - r * S;
+                if (fh < 0 || fh > 2) continue;
+                const int lo = (int)wlo[fh][c], hi = (int)whi[fh][c];
+                // the first filter row of an output row starts from the bias
+                const int p0 = fh ? acc[r][0][c] : bias4[c], p1 = fh ? acc[r][1][c] : bias4[c];
+                const int p2 = fh ? acc[r][2][c] : bias4[c], p3 = fh ? acc[r][3][c] : bias4[c];
+                acc[r][0][c] = __builtin_amdgcn_sdot4((int)e0, lo, p0, false);
+                acc[r][1][c] = __builtin_amdgcn_sdot4((int)e1, S == 1 ? lo : hi, p1, false);
+                acc[r][2][c] = __builtin_amdgcn_sdot4((int)e2, S == 1 ? hi : lo, p2, false);
+                acc[r][3][c] = __builtin_amdgcn_sdot4((int)e3, hi, p3, false);
+            }
+        }
+    }
+
+    if (!a.epi.fast) {
+        dw3_store<R, 0, false, false>(a, acc, n, cg, oh0, ow0);
+    } else if (a.epi.has_z) {
+        switch (a.epi.nonline) {
+            case NL_RELU: dw3_store<R, NL_RELU, true, true>(a, acc, n, cg, oh0, ow0); break;
+            case NL_H_SWISH: dw3_store<R, NL_H_SWISH, true, true>(a, acc, n, cg, oh0, ow0); break;
+            default: dw3_store<R, NL_IDENTITY, true, true>(a, acc, n, cg, oh0, ow0); break;
+        }
+    } else {
+        switch (a.epi.nonline) {
+            case NL_RELU: dw3_store<R, NL_RELU, false, true>(a, acc, n, cg, oh0, ow0); break;
+            case NL_H_SWISH: dw3_store<R, NL_H_SWISH, false, true>(a, acc, n, cg, oh0, ow0); break;
+            default: dw3_store<R, NL_IDENTITY, false, true>(a, acc, n, cg, oh0, ow0); break;
+        }
+    }
+}
+
 }  // namespace
 
 bool depthwise_usable(const ConvProblem& p) {
@@ -151,17 +379,35 @@ int launch_conv_depthwise(hipStream_t st, const ConvProblem& p, const int8_t* sr
     a.has_bias = d.bias_mode == MI355_BIAS_BROADCAST_CHANNEL;
     a.vec_ok = (p.ow % 4 == 0) && (p.dst_sn % 16 == 0) && (!d.has_z || p.z_sn % 16 == 0);
     a.epi = p.epi;
+    if (d.n == 0 || p.oh == 0 || p.ow == 0) return 0;
+    const bool sq = d.fh == 3 && d.fw == 3 && d.stride_h == d.stride_w && (d.stride_h == 1 || d.stride_h == 2);
+    if (sq) {
+        const int R = d.stride_h == 1 ? (p.oh % 4 == 0 ? 4 : 2) : (p.oh % 2 == 0 ? 2 : 1);
+        Dw3Args b;
+        b.src = src; b.flt = flt; b.bias = bias; b.z = z; b.dst = dst;
+        b.CG = a.CG; b.IH = a.IH; b.IW = a.IW; b.OH = a.OH; b.OW = a.OW; b.QW = a.QW; b.OHS = (a.OH + R - 1) / R;
+        b.ph = a.ph; b.pw = a.pw;
+        b.src_sn = a.src_sn; b.dst_sn = a.dst_sn; b.z_sn = a.z_sn; b.has_bias = a.has_bias; b.epi = a.epi;
+        const int64_t items = (int64_t)d.n * b.CG * b.OHS * b.QW;
+        if (items < ((int64_t)1 << 31) - 256) {
+            b.items = (uint32_t)items;
+            b.div_qw = make_fastdiv(b.QW); b.div_ohs = make_fastdiv(b.OHS); b.div_cg = make_fastdiv(b.CG);
+            dim3 grid((unsigned)((items + 255) / 256)), block(256);
+            if (d.stride_h == 1 && R == 4)
+                hipLaunchKernelGGL((dw3x3_kernel<1, 4>), grid, block, 0, st, b);
+            else if (d.stride_h == 1)
+                hipLaunchKernelGGL((dw3x3_kernel<1, 2>), grid, block, 0, st, b);
+            else if (R == 2)
+                hipLaunchKernelGGL((dw3x3_kernel<2, 2>), grid, block, 0, st, b);
+            else
+                hipLaunchKernelGGL((dw3x3_kernel<2, 1>), grid, block, 0, st, b);
+            return (int)hipGetLastError();
+        }
+    }
     const int quads = a.OH * a.QW;
-    if (quads == 0 || d.n == 0) return 0;
     const int threads = quads >= 192 ? 256 : (quads > 64 ? 128 : 64);
     dim3 grid((quads + threads - 1) / threads, d.n * a.CG), block(threads);
-    const bool sq = d.fh == 3 && d.fw == 3 && d.stride_h == d.stride_w;
-    if (sq && d.stride_h == 1)
-        hipLaunchKernelGGL((dw4_kernel<3, 1>), grid, block, 0, st, a);
-    else if (sq && d.stride_h == 2)
-        hipLaunchKernelGGL((dw4_kernel<3, 2>), grid, block, 0, st, a);
-    else
-        hipLaunchKernelGGL((dw4_kernel<0, 0>), grid, block, 0, st, a);
+    hipLaunchKernelGGL((dw4_kernel<0, 0>), grid, block, 0, st, a);
     return (int)hipGetLastError();
 }
 

@@ -33,31 +33,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int IG_THREADS = 256;
 constexpr int IG_MAX_ENTRIES = 2048;  // k-unit table capacity (entries of 8 bytes)
 
-// unsigned division by a runtime constant: q = (t + ((x - t) >> s1)) >> s2, t = mulhi(x, m)
-struct FastDiv {
-    uint32_t m, s1, s2, d;
-};
-
-FastDiv make_fastdiv(uint32_t d) {
-    FastDiv f;
-    f.d = d;
-    if (d <= 1) {
-        f.m = 0; f.s1 = 0; f.s2 = 0;
-        return f;
-    }
-    uint32_t l = 0;
-    while ((1ull << l) < d) ++l;
-    f.m = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
-    f.s1 = 1;
-    f.s2 = l - 1;
-    return f;
-}
-
-__device__ __forceinline__ uint32_t fdiv(uint32_t x, const FastDiv& f) {
-    uint32_t t = __umulhi(x, f.m);
-    return (t + ((x - t) >> f.s1)) >> f.s2;
-}
-
 struct IgemmArgs {
     const int8_t* src;
     const int8_t* flt;

@@ -170,6 +170,11 @@ DW_CASES = [
     ("NCHW4", 1, 8, 12, 12, 5, 2, 1),      # generic filter size
     ("NCHW4", 1, 8, 9, 16, 3, 0, 1),       # no padding
     ("NCHW44", 1, 8, 11, 11, 3, 1, 3),     # generic stride
+    ("NCHW4", 1, 8, 15, 9, 3, 1, 1),       # odd output height: the last row strip is half empty
+    ("NCHW4", 1, 8, 10, 10, 3, 0, 2),      # stride 2 without padding
+    ("NCHW4", 1, 8, 9, 9, 3, 2, 1),        # padding wider than the filter radius
+    ("NCHW4", 3, 12, 5, 5, 3, 1, 2),       # planes much smaller than a wavefront
+    ("NCHW4", 2, 8, 6, 37, 3, 1, 1),       # ragged row ends (iw % 4 = 1)
 ]
 
 
@@ -182,6 +187,10 @@ def test_depthwise(oracle, i):
             a, _ = ops.conv_bias_query(d)
             assert a.id == DW
             check_case(oracle, d, seed=200 + i, tag="dw%d" % i)
+    # scales outside the range of the divide-free epilogue: the kernel must take the literal chain
+    d = _abi.make_conv_desc(fmt, n, c, ih, iw, c, f, group=c, pad=pad, stride=stride, nonline="RELU", has_z=True,
+                            scale_bias=1e-20, scale_z=3e-19, scale_dst=1e-18)
+    check_case(oracle, d, seed=300 + i, tag="dw%d-literal" % i)
 
 
 # ---------------------------------------------------------------------------------------------
