@@ -21,69 +21,10 @@
 // oc = 8*(v/4) + 4*(l/32) + v%4.  NCHW4 output stores one dword (4 channels) per register quad;
 // NCHW32 output first exchanges quads between lanes l and l+32 (v_permlane32_swap) so that each
 // lane owns 16 consecutive channels of one pixel and stores 16 bytes.
-#include "common.h"
+#include "igemm_shared.h"
 
 namespace mi355 {
 namespace {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-constexpr int IG_THREADS = 256;
-constexpr int IG_MAX_ENTRIES = 2048;  // k-unit table capacity (entries of 8 bytes)
-
-struct IgemmArgs {
-    const int8_t* src;
-    const int8_t* flt;
-    const int32_t* bias;
-    const int8_t* z;
-    int8_t* dst;
-    uint32_t src_bytes, flt_bytes, z_bytes, dst_bytes;
-    int IH, IW, OH, OW, OHW;
-    int FH, FW, T;
-    int sh, sw, ph, pw;
-    int OC;
-    int M;            // n * oh * ow
-    int kbytes;       // filter bytes per output channel
-    int KC;           // 32-byte k-chunks (ceil)
-    int entries;      // valid k-unit table entries (KC for NCHW32, ic/4*T for NCHW4)
-    int nstages;
-    int src_sn, src_scb;      // bytes: per image, per channel block
-    int dst_sn, dst_scb;      // bytes: per image, per output channel block
-    int z_sn;
-    int tiles_m, tiles_n, tiles;
-    int has_bias;
-    FastDiv div_ohw, div_ow, div_t, div_fw;
-    EpiParams epi;
-};
-
-struct KEntry {
-    int off;    // byte offset of the k-unit relative to the pixel's (ih0, iw0) base
-    int fhfw;   // fh | fw << 16 ; fh = 0x4000 marks a padding entry (never valid)
-};
-
-// 16-byte slot swizzle (S = slots per row), derived from how gfx950 serves 128-bit LDS accesses
-// (measured with SQ_LDS_BANK_CONFLICT on single-wave probes):
-//   ds_read_b128 : 64 banks; 4 passes over all 64 lanes; in pass k lane l reads dword (k + l/16) % 4
-//   ds_write_b128: behaves as 32 banks; half-wave at a time, 4 passes; lane l writes dword (k + l/8) % 4
-// MFMA fragment reads (lane -> row l%32, slot-half l/32) need, per row class (row mod 256/ROWB rows),
-// distinct slots for the rows of one 16-lane group; loader writes (lane -> row l/2, half l%2) need
-// disjoint slot pairs for the rows of one 8-lane group.  With r_i = bit i of the row:
-template <int S>
-__device__ __forceinline__ int swz(int row) {
-    const int r0 = row & 1, r1 = (row >> 1) & 1, r2 = (row >> 2) & 1, r3 = (row >> 3) & 1;
-    if (S == 4) return ((r1 ^ r2) << 1) | r3;
-    if (S == 8) return (r1 << 2) | ((r0 ^ r2) << 1) | r3;
-    if (S == 16) return r2 | (r0 << 1) | (r1 << 2) | (r3 << 3);
-    return 0;
-}
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
-}
-
-constexpr int SENT = (int)0x80000000;  // byte offset that is out of range for every buffer (< 2 GiB)
 
 // PW = pointwise fast path: 1x1 filter, no padding, K a multiple of the stage depth.  Its loaders need no
 // bounds tests and no k-unit table: every address is a per-row base plus a wave-uniform term.
@@ -413,7 +354,7 @@ struct IgemmKernel {
             // ---- bookkeeping
             if (last_stage) {
                 if (DUAL) acc[0][0] += alt;
-                run_epilogue(a, acc, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh);
+                igemm_run_epilogue<POUT, MT, NT>(a, acc, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh);
                 c_stage = 0;
                 c_tile += step;
                 if (a.tiles_m > 1) {
@@ -436,74 +377,6 @@ struct IgemmKernel {
         }
     }
 
-    __device__ static __forceinline__ void run_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w,
-                                                        int l32, int lh) {
-        if (a.epi.has_z) {
-            switch (a.epi.nonline) {
-                case NL_RELU: epilogue<NL_RELU, true>(a, acc, oc_w, pix_w, l32, lh); break;
-                case NL_H_SWISH: epilogue<NL_H_SWISH, true>(a, acc, oc_w, pix_w, l32, lh); break;
-                default: epilogue<NL_IDENTITY, true>(a, acc, oc_w, pix_w, l32, lh); break;
-            }
-        } else {
-            switch (a.epi.nonline) {
-                case NL_RELU: epilogue<NL_RELU, false>(a, acc, oc_w, pix_w, l32, lh); break;
-                case NL_H_SWISH: epilogue<NL_H_SWISH, false>(a, acc, oc_w, pix_w, l32, lh); break;
-                default: epilogue<NL_IDENTITY, false>(a, acc, oc_w, pix_w, l32, lh); break;
-            }
-        }
-    }
-
-    template <int NL, bool HZ>
-    __device__ static __forceinline__ void epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w,
-                                                    int l32, int lh) {
-        const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(a.z, HZ ? a.z_bytes : 0);
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-            const int m = pix_w + j * 32 + l32;
-            const bool pok = m < a.M;
-            const uint32_t mm = pok ? m : 0;
-            const uint32_t n = fdiv(mm, a.div_ohw), rem = mm - n * a.OHW;
-            const int d_pix = (int)n * a.dst_sn + (int)rem * POUT;
-            const int z_pix = (int)n * a.z_sn + (int)rem * POUT;
-#pragma unroll
-            for (int i = 0; i < MT; ++i) {
-                const int ocb = oc_w + i * 32;  // first channel of this 32-channel block
-                if (ocb >= a.OC) continue;      // wave-uniform
-                const v16i& c = acc[i][j];
-                if (POUT == 32) {
-                    const int blk_off = (ocb >> 5) * a.dst_scb + lh * 16;
-                    uint32_t zq[4] = {0, 0, 0, 0};
-                    if (HZ) {
-                        v4i zv = __builtin_amdgcn_raw_buffer_load_b128(rs_z, pok ? z_pix + blk_off : -1, 0, 0);
-                        // stored order (16 consecutive channels per lane) -> accumulator order
-                        auto s0 = __builtin_amdgcn_permlane32_swap((uint32_t)zv[0], (uint32_t)zv[1], false, false);
-                        auto s1 = __builtin_amdgcn_permlane32_swap((uint32_t)zv[2], (uint32_t)zv[3], false, false);
-                        zq[0] = s0[0]; zq[2] = s0[1]; zq[1] = s1[0]; zq[3] = s1[1];
-                    }
-                    uint32_t o[4];
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        o[q] = requant4_fast<NL, HZ>(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], zq[q], a.epi);
-                    // accumulator order -> stored order
-                    auto s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
-                    auto s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
-                    u32x4 out = {s0[0], s0[1], s1[0], s1[1]};
-                    if (pok) *reinterpret_cast<u32x4*>(a.dst + d_pix + blk_off) = out;
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int oc4 = ocb + 8 * q + 4 * lh;  // first of 4 channels; oc is a multiple of 4
-                        const bool ok = pok && oc4 < a.OC;
-                        const int off = (oc4 >> 2) * a.dst_scb;
-                        uint32_t zw = 0;
-                        if (HZ) zw = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_z, ok ? z_pix + off : -1, 0, 0);
-                        uint32_t o = requant4_fast<NL, HZ>(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], zw, a.epi);
-                        if (ok) *reinterpret_cast<uint32_t*>(a.dst + d_pix + off) = o;
-                    }
-                }
-            }
-        }
-    }
 };
 
 template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH, int MINW, bool PW>
@@ -594,8 +467,12 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
 
 }  // namespace
 
-int igemm_num_cfgs() { return kNumCfgs; }
-const char* igemm_cfg_name(int cfg) { return cfg >= 0 && cfg < kNumCfgs ? kCfgs[cfg].name : "?"; }
+// tile_cfg numbering: the register-staged tiles first, then the LDS-direct ones
+int igemm_num_cfgs() { return kNumCfgs + igemm_dma_num_cfgs(); }
+const char* igemm_cfg_name(int cfg) {
+    if (cfg >= 0 && cfg < kNumCfgs) return kCfgs[cfg].name;
+    return igemm_dma_cfg_name(cfg - kNumCfgs);
+}
 
 bool igemm_usable(const ConvProblem& p) {
     const mi355_conv_desc& d = p.d;
@@ -629,6 +506,21 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
     auto tiles = [&](int cfg) { return ((OC + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm) * ((M + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn); };
     const int kbytes = d.ic * d.fh * d.fw;
     if (OC <= 32) return 4;
+    if (p.pin == 32) {
+        // 32-packed inputs: LDS-direct tiles (ids after the register-staged ones), chosen from a sweep of every
+        // tile over the ResNet-50 / large-convolution shapes.  t128 = number of 128x128 tiles.
+        enum {
+            D128x128x64 = kNumCfgs + 0, D64x64x128 = kNumCfgs + 1, D128x64x128 = kNumCfgs + 2, D128x128x128r2 = kNumCfgs + 7,
+            D64x64x64r4 = kNumCfgs + 10, D64x128x128r2 = kNumCfgs + 13, D128x64x128r2 = kNumCfgs + 11
+        };
+        if (OC <= 64) return kbytes <= 64 ? D64x64x64r4 : D64x128x128r2;
+        const int64_t t128 = tiles(0);
+        if (t128 >= 4 * cu_count) return kbytes >= 1024 ? D128x128x128r2 : 0;
+        if (t128 >= 2 * cu_count) return D128x64x128r2;
+        if (2 * t128 >= 3 * cu_count) return kbytes >= 512 ? D128x128x128r2 : D128x128x64;
+        // few tiles, long reductions: the deeper ring hides the cold first touch of every weight byte
+        return tiles(7) >= cu_count ? D128x64x128 : D64x64x128;
+    }
     if (OC <= 64) return tiles(1) >= cu_count ? 1 : 3;
     // 128x128 tiles as soon as they give every CU 1.5 tiles; the deeper k stage pays once the
     // reduction is long enough to amortise its larger prologue
@@ -668,6 +560,17 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
     a.div_fw = make_fastdiv(a.FW);
     a.epi = p.epi;
     if (a.M == 0 || a.OC == 0) return 0;
+    if (cfg >= kNumCfgs) {
+        const int dcfg = cfg - kNumCfgs;
+        if (dcfg >= igemm_dma_num_cfgs()) return (int)hipErrorInvalidValue;
+        if (p.pin == 32) return launch_igemm_dma(st, a, p.pout, dcfg, cu_count);
+        // 4-packed inputs have no LDS-direct path: run the register-staged tile of the same shape
+        int bm, bn, kch;
+        igemm_dma_cfg_shape(dcfg, &bm, &bn, &kch);
+        cfg = 0;
+        for (int i = 0; i < kNumCfgs; ++i)
+            if (kCfgs[i].bm == bm && kCfgs[i].bn == bn && kCfgs[i].kch == kch) cfg = i;
+    }
     if (p.pin == 32 && p.pout == 32) return launch_fmt<32, 32>(st, a, cfg, cu_count);
     if (p.pin == 4 && p.pout == 4) return launch_fmt<4, 4>(st, a, cfg, cu_count);
     if (p.pin == 4 && p.pout == 32) return launch_fmt<4, 32>(st, a, cfg, cu_count);
