@@ -510,16 +510,18 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
         // 32-packed inputs: LDS-direct tiles (ids after the register-staged ones), chosen from a sweep of every
         // tile over the ResNet-50 / large-convolution shapes.  t128 = number of 128x128 tiles.
         enum {
-            D128x128x64 = kNumCfgs + 0, D64x64x128 = kNumCfgs + 1, D128x64x128 = kNumCfgs + 2, D128x128x128r2 = kNumCfgs + 7,
-            D64x64x64r4 = kNumCfgs + 10, D64x128x128r2 = kNumCfgs + 13, D128x64x128r2 = kNumCfgs + 11
+            D128x128x64 = kNumCfgs + 0, D64x64x128 = kNumCfgs + 1, D128x128x128r2 = kNumCfgs + 7, D64x64x64r4 = kNumCfgs + 10,
+            D128x64x128r2 = kNumCfgs + 11, D64x128x128r2 = kNumCfgs + 13, D128x128x64w8 = kNumCfgs + 14,
+            D128x64x128w8 = kNumCfgs + 15, D256x128x64w8 = kNumCfgs + 16, D128x128x128r2w8 = kNumCfgs + 17
         };
         if (OC <= 64) return kbytes <= 64 ? D64x64x64r4 : D64x128x128r2;
         const int64_t t128 = tiles(0);
-        if (t128 >= 4 * cu_count) return kbytes >= 1024 ? D128x128x128r2 : 0;
+        if (t128 >= 4 * cu_count)
+            return kbytes >= 1024 ? (OC >= 256 ? D256x128x64w8 : D128x128x128r2) : (kbytes <= 128 ? D128x128x64w8 : 0);
         if (t128 >= 2 * cu_count) return D128x64x128r2;
-        if (2 * t128 >= 3 * cu_count) return kbytes >= 512 ? D128x128x128r2 : D128x128x64;
+        if (2 * t128 >= 3 * cu_count) return kbytes >= 512 ? D128x128x128r2w8 : D128x128x64;
         // few tiles, long reductions: the deeper ring hides the cold first touch of every weight byte
-        return tiles(7) >= cu_count ? D128x64x128 : D64x64x128;
+        return tiles(7) >= cu_count ? D128x64x128w8 : D64x64x128;
     }
     if (OC <= 64) return tiles(1) >= cu_count ? 1 : 3;
     // 128x128 tiles as soon as they give every CU 1.5 tiles; the deeper k stage pays once the

@@ -50,6 +50,8 @@ __device__ __forceinline__ v4i uniform_rsrc(const void* p, uint32_t bytes) {
 
 template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, bool PW>
 struct DmaKernel {
+    static constexpr int NW = WM * WN;             // waves per workgroup (4 or 8)
+    static constexpr int THREADS = NW * 64;
     static constexpr int WTM = BM / WM, WTN = BN / WN;
     static constexpr int MT = WTM / 32, NT = WTN / 32;
     static constexpr int S = KCH * 2;              // 16-byte slots per LDS row
@@ -57,15 +59,15 @@ struct DmaKernel {
     static constexpr int RPL = 64 / S;             // rows per wave copy (64 slots = 1 KiB)
     static constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB;
     static constexpr int STG = A_BYTES + B_BYTES;  // one stage
-    static constexpr int UA = BM / (RPL * 4);      // copies per wave per stage
-    static constexpr int UB = BN / (RPL * 4);
+    static constexpr int UA = BM / (RPL * NW);     // copies per wave per stage
+    static constexpr int UB = BN / (RPL * NW);
     static constexpr int U = UA + UB;
     static constexpr int BIAS_BYTES = 2 * BM * 4;
     static constexpr int RING_BYTES = NS * STG + BIAS_BYTES;
-    static_assert(WM * WN * 64 == IG_THREADS, "4 waves");
-    static_assert(UA >= 1 && UB >= 1 && BM % (RPL * 4) == 0 && BN % (RPL * 4) == 0, "tile vs copy granularity");
+    static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+    static_assert(UA >= 1 && UB >= 1 && BM % (RPL * NW) == 0 && BN % (RPL * NW) == 0, "tile vs copy granularity");
     static_assert(NS >= 2 && (NS - 2) * U < 64, "ring depth");
-    // swz() looks at row bits 0..3; rows of copy j of wave w are (4 j + w) * RPL + lane / S, so with RPL >= 8 those
+    // swz() looks at row bits 0..3; rows of copy j of wave w are (NW j + w) * RPL + lane / S, so with RPL >= 8 those
     // bits never depend on j: a lane's logical slot is the same for all of its copies
     static_assert(RPL >= 8, "slot must not depend on the copy index");
 
@@ -83,7 +85,7 @@ struct DmaKernel {
     }
 
     // lane's row inside copy j of wave w, and its logical slot (constant per lane)
-    __device__ static __forceinline__ int row_of(int w, int lane, int j) { return (4 * j + w) * RPL + lane / S; }
+    __device__ static __forceinline__ int row_of(int w, int lane, int j) { return (NW * j + w) * RPL + lane / S; }
     __device__ static __forceinline__ int slot_of(int w, int lane) { return (lane % S) ^ swz<S>(w * RPL + lane / S); }
 
     __device__ static __forceinline__ void loader_enter_tile(const IgemmArgs& a, Loader& L, int tile, int w, int lane) {
@@ -132,13 +134,13 @@ struct DmaKernel {
 #pragma unroll
         for (int j = 0; j < UA; ++j) {
             // SENT plus a stage offset is still out of range
-            lds_copy64x16(stage_addr + (uint32_t)((4 * j + w) * 1024), L.a_off[j] + a_k, rs_flt);
+            lds_copy64x16(stage_addr + (uint32_t)((NW * j + w) * 1024), L.a_off[j] + a_k, rs_flt);
         }
         if (PW) {
             const int b_k = L.kc0 * a.src_scb;
 #pragma unroll
             for (int j = 0; j < UB; ++j) {
-                lds_copy64x16(stage_addr + (uint32_t)(A_BYTES + (4 * j + w) * 1024), L.b_off[j] + b_k, rs_src);
+                lds_copy64x16(stage_addr + (uint32_t)(A_BYTES + (NW * j + w) * 1024), L.b_off[j] + b_k, rs_src);
             }
         } else {
             const KEntry k = tab[L.kc0 + (slot_of(w, lane) >> 1)];  // this lane's k-chunk: channel block and tap
@@ -147,7 +149,7 @@ struct DmaKernel {
             for (int j = 0; j < UB; ++j) {
                 const int ih = L.ih0[j] + fh, iw = L.iw0[j] + fw;
                 const bool ok = (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
-                lds_copy64x16(stage_addr + (uint32_t)(A_BYTES + (4 * j + w) * 1024), ok ? L.b_off[j] + k.off : SENT, rs_src);
+                lds_copy64x16(stage_addr + (uint32_t)(A_BYTES + (NW * j + w) * 1024), ok ? L.b_off[j] + k.off : SENT, rs_src);
             }
         }
     }
@@ -202,7 +204,7 @@ struct DmaKernel {
 
         if (!PW) {
             const int cap = a.nstages * KCH;
-            for (int e = t; e < cap; e += IG_THREADS) {
+            for (int e = t; e < cap; e += THREADS) {
                 KEntry k;
                 if (e < a.entries) {
                     const uint32_t cb = fdiv(e, a.div_t), tap = e - cb * a.T;
@@ -342,7 +344,7 @@ struct DmaKernel {
 };
 
 template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW>
-__global__ __launch_bounds__(IG_THREADS, MINW) void igemm_dma_kernel(IgemmArgs a) {
+__global__ __launch_bounds__(WM * WN * 64, MINW) void igemm_dma_kernel(IgemmArgs a) {
     DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW>::run(a);
 }
 
@@ -366,6 +368,11 @@ const DmaCfg kDma[] = {
         {"dma128x64x128r2", 128, 64, 4},
         {"dma64x64x128r4", 64, 64, 4},
         {"dma64x128x128r2", 64, 128, 4},
+        {"dma128x128x64w8", 128, 128, 2},
+        {"dma128x64x128w8", 128, 64, 4},
+        {"dma256x128x64w8", 256, 128, 2},
+        {"dma128x128x128r2w8", 128, 128, 4},
+        {"dma64x128x128w8", 64, 128, 4},
 };
 constexpr int kNumDma = sizeof(kDma) / sizeof(kDma[0]);
 
@@ -393,7 +400,7 @@ int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
     int occ = occ_val;
     if (occ_lds != lds) {
         hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(kern),
-                                                                    IG_THREADS, (size_t)lds);
+                                                                    K::THREADS, (size_t)lds);
         if (e != hipSuccess || occ < 1) {
             (void)hipGetLastError();
             occ = 1;
@@ -405,7 +412,7 @@ int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
     int64_t grid = (int64_t)occ * cu_count;
     if (grid > tiles) grid = tiles;
     if (grid >= 8) grid &= ~(int64_t)7;
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(IG_THREADS), lds, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(K::THREADS), lds, st, a);
     return (int)hipGetLastError();
 }
 
@@ -433,6 +440,11 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
         case 11: return launch_one<POUT, 128, 64, 2, 2, 4, 2, 2>(st, a, cu);
         case 12: return launch_one<POUT, 64, 64, 2, 2, 4, 4, 3>(st, a, cu);
         case 13: return launch_one<POUT, 64, 128, 2, 2, 4, 2, 2>(st, a, cu);
+        case 14: return launch_one<POUT, 128, 128, 2, 4, 2, 3, 2>(st, a, cu);
+        case 15: return launch_one<POUT, 128, 64, 4, 2, 4, 3, 2>(st, a, cu);
+        case 16: return launch_one<POUT, 256, 128, 4, 2, 2, 3, 1>(st, a, cu);
+        case 17: return launch_one<POUT, 128, 128, 2, 4, 4, 2, 2>(st, a, cu);
+        case 18: return launch_one<POUT, 64, 128, 2, 4, 4, 3, 2>(st, a, cu);
         default: return (int)hipErrorInvalidValue;
     }
 }
