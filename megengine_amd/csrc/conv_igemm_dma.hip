@@ -264,6 +264,11 @@ struct DmaKernel {
             // stage `it` of this wave has landed once at most the NS - 2 younger stages are in flight
             wait_vmcnt<(NS - 2) * U>();
             __syncthreads();  // ... of every wave; and every wave is done reading the buffer refilled next
+            // the residual of a tile is requested at the start of its last stage -- before this iteration's copies, so
+            // that waiting for it in the epilogue does not also wait for them
+            const bool last_stage = c_stage + 1 == a.nstages;
+            ZRegs<MT, NT> zr;
+            if (last_stage && a.epi.has_z) igemm_load_z<POUT, MT, NT>(a, zr, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh);
             issue(a, L, tab, rs_src, rs_flt, lds0 + (uint32_t)(wr * STG), wave, lane);
             advance();
 
@@ -271,7 +276,6 @@ struct DmaKernel {
                 init_acc(acc, sBias + c_par * BM, wm, lh);
                 if (DUAL) alt = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
             }
-            const bool last_stage = c_stage + 1 == a.nstages;
             int n_oc0 = c_oc0, n_pix0 = c_pix0;
             if (last_stage && it + 1 < total) {
                 tile_coords(a, c_tile + step, n_oc0, n_pix0);
@@ -323,7 +327,7 @@ struct DmaKernel {
 
             if (last_stage) {
                 if (DUAL) acc[0][0] += alt;
-                igemm_run_epilogue<POUT, MT, NT>(a, acc, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh);
+                igemm_run_epilogue<POUT, MT, NT, true>(a, acc, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh, &zr);
                 c_stage = 0;
                 c_tile += step;
                 if (a.tiles_m > 1) {

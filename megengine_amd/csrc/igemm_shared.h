@@ -63,9 +63,46 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 
 constexpr int SENT = (int)0x80000000;  // byte offset that is out of range for every buffer (< 2 GiB)
 
-template <int POUT, int MT, int NT, int NL, bool HZ>
-__device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w, int l32,
-                                           int lh) {
+// Residual (z) of one wave tile in the order the epilogue consumes it: POUT = 32: one 16-byte vector per 32x32 block
+// (16 consecutive channels of the lane's pixel); POUT = 4: four dwords per block.
+template <int MT, int NT>
+struct ZRegs {
+    v4i v[MT][NT];
+};
+
+// Fetches the whole wave tile's residual at once, so that a caller can issue it ahead of the epilogue
+template <int POUT, int MT, int NT>
+__device__ __forceinline__ void igemm_load_z(const IgemmArgs& a, ZRegs<MT, NT>& zr, int oc_w, int pix_w, int l32, int lh) {
+    const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(a.z, a.z_bytes);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int m = pix_w + j * 32 + l32;
+        const bool pok = m < a.M;
+        const uint32_t mm = pok ? m : 0;
+        const uint32_t n = fdiv(mm, a.div_ohw), rem = mm - n * a.OHW;
+        const int z_pix = (int)n * a.z_sn + (int)rem * POUT;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int ocb = oc_w + i * 32;
+            if (POUT == 32) {
+                const int blk_off = (ocb >> 5) * a.dst_scb + lh * 16;
+                zr.v[i][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_z, (pok && ocb < a.OC) ? z_pix + blk_off : SENT, 0, 0);
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int oc4 = ocb + 8 * q + 4 * lh;
+                    const int off = (oc4 >> 2) * a.dst_scb;
+                    zr.v[i][j][q] = __builtin_amdgcn_raw_buffer_load_b32(rs_z, (pok && oc4 < a.OC) ? z_pix + off : SENT, 0, 0);
+                }
+            }
+        }
+    }
+}
+
+// ZPRE: the residual was fetched by igemm_load_z into *zr; otherwise it is loaded here, block by block
+template <int POUT, int MT, int NT, int NL, bool HZ, bool ZPRE>
+__device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], const ZRegs<MT, NT>* zr, int oc_w,
+                                               int pix_w, int l32, int lh) {
     const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(a.z, HZ ? a.z_bytes : 0);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
@@ -84,7 +121,11 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
                 const int blk_off = (ocb >> 5) * a.dst_scb + lh * 16;
                 uint32_t zq[4] = {0, 0, 0, 0};
                 if (HZ) {
-                    v4i zv = __builtin_amdgcn_raw_buffer_load_b128(rs_z, pok ? z_pix + blk_off : -1, 0, 0);
+                    v4i zv;
+                    if (ZPRE)
+                        zv = zr->v[i][j];
+                    else
+                        zv = __builtin_amdgcn_raw_buffer_load_b128(rs_z, pok ? z_pix + blk_off : -1, 0, 0);
                     // stored order (16 consecutive channels per lane) -> accumulator order
                     auto s0 = __builtin_amdgcn_permlane32_swap((uint32_t)zv[0], (uint32_t)zv[1], false, false);
                     auto s1 = __builtin_amdgcn_permlane32_swap((uint32_t)zv[2], (uint32_t)zv[3], false, false);
@@ -106,7 +147,8 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
                     const bool ok = pok && oc4 < a.OC;
                     const int off = (oc4 >> 2) * a.dst_scb;
                     uint32_t zw = 0;
-                    if (HZ) zw = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_z, ok ? z_pix + off : -1, 0, 0);
+                    if (HZ) zw = ZPRE ? (uint32_t)zr->v[i][j][q]
+                                      : (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_z, ok ? z_pix + off : -1, 0, 0);
                     uint32_t o = requant4_fast<NL, HZ>(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], zw, a.epi);
                     if (ok) *reinterpret_cast<uint32_t*>(a.dst + d_pix + off) = o;
                 }
@@ -116,20 +158,20 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
 }
 
 // Fused requantisation + store of one wave tile (MT x NT blocks of 32 channels x 32 pixels).
-template <int POUT, int MT, int NT>
+template <int POUT, int MT, int NT, bool ZPRE = false>
 __device__ __forceinline__ void igemm_run_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w, int l32,
-                                               int lh) {
+                                                   int lh, const ZRegs<MT, NT>* zr = nullptr) {
     if (a.epi.has_z) {
         switch (a.epi.nonline) {
-            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, true>(a, acc, oc_w, pix_w, l32, lh); break;
-            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, true>(a, acc, oc_w, pix_w, l32, lh); break;
-            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, true>(a, acc, oc_w, pix_w, l32, lh); break;
+            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
+            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
+            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
         }
     } else {
         switch (a.epi.nonline) {
-            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, false>(a, acc, oc_w, pix_w, l32, lh); break;
-            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, false>(a, acc, oc_w, pix_w, l32, lh); break;
-            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, false>(a, acc, oc_w, pix_w, l32, lh); break;
+            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
+            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
+            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
         }
     }
 }
