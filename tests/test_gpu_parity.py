@@ -206,3 +206,35 @@ def test_heuristic_picks(oracle):
     assert ops.conv_bias_query(d)[0].id == DW
     d = _abi.make_conv_desc("NCHW32", 1, 64, 8, 8, 64, 3, pad=1, group=2)
     assert ops.conv_bias_query(d)[0].id == DIRECT
+
+
+# ---------------------------------------------------------------------------------------------
+# every tile configuration (register-staged and LDS-direct, 4- and 8-wave) on ragged shapes
+# ---------------------------------------------------------------------------------------------
+
+RAGGED = [
+    # fmt, n, ic, ih, iw, oc, f, stride, pad, nonline, z, extra
+    ("NCHW32", 3, 96, 9, 11, 96, 3, 1, 1, "RELU", True, {}),             # pixels % 32 != 0, oc % 64 != 0, K = 864
+    ("NCHW32", 2, 160, 7, 7, 32, 1, 1, 0, "IDENTITY", False, {}),        # pointwise, K = 160: not a multiple of a stage
+    ("NCHW32", 2, 256, 10, 10, 160, 1, 2, 0, "H_SWISH", True, {}),       # strided pointwise fast path
+    ("NCHW32", 1, 64, 13, 5, 224, 5, 2, 2, "RELU", False, {}),           # 5x5 stride 2, one image
+    ("NCHW32_NCHW4", 2, 64, 8, 8, 40, 3, 1, 1, "RELU", False, {}),       # 32-packed in, 4-packed out, oc % 32 != 0
+    ("NCHW32", 4, 128, 6, 6, 64, 3, 1, 0, "RELU", True, {"batch_pad": 64}),  # batch-strided src / dst / z views
+    ("NCHW4", 2, 24, 9, 9, 48, 3, 1, 1, "RELU", True, {}),               # 4-packed: LDS-direct ids fall back
+]
+
+
+@pytest.mark.parametrize("i", range(len(RAGGED)))
+def test_every_tile_on_ragged_shapes(oracle, i):
+    fmt, n, ic, ih, iw, oc, f, stride, pad, nl, z, extra = RAGGED[i]
+    kw = dict(S)
+    d0 = _abi.make_conv_desc(fmt, n, ic, ih, iw, oc, f, stride=stride, pad=pad, nonline=nl, has_z=z, **kw)
+    if extra.get("batch_pad"):
+        ss, fs, bs, ds = _abi.conv_shapes(d0)
+        per_src = int(np.prod(ss[1:])) + extra["batch_pad"]
+        per_dst = int(np.prod(ds[1:])) + extra["batch_pad"]
+        kw.update(src_stride_n=per_src, dst_stride_n=per_dst, z_stride_n=per_dst)
+    d = _abi.make_conv_desc(fmt, n, ic, ih, iw, oc, f, stride=stride, pad=pad, nonline=nl, has_z=z, **kw)
+    from megengine_amd import lib
+    for tile in range(len(lib.tile_names())):
+        check_case(oracle, d, seed=400 + i, algo=IGEMM, tile=tile, tag="ragged%d/%s" % (i, lib.tile_names()[tile]))
