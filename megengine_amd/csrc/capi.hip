@@ -136,22 +136,25 @@ int cu_count() {
     return g_dev[dev].cu;
 }
 
-const char* kAlgoNames[ALGO_COUNT] = {"MI355_DIRECT_DOT4", "MI355_IGEMM_MFMA_I8", "MI355_DEPTHWISE_DOT4"};
+const char* kAlgoNames[ALGO_COUNT] = {"MI355_DIRECT_DOT4", "MI355_IGEMM_MFMA_I8", "MI355_DEPTHWISE_DOT4",
+                                      "MI355_C4_MFMA_I8"};
 
 bool algo_usable(const ConvProblem& p, int id) {
     switch (id) {
         case ALGO_DIRECT: return true;
         case ALGO_IGEMM_MFMA: return igemm_usable(p);
         case ALGO_DEPTHWISE: return depthwise_usable(p);
+        case ALGO_C4_MFMA: return c4_usable(p);
         default: return false;
     }
 }
 
 // Heuristic order (cf. the reference's per-backend get_algorithm_heuristic, e.g.
-// dnn/src/cuda/conv_bias/opr_impl.cpp:44-238): channel-wise kernel, then the MFMA implicit GEMM,
-// then the generic direct kernel.
+// dnn/src/cuda/conv_bias/opr_impl.cpp:44-238): channel-wise kernel, the 4-channel first-layer kernel,
+// then the MFMA implicit GEMM, then the generic direct kernel.
 int pick_algo(const ConvProblem& p) {
     if (depthwise_usable(p)) return ALGO_DEPTHWISE;
+    if (c4_usable(p)) return ALGO_C4_MFMA;
     if (igemm_usable(p)) return ALGO_IGEMM_MFMA;
     return ALGO_DIRECT;
 }
@@ -288,6 +291,9 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
             break;
         case ALGO_DEPTHWISE:
             rc = launch_conv_depthwise(hs, p, src, filter, bias, z, reinterpret_cast<int8_t*>(dst));
+            break;
+        case ALGO_C4_MFMA:
+            rc = launch_conv_c4(hs, p, cu_count(), src, filter, bias, z, reinterpret_cast<int8_t*>(dst));
             break;
     }
     if (rc) return fail(MI355_ERR_LAUNCH, "%s: %s", kAlgoNames[id], hipGetErrorString((hipError_t)rc));

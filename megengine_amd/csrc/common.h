@@ -14,7 +14,8 @@ enum AlgoId {
     ALGO_DIRECT = 0,       // generic one-thread-per-output kernel: every format / mode
     ALGO_IGEMM_MFMA = 1,   // dense implicit GEMM on int8 MFMA (NCHW4 / NCHW32 / mixed)
     ALGO_DEPTHWISE = 2,    // channel-wise, bandwidth bound (NCHW4-packed and NCHW)
-    ALGO_COUNT = 3
+    ALGO_C4_MFMA = 3,      // first layers: NCHW4 with 4 input channels, patch-staged MFMA
+    ALGO_COUNT = 4
 };
 
 // Canonical problem description used by every launcher (derived from mi355_conv_desc)
@@ -43,6 +44,10 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int tile_cfg, int cu
 bool depthwise_usable(const ConvProblem& p);
 int launch_conv_depthwise(hipStream_t st, const ConvProblem& p, const int8_t* src, const int8_t* flt,
                           const int32_t* bias, const int8_t* z, int8_t* dst);
+
+bool c4_usable(const ConvProblem& p);
+int launch_conv_c4(hipStream_t st, const ConvProblem& p, int cu_count, const int8_t* src, const int8_t* flt,
+                   const int32_t* bias, const int8_t* z, int8_t* dst);
 
 int launch_relayout(hipStream_t st, const mi355_relayout_desc& d, const uint32_t* oshape, uint32_t ondim,
                     const void* src, void* dst, bool allow_fast);

@@ -15,7 +15,7 @@ from tests.gpu_util import say
 
 pytestmark = pytest.mark.gpu
 
-DIRECT, IGEMM, DW = 0, 1, 2
+DIRECT, IGEMM, DW, C4 = 0, 1, 2, 3
 
 
 def dev_tensors(d, seed):
@@ -65,11 +65,11 @@ def test_igemm_full_size(oracle, case):
     say("full-size", case)
     src, flt, bias, zt = dev_tensors(d, 17)
     algo, _ = ops.conv_bias_query(d)
-    assert algo.id == IGEMM
+    assert algo.id == (C4 if ic == 4 else IGEMM)   # 4-channel first layers have their own kernel
     got = ops.conv_bias_exec(d, src, flt, bias, zt, algo=algo)
     torch.cuda.synchronize()
     spot_check(oracle, d, src, flt, bias, zt, got)
-    say("  heuristic tile", lib.tile_names()[algo.tile_cfg], "spot check ok; comparing with the direct kernel")
+    say("  heuristic", lib.algo_names()[algo.id], lib.tile_names()[algo.tile_cfg], "spot check ok; comparing with the direct kernel")
     ref = ops.conv_bias_exec(d, src, flt, bias, zt, algo=DIRECT)
     torch.cuda.synchronize()
     assert torch.equal(got, ref)

@@ -10,7 +10,7 @@ from tests.gpu_util import check_case, run_gpu, say, to_dev
 
 pytestmark = pytest.mark.gpu
 
-DIRECT, IGEMM, DW = 0, 1, 2
+DIRECT, IGEMM, DW, C4 = 0, 1, 2, 3
 S = dict(scale_bias=2e-4, scale_z=0.05, scale_dst=0.05)
 
 
@@ -238,3 +238,37 @@ def test_every_tile_on_ragged_shapes(oracle, i):
     from megengine_amd import lib
     for tile in range(len(lib.tile_names())):
         check_case(oracle, d, seed=400 + i, algo=IGEMM, tile=tile, tag="ragged%d/%s" % (i, lib.tile_names()[tile]))
+
+
+# ---------------------------------------------------------------------------------------------
+# first-layer kernel: NCHW4 with 4 input channels, the patch-staged MFMA path
+# ---------------------------------------------------------------------------------------------
+
+C4_CASES = [
+    # n, ih, iw, oc, fh, fw, stride, pad
+    (2, 30, 30, 64, 7, 7, 2, 3),      # ResNet stem family
+    (1, 33, 29, 32, 7, 7, 2, 3),      # odd sizes: ragged tiles in both directions, half a channel tile
+    (2, 17, 40, 96, 3, 3, 2, 1),      # 3x3 stride 2 stem, two channel tiles (oc % 64 != 0)
+    (1, 20, 20, 24, 3, 3, 1, 1),      # stride 1, oc % 32 != 0
+    (3, 9, 9, 16, 5, 3, 1, 2),        # non-square filter, padding wider than the filter radius
+    (1, 12, 50, 128, 1, 1, 1, 0),     # pointwise
+    (2, 16, 16, 40, 8, 8, 2, 0),      # largest supported filter, no padding
+]
+
+
+@pytest.mark.parametrize("i", range(len(C4_CASES)))
+def test_first_layer_kernel(oracle, i):
+    n, ih, iw, oc, fh, fw, stride, pad = C4_CASES[i]
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        for has_z in (False, True):
+            d = _abi.make_conv_desc("NCHW4", n, 4, ih, iw, oc, fh, fw, stride=stride, pad=pad, nonline=nl, has_z=has_z, **S)
+            a, _ = ops.conv_bias_query(d)
+            assert a.id == C4
+            check_case(oracle, d, seed=500 + i, tag="c4-%d" % i)
+    # no bias, batch-strided views
+    d0 = _abi.make_conv_desc("NCHW4", n, 4, ih, iw, oc, fh, fw, stride=stride, pad=pad, nonline="RELU", has_z=True, **S)
+    ss, fs, bs, ds = _abi.conv_shapes(d0)
+    d = _abi.make_conv_desc("NCHW4", n, 4, ih, iw, oc, fh, fw, stride=stride, pad=pad, nonline="RELU", has_z=True,
+                            bias_mode=_abi.BIAS_NONE, src_stride_n=int(np.prod(ss[1:])) + 20,
+                            dst_stride_n=int(np.prod(ds[1:])) + 12, z_stride_n=int(np.prod(ds[1:])) + 36, **S)
+    check_case(oracle, d, seed=600 + i, tag="c4-%d-strided" % i)
