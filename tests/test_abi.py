@@ -39,7 +39,7 @@ def test_status_strings():
 
 def test_algorithm_table():
     names = lib.algo_names()
-    assert names == ["MI355_DIRECT_DOT4", "MI355_IGEMM_MFMA_I8", "MI355_DEPTHWISE_DOT4"]
+    assert names == ["MI355_DIRECT_DOT4", "MI355_IGEMM_MFMA_I8", "MI355_DEPTHWISE_DOT4", "MI355_C4_MFMA_I8"]
     assert lib.lib().mi355_convbias_algo_name(17) is None
     assert len(lib.tile_names()) >= 3
 
