@@ -198,13 +198,13 @@ def main():
                           algo=lib.algo_names()[p["algo"].id], tile=lib.tile_names()[p["algo"].tile_cfg],
                           us=round(ms * 1e3, 2), tops=round(l.ops / t / 1e12, 1), gbs=round(l.bytes / t / 1e9, 1),
                           frac_roof=round(roof / t, 3)))
-    # dominant kernel = the implicit-GEMM kernel (all 53 launches).  Average launch duration = the
+    # dominant kernels = the MFMA ConvBias kernels (all 53 launches).  Average launch duration = the
     # timed region of K steps (two HIP events on the launch stream) / (K * 53): the launches run
     # back to back, so this is the kernel duration plus the sub-microsecond gap between launches.
     t_launch = ms_per_step * 1e-3 / nl
     roofline = dict(bound="hbm", achieved=round(tot_bytes / nl / t_launch / 1e9, 1), peak=HBM_PEAK / 1e9,
                     unit="GB/s", frac=round(tot_bytes / nl / t_launch / HBM_PEAK, 4), traffic=None,
-                    kernel="igemm_kernel (MI355_IGEMM_MFMA_I8), 53 launches per step",
+                    kernel="ConvBias MFMA kernels (igemm_dma_kernel, igemm_kernel, c4_kernel), 53 launches per step",
                     bytes_per_launch=round(tot_bytes / nl), avg_launch_us=round(t_launch * 1e6, 2),
                     per_launch_event_sum_ms=round(kern_ms, 4),
                     mfma_tops=round(tot_ops / (ms_per_step * 1e-3) / 1e12, 1),
