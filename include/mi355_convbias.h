@@ -20,6 +20,11 @@
  *                                 (dnn/src/naive/conv_bias/opr_impl.cpp:211-292)
  *   mi355_convbias_algo_*      <- MultiAlgoOpr::get_all_algorithms / Algorithm::name
  *                                 (dnn/include/megdnn/oprs/base.h:545-615)
+ *   mi355_requant_s32_s8_exec  <- the ConvBias post-process as its own pass, handle_z_inp_and_activation_naive
+ *                                 (dnn/src/naive/conv_bias/opr_impl.cpp:21-98); without z that is the unary
+ *                                 ElemwiseMultiType Q<mode> s32 -> s8 (dnn/src/naive/elemwise_multi_type/
+ *                                 opr_impl.h:47-68, opr_impl_3.cpp:12-59) or TypeCvt s32 -> s8
+ *                                 (dnn/src/naive/type_cvt/opr_impl.cpp:24-56)
  *   mi355_relayout_exec        <- RelayoutFormat::exec (dnn/include/megdnn/oprs/general.h:1353-1359),
  *                                 arithmetic of naive::RelayoutFormatImpl::exec
  *                                 (dnn/src/naive/relayout_format/opr_impl.cpp:486-773)
@@ -185,6 +190,24 @@ typedef struct mi355_relayout_desc {
 /* dst shape for the descriptor (dnn/src/common/relayout_format.cpp:7-296) */
 int mi355_relayout_deduce(const mi355_relayout_desc* d, uint32_t* ndim, uint32_t shape[7]);
 int mi355_relayout_exec(void* stream, const mi355_relayout_desc* d, const void* src, void* dst);
+
+/* ---- stand-alone requantisation: dst[i] = quantize_s8(act(dequant_s32(src[i]) [+ dequant_s8(z[i])]), scale_dst) ----
+ * The reference runs this as a separate pass over a QuantizedS32 convolution result
+ * (handle_z_inp_and_activation_naive, naive/conv_bias/opr_impl.cpp:21-98), and a graph that keeps a convolution with
+ * dst_dtype QuantizedS32 apart from its activation runs the same arithmetic as operators of its own: the unary
+ * ElemwiseMultiType quantized modes QRELU / QH_SWISH from QuantizedS32 to QuantizedS8 (has_z = 0), and TypeCvt
+ * QuantizedS32 -> QuantizedS8 (nonline IDENTITY, has_z = 0).  With has_z the chain is the post-process's own
+ * TypeCvt -> float ADD -> activation -> TypeCvt.  Tensors are contiguous; src and dst need 16- and 4-byte alignment. */
+typedef struct mi355_requant_desc {
+    uint32_t nonline;   /* MI355_NL_* (no SIGMOID) */
+    uint32_t has_z;
+    float scale_src;    /* scale of the QuantizedS32 input */
+    float scale_z;      /* scale of the QuantizedS8 second input */
+    float scale_dst;
+    uint32_t reserved;
+    uint64_t count;     /* elements */
+} mi355_requant_desc;
+int mi355_requant_s32_s8_exec(void* stream, const mi355_requant_desc* d, const int32_t* src, const int8_t* z, int8_t* dst);
 
 #ifdef __cplusplus
 }

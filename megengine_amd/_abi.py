@@ -74,6 +74,13 @@ class RelayoutDesc(C.Structure):
     ]
 
 
+class RequantDesc(C.Structure):
+    _fields_ = [
+        ("nonline", C.c_uint32), ("has_z", C.c_uint32), ("scale_src", C.c_float), ("scale_z", C.c_float),
+        ("scale_dst", C.c_float), ("reserved", C.c_uint32), ("count", C.c_uint64),
+    ]
+
+
 def in_pack(fmt):
     return {FMT_NCHW: 1, FMT_NCHW4: 4, FMT_NCHW44: 4, FMT_NCHW4_NCHW32: 4}.get(fmt, 32)
 

@@ -16,7 +16,8 @@
 //       q  = fma(e, y_hi, q0)            correctly rounded r / s_dst (Markstein's correction step)
 //   * RELU is folded into the clamp: for s_dst > 0, r <= 0 gives q <= 0 which clamps to 0.
 //   * roundf + clamp + convert: clamp first, then trunc(q + copysign(pred(0.5), q)); for
-//     |q| <= 128 the sum is exact except below 0.5 where pred(0.5) keeps it under 1.
+//     |q| <= 128 the sum is exact except below 0.5 where pred(0.5) keeps it under 1.  After a RELU
+//     clamp q >= 0 and the hardware's round-to-plus-infinity conversion does the same in one step.
 // The host only selects the fast form when the scales are positive, normal and small enough
 // that no intermediate overflows (see epi_fast_ok in capi.hip); otherwise kernels run the
 // literal form with the IEEE divide.
@@ -95,7 +96,10 @@ __device__ __forceinline__ int requant_s8_fast(int sfb, int z, const EpiParams& 
     int out;
     if (NL == NL_RELU) {
         q = __builtin_amdgcn_fmed3f(q, 0.f, 127.f);  // q is finite here: same as min(max(q, 0), 127)
-        out = (int)(q + 0.49999997f);
+        // floor(q + 0.5) computed exactly by the hardware (round to nearest, ties to +infinity): for q >= 0 that is
+        // round-half-away, one instruction instead of add + truncate.  Equal to (int)(q + 0.49999997f) on every
+        // float in [0, 127] (checked exhaustively on gfx950).
+        asm("v_cvt_rpi_i32_f32 %0, %1" : "=v"(out) : "v"(q));
     } else {
         q = __builtin_amdgcn_fmed3f(q, -128.f, 127.f);
         out = (int)(q + __builtin_copysignf(0.49999997f, q));

@@ -1,0 +1,42 @@
+// Stand-alone requantisation QuantizedS32 (+ QuantizedS8) -> QuantizedS8 with the ConvBias epilogue arithmetic
+// (epilogue.h): the reference's post-process pass, unary quantized ElemwiseMultiType modes and TypeCvt s32 -> s8.  Pure streaming:
+// 16 bytes in (+ 4), 4 bytes out per thread step; bound by HBM (5-6 bytes per element) and by the ~10 VALU operations
+// per element of the bit-exact requantisation.
+#include "common.h"
+
+namespace mi355 {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void requant_kernel(const int32_t* __restrict__ src, const int8_t* __restrict__ z,
+                                                      int8_t* __restrict__ dst, uint64_t quads, uint64_t count, EpiParams e) {
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < quads; i += stride) {
+        const v4i a = reinterpret_cast<const v4i*>(src)[i];
+        const uint32_t zw = e.has_z ? reinterpret_cast<const uint32_t*>(z)[i] : 0u;
+        reinterpret_cast<uint32_t*>(dst)[i] = requant4(a[0], a[1], a[2], a[3], zw, e);
+    }
+    // ragged tail (count % 4 elements), one thread
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        for (uint64_t j = quads * 4; j < count; ++j)
+            dst[j] = (int8_t)requant_s8_exact(src[j], e.has_z != 0, e.has_z ? (int)z[j] : 0, e);
+    }
+}
+
+}  // namespace
+
+int launch_requant(hipStream_t st, const EpiParams& e, const int32_t* src, const int8_t* z, int8_t* dst, uint64_t count,
+                   int cu_count) {
+    if (count == 0) return 0;
+    const uint64_t quads = count / 4;
+    if (cu_count <= 0) cu_count = 256;
+    uint64_t blocks = (quads + 255) / 256;
+    const uint64_t cap = (uint64_t)cu_count * 16;
+    if (blocks > cap) blocks = cap;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(requant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, src, z, dst, quads, count, e);
+    return (int)hipGetLastError();
+}
+
+}  // namespace mi355

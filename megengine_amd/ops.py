@@ -8,7 +8,8 @@ The calls mirror megdnn::ConvBiasForward (dnn/include/megdnn/oprs/nn.h:358-536):
     get_workspace_in_bytes   -> conv_bias_workspace(desc, algo)
     get_algorithm_heuristic  -> conv_bias_query(desc)
     exec(src, filter, bias, z, dst, workspace) -> conv_bias_exec(...)
-and megdnn::RelayoutFormat (dnn/include/megdnn/oprs/general.h:1348-1373).
+and megdnn::RelayoutFormat (dnn/include/megdnn/oprs/general.h:1348-1373); requant_exec is the unfused
+epilogue (the reference's post-process pass; unary ElemwiseMultiType quantized modes and TypeCvt s32 -> s8).
 """
 import ctypes as C
 
@@ -110,4 +111,18 @@ def relayout_exec(d, src, dst=None):
     if dst is None:
         dst = torch.empty(relayout_deduce_layout(d), dtype=src.dtype, device=src.device)
     check(lib().mi355_relayout_exec(_stream(), C.byref(d), _ptr(src), _ptr(dst)))
+    return dst
+
+
+def requant_exec(src, scale_src, scale_dst, nonline="IDENTITY", z=None, scale_z=1.0, dst=None):
+    """QuantizedS32 (+ QuantizedS8 z) -> QuantizedS8 with the ConvBias epilogue arithmetic."""
+    nl = nonline if isinstance(nonline, int) else {"IDENTITY": _abi.NL_IDENTITY, "RELU": _abi.NL_RELU,
+                                                    "H_SWISH": _abi.NL_H_SWISH, "SIGMOID": 2}[nonline]
+    if src.dtype != torch.int32:
+        raise RuntimeError("requant_exec takes an int32 tensor")
+    if dst is None:
+        dst = torch.empty(src.shape, dtype=torch.int8, device=src.device)
+    d = _abi.RequantDesc(nonline=nl, has_z=int(z is not None), scale_src=scale_src, scale_z=scale_z, scale_dst=scale_dst,
+                         count=src.numel())
+    check(lib().mi355_requant_s32_s8_exec(_stream(), C.byref(d), _ptr(src), _ptr(z), _ptr(dst)))
     return dst

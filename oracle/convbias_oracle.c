@@ -88,6 +88,20 @@ int32_t oracle_epilogue_s32(int32_t sfb, float s_bias, int has_z, int32_t z, flo
     return oracle_quantize_s32(oracle_epilogue_float(sfb, s_bias, has_z, zf, nonline), s_dst);
 }
 
+/* The post-process as a stand-alone pass over n elements (handle_z_inp_and_activation_naive,
+ * naive/conv_bias/opr_impl.cpp:21-98); without z it is the unary ElemwiseMultiType Q<mode> s32 -> s8
+ * (naive/elemwise_multi_type/opr_impl.h:47-68, opr_impl_3.cpp:12-59) or TypeCvt s32 -> s8
+ * (naive/type_cvt/opr_impl.cpp:24-56).  Same scalar chain as oracle_epilogue_s8. */
+int oracle_requant_s32_s8(const mi355_requant_desc* d, const int32_t* src, const int8_t* z, int8_t* dst) {
+    if (d->nonline == MI355_NL_SIGMOID || d->nonline > MI355_NL_H_SWISH) return MI355_ERR_UNSUPPORTED;
+    const int64_t n = (int64_t)d->count;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i)
+        dst[i] = oracle_epilogue_s8(src[i], d->scale_src, d->has_z != 0, d->has_z ? z[i] : 0, d->scale_z, (int)d->nonline,
+                                    d->scale_dst);
+    return MI355_OK;
+}
+
 /* infer_conv_shape, dnn/src/common/utils.cpp:130-138 */
 static uint32_t out_size(uint32_t i, uint32_t f, uint32_t d, uint32_t s, uint32_t p) {
     uint32_t df = (f - 1) * d + 1;

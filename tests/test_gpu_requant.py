@@ -1,0 +1,84 @@
+"""Stand-alone requantisation (the unfused ConvBias epilogue) against the CPU checker: dense sweeps of the int32 input
+through every rounding boundary, tie-heavy scale pairs, all activations, with and without the second input, plus
+scales that force the literal (IEEE divide) form.  The same arithmetic is the epilogue of every ConvBias kernel."""
+import numpy as np
+import pytest
+import torch
+
+from megengine_amd import _abi, ops
+from tests.gpu_util import say
+
+pytestmark = pytest.mark.gpu
+
+NL = {"IDENTITY": _abi.NL_IDENTITY, "RELU": _abi.NL_RELU, "H_SWISH": _abi.NL_H_SWISH}
+
+# (scale_src, scale_dst, scale_z): the first three make x * s_src / s_dst land exactly on .5 for every odd / every
+# fourth input; the others are "ordinary" float scales
+SCALES = [
+    (0.5, 1.0, 1.0),
+    (0.25, 2.0, 0.5),
+    (0.125, 0.25, 0.75),
+    (2e-4, 0.05, 0.05),
+    (float(np.float32(0.02) * np.float32(0.01)), 0.05, 0.04),
+    (1.3e-3, 0.0271, 0.113),
+    (7.7e-5, 3.3e-3, 1.9e-2),
+]
+
+
+def run_case(oracle, x, z, s_src, s_dst, s_z, nl):
+    xt = torch.from_numpy(x).cuda()
+    zt = None if z is None else torch.from_numpy(z).cuda()
+    got = ops.requant_exec(xt, s_src, s_dst, nonline=nl, z=zt, scale_z=s_z)
+    torch.cuda.synchronize()
+    want = oracle.requant(x, s_src, s_dst, NL[nl], z=z, scale_z=s_z)
+    g = got.cpu().numpy()
+    if not np.array_equal(g, want):
+        bad = np.nonzero(g != want)[0]
+        raise AssertionError("%d mismatches, first: x=%d z=%s got %d want %d (scales %r %r %r, %s)" % (
+            len(bad), x[bad[0]], None if z is None else z[bad[0]], g[bad[0]], want[bad[0]], s_src, s_dst, s_z, nl))
+
+
+@pytest.mark.parametrize("si", range(len(SCALES)))
+def test_dense_sweep_through_every_boundary(oracle, si):
+    s_src, s_dst, s_z = SCALES[si]
+    # inputs whose quotient covers [-140, 140]: every output value and both saturation edges, contiguous integers
+    span = int(min(2 ** 23, 140.0 * s_dst / s_src))
+    x = np.arange(-span, span + 1, dtype=np.int32)
+    if x.size > (1 << 22):   # thin out very long ranges but keep a contiguous window around each boundary
+        step = x.size // (1 << 22) + 1
+        x = np.unique(np.concatenate([x[::step], np.arange(-4096, 4097, dtype=np.int32)]))
+    rng = np.random.RandomState(si)
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        say("requant sweep", SCALES[si], nl, x.size)
+        run_case(oracle, x, None, s_src, s_dst, s_z, nl)
+        z = rng.randint(-128, 128, x.size).astype(np.int8)
+        run_case(oracle, x, z, s_src, s_dst, s_z, nl)
+
+
+def test_full_range_inputs_and_tail(oracle):
+    rng = np.random.RandomState(9)
+    for n in (1, 3, 4, 5, 1023, 65537):     # count % 4 != 0: the scalar tail
+        x = rng.randint(-2 ** 31, 2 ** 31 - 1, n, dtype=np.int64).astype(np.int32)
+        z = rng.randint(-128, 128, n).astype(np.int8)
+        for nl in ("IDENTITY", "RELU", "H_SWISH"):
+            run_case(oracle, x, z, 3.1e-9, 0.043, 0.07, nl)
+            run_case(oracle, x, None, 1.0, 1.0, 1.0, nl)
+
+
+def test_literal_form_scales(oracle):
+    """scales outside the range of the divide-free form take the IEEE divide path"""
+    rng = np.random.RandomState(4)
+    x = rng.randint(-100000, 100000, 100003).astype(np.int32)
+    z = rng.randint(-128, 128, x.size).astype(np.int8)
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        run_case(oracle, x, z, 1e-20, 1e-17, 3e-16, nl)
+        run_case(oracle, x, None, 1e-20, 1e-17, 1.0, nl)
+
+
+def test_rejects_bad_arguments():
+    from megengine_amd.lib import Mi355Error
+    x = torch.zeros(16, dtype=torch.int32, device="cuda")
+    with pytest.raises(Mi355Error):
+        ops.requant_exec(x, 1.0, 1.0, nonline="SIGMOID")
+    with pytest.raises(Mi355Error):
+        ops.requant_exec(x[1:], 1.0, 1.0)     # misaligned int32 view

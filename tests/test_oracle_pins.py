@@ -378,3 +378,21 @@ def test_relayout_nchw32_extension_modes(oracle):
         assert np.array_equal(z4, _pack(_pack(x, 32).transpose(0, 1, 4, 2, 3).reshape(n, -1, h, w), 4))
         z4c = np.ascontiguousarray(z4[:, :-(-c // 4)])   # mode 25 crops inside the last 4-pack only
         assert np.array_equal(oracle.relayout(oracle.relayout_desc(_abi.RL_NCHW4_NCHW, z4c.shape, oc=c), z4c), x)
+
+
+def test_requant_operator_is_the_epilogue(oracle):
+    """The stand-alone requantisation of the checker is the scalar epilogue applied element by element, and with
+    integer scales it is plain integer arithmetic (round half away, saturate)."""
+    L = oracle.lib()
+    rng = np.random.RandomState(12)
+    x = rng.randint(-70000, 70000, 5000).astype(np.int32)
+    z = rng.randint(-128, 128, x.size).astype(np.int8)
+    for nl in (0, 1, 3):
+        got = oracle.requant(x, 2e-4, 0.05, nl, z=z, scale_z=0.07)
+        want = np.array([L.oracle_epilogue_s8(int(a), 2e-4, 1, int(b), 0.07, nl, 0.05) for a, b in zip(x, z)], np.int8)
+        assert np.array_equal(got, want)
+    xi = np.arange(-600, 601, dtype=np.int32)
+    got = oracle.requant(xi, 1.0, 4.0, 0)
+    q = xi.astype(np.int64)
+    want = np.clip(np.sign(q) * ((2 * np.abs(q) + 4) // 8), -128, 127).astype(np.int8)   # round-half-away of q / 4
+    assert np.array_equal(got, want)
