@@ -25,6 +25,8 @@
  *                                 ElemwiseMultiType Q<mode> s32 -> s8 (dnn/src/naive/elemwise_multi_type/
  *                                 opr_impl.h:47-68, opr_impl_3.cpp:12-59) or TypeCvt s32 -> s8
  *                                 (dnn/src/naive/type_cvt/opr_impl.cpp:24-56)
+ *   mi355_requant_s8_s8_exec   <- ElemwiseMultiType binary quantized modes on two QuantizedS8 tensors
+ *                                 (dnn/src/naive/elemwise_multi_type/opr_impl.h:88-116, opr_impl_4.cpp:11-60)
  *   mi355_relayout_exec        <- RelayoutFormat::exec (dnn/include/megdnn/oprs/general.h:1353-1359),
  *                                 arithmetic of naive::RelayoutFormatImpl::exec
  *                                 (dnn/src/naive/relayout_format/opr_impl.cpp:486-773)
@@ -208,6 +210,13 @@ typedef struct mi355_requant_desc {
     uint64_t count;     /* elements */
 } mi355_requant_desc;
 int mi355_requant_s32_s8_exec(void* stream, const mi355_requant_desc* d, const int32_t* src, const int8_t* z, int8_t* dst);
+/* The same with a QuantizedS8 first operand (scale_src is its scale): the binary quantized modes of ElemwiseMultiType
+ * on two QuantizedS8 tensors -- QADD (IDENTITY), QFUSE_ADD_RELU, QFUSE_ADD_H_SWISH: quantize(mode(dequantize(a),
+ * dequantize(b))), dnn/src/naive/elemwise_multi_type/opr_impl.h:88-116, opr_impl_4.cpp:11-60, kernels
+ * dnn/src/common/elemwise/kern_defs.cuh:52-55,:234,:268 -- and with has_z = 0 the unary QRELU / QH_SWISH and the
+ * rescaling TypeCvt QuantizedS8 -> QuantizedS8.  The residual add of a network whose fuser left it outside ConvBias.
+ * All three tensors need 16-byte alignment. */
+int mi355_requant_s8_s8_exec(void* stream, const mi355_requant_desc* d, const int8_t* src, const int8_t* z, int8_t* dst);
 
 #ifdef __cplusplus
 }

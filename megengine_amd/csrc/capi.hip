@@ -320,6 +320,26 @@ int mi355_requant_s32_s8_exec(void* stream, const mi355_requant_desc* d, const i
     return MI355_OK;
 }
 
+int mi355_requant_s8_s8_exec(void* stream, const mi355_requant_desc* d, const int8_t* src, const int8_t* z, int8_t* dst) {
+    if (!d) return fail(MI355_ERR_BAD_ARG, "null descriptor");
+    if (d->nonline == MI355_NL_SIGMOID || d->nonline > MI355_NL_H_SWISH)
+        return fail(MI355_ERR_UNSUPPORTED, "nonlinearity %u has no quantized definition", d->nonline);
+    if (d->count == 0) return MI355_OK;
+    if (!src || !dst) return fail(MI355_ERR_BAD_ARG, "null tensor pointer");
+    if (d->has_z && !z) return fail(MI355_ERR_BAD_ARG, "has_z set but z is null");
+    if (!aligned16(src) || !aligned16(dst) || (d->has_z && !aligned16(z)))
+        return fail(MI355_ERR_BAD_ARG, "src, z and dst need 16-byte alignment");
+    EpiParams e;
+    e.s_b = d->scale_src; e.s_z = d->scale_z; e.s_d = d->scale_dst;
+    e.nonline = (int)d->nonline; e.has_z = d->has_z != 0;
+    e.fast = epi_fast_ok(d->scale_src, d->scale_z, d->scale_dst, d->has_z != 0);
+    e.y_hi = 1.0f / d->scale_dst;
+    e.y_lo = (float)(1.0 / (double)d->scale_dst - (double)e.y_hi);
+    int rc = launch_requant8(reinterpret_cast<hipStream_t>(stream), e, src, z, dst, d->count, cu_count());
+    if (rc) return fail(MI355_ERR_LAUNCH, "requant: %s", hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
+}
+
 int mi355_igemm_tile_count(void) { return igemm_num_cfgs(); }
 const char* mi355_igemm_tile_name(int cfg) { return igemm_cfg_name(cfg); }
 

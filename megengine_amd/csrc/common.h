@@ -51,6 +51,8 @@ int launch_conv_c4(hipStream_t st, const ConvProblem& p, int cu_count, const int
 
 int launch_requant(hipStream_t st, const EpiParams& e, const int32_t* src, const int8_t* z, int8_t* dst, uint64_t count,
                    int cu_count);
+int launch_requant8(hipStream_t st, const EpiParams& e, const int8_t* src, const int8_t* z, int8_t* dst, uint64_t count,
+                    int cu_count);
 
 int launch_relayout(hipStream_t st, const mi355_relayout_desc& d, const uint32_t* oshape, uint32_t ondim,
                     const void* src, void* dst, bool allow_fast);

@@ -378,7 +378,7 @@ struct DmaKernel {
     // Nested schedule: per tile a steady loop whose refills stay inside the tile (the loader only steps along k: no
     // tile bookkeeping, a third of the scalar instructions of the flat loop) and the last NS stages, whose refills
     // cross into the next tile.  Used when every workgroup owns one tile and the reduction is long.
-    __device__ static __forceinline__ void run_lean(const IgemmArgs& a) {
+    __device__ static __forceinline__ void run_nested(const IgemmArgs& a) {
         extern __shared__ __attribute__((aligned(16))) int8_t lds[];
         KEntry* tab = reinterpret_cast<KEntry*>(lds + RING_BYTES);
         const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)lds);
@@ -566,7 +566,7 @@ struct DmaKernel {
 template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, bool NESTED>
 __global__ __launch_bounds__(WM * WN * 64, MINW) void igemm_dma_kernel(IgemmArgs a) {
     if (NESTED)
-        DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW>::run_lean(a);
+        DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW>::run_nested(a);
     else
         DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW>::run_flat(a);
 }

@@ -1,4 +1,4 @@
-// Stand-alone requantisation QuantizedS32 (+ QuantizedS8) -> QuantizedS8 with the ConvBias epilogue arithmetic
+// Stand-alone requantisation QuantizedS32 | QuantizedS8 (+ QuantizedS8) -> QuantizedS8 with the ConvBias epilogue arithmetic
 // (epilogue.h): the reference's post-process pass, unary quantized ElemwiseMultiType modes and TypeCvt s32 -> s8.  Pure streaming:
 // 16 bytes in (+ 4), 4 bytes out per thread step; bound by HBM (5-6 bytes per element) and by the ~10 VALU operations
 // per element of the bit-exact requantisation.
@@ -24,7 +24,42 @@ __global__ __launch_bounds__(256) void requant_kernel(const int32_t* __restrict_
     }
 }
 
+// QuantizedS8 first operand: 16 elements per thread step (16 + 16 bytes in, 16 out; 2-3 bytes per element)
+__global__ __launch_bounds__(256) void requant8_kernel(const int8_t* __restrict__ src, const int8_t* __restrict__ z,
+                                                       int8_t* __restrict__ dst, uint64_t blocks16, uint64_t count, EpiParams e) {
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < blocks16; i += stride) {
+        const v4i a = reinterpret_cast<const v4i*>(src)[i];
+        v4i zv = {0, 0, 0, 0};
+        if (e.has_z) zv = reinterpret_cast<const v4i*>(z)[i];
+        v4i o;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int w = a[q];
+            o[q] = (int)requant4((w << 24) >> 24, (w << 16) >> 24, (w << 8) >> 24, w >> 24, (uint32_t)zv[q], e);
+        }
+        reinterpret_cast<v4i*>(dst)[i] = o;
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        for (uint64_t j = blocks16 * 16; j < count; ++j)
+            dst[j] = (int8_t)requant_s8_exact((int)src[j], e.has_z != 0, e.has_z ? (int)z[j] : 0, e);
+    }
+}
+
 }  // namespace
+
+int launch_requant8(hipStream_t st, const EpiParams& e, const int8_t* src, const int8_t* z, int8_t* dst, uint64_t count,
+                    int cu_count) {
+    if (count == 0) return 0;
+    const uint64_t blocks16 = count / 16;
+    if (cu_count <= 0) cu_count = 256;
+    uint64_t blocks = (blocks16 + 255) / 256;
+    const uint64_t cap = (uint64_t)cu_count * 16;
+    if (blocks > cap) blocks = cap;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(requant8_kernel, dim3((unsigned)blocks), dim3(256), 0, st, src, z, dst, blocks16, count, e);
+    return (int)hipGetLastError();
+}
 
 int launch_requant(hipStream_t st, const EpiParams& e, const int32_t* src, const int8_t* z, int8_t* dst, uint64_t count,
                    int cu_count) {

@@ -115,14 +115,15 @@ def relayout_exec(d, src, dst=None):
 
 
 def requant_exec(src, scale_src, scale_dst, nonline="IDENTITY", z=None, scale_z=1.0, dst=None):
-    """QuantizedS32 (+ QuantizedS8 z) -> QuantizedS8 with the ConvBias epilogue arithmetic."""
+    """QuantizedS32 or QuantizedS8 (+ QuantizedS8 z) -> QuantizedS8 with the ConvBias epilogue arithmetic."""
     nl = nonline if isinstance(nonline, int) else {"IDENTITY": _abi.NL_IDENTITY, "RELU": _abi.NL_RELU,
                                                     "H_SWISH": _abi.NL_H_SWISH, "SIGMOID": 2}[nonline]
-    if src.dtype != torch.int32:
-        raise RuntimeError("requant_exec takes an int32 tensor")
+    if src.dtype not in (torch.int32, torch.int8):
+        raise RuntimeError("requant_exec takes an int32 or int8 tensor")
     if dst is None:
         dst = torch.empty(src.shape, dtype=torch.int8, device=src.device)
     d = _abi.RequantDesc(nonline=nl, has_z=int(z is not None), scale_src=scale_src, scale_z=scale_z, scale_dst=scale_dst,
                          count=src.numel())
-    check(lib().mi355_requant_s32_s8_exec(_stream(), C.byref(d), _ptr(src), _ptr(z), _ptr(dst)))
+    fn = lib().mi355_requant_s32_s8_exec if src.dtype == torch.int32 else lib().mi355_requant_s8_s8_exec
+    check(fn(_stream(), C.byref(d), _ptr(src), _ptr(z), _ptr(dst)))
     return dst

@@ -102,6 +102,20 @@ int oracle_requant_s32_s8(const mi355_requant_desc* d, const int32_t* src, const
     return MI355_OK;
 }
 
+/* Binary quantized ElemwiseMultiType modes on two QuantizedS8 tensors (ADD, FUSE_ADD_RELU, FUSE_ADD_H_SWISH) and the
+ * unary ones without z: dst = quantize(mode(dequantize(a), dequantize(b))), naive/elemwise_multi_type/opr_impl.h:88-116;
+ * the float kernels (common/elemwise/kern_defs.cuh:52-55 fuse_add_hswish, :234 ADD, :268 FUSE_ADD_RELU) are the
+ * activation chain of oracle_epilogue_s8 applied to dequantize(a) + dequantize(b). */
+int oracle_requant_s8_s8(const mi355_requant_desc* d, const int8_t* src, const int8_t* z, int8_t* dst) {
+    if (d->nonline == MI355_NL_SIGMOID || d->nonline > MI355_NL_H_SWISH) return MI355_ERR_UNSUPPORTED;
+    const int64_t n = (int64_t)d->count;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; ++i)
+        dst[i] = oracle_epilogue_s8((int32_t)src[i], d->scale_src, d->has_z != 0, d->has_z ? z[i] : 0, d->scale_z,
+                                    (int)d->nonline, d->scale_dst);
+    return MI355_OK;
+}
+
 /* infer_conv_shape, dnn/src/common/utils.cpp:130-138 */
 static uint32_t out_size(uint32_t i, uint32_t f, uint32_t d, uint32_t s, uint32_t p) {
     uint32_t df = (f - 1) * d + 1;

@@ -133,7 +133,17 @@ def relayout(d, src):
 
 
 def requant(src, scale_src, scale_dst, nonline=0, z=None, scale_z=1.0):
-    """int32 array (+ int8 z) -> int8 with the epilogue chain; nonline is the MI355_NL_* value"""
+    """int32 or int8 array (+ int8 z) -> int8 with the epilogue chain; nonline is the MI355_NL_* value"""
+    if np.asarray(src).dtype == np.int8:
+        src = np.ascontiguousarray(src)
+        d = _abi.RequantDesc(nonline=nonline, has_z=int(z is not None), scale_src=scale_src, scale_z=scale_z,
+                             scale_dst=scale_dst, count=src.size)
+        dst = np.empty(src.shape, np.int8)
+        zc = None if z is None else np.ascontiguousarray(z, dtype=np.int8)
+        st = lib().oracle_requant_s8_s8(C.byref(d), _ptr(src), _ptr(zc) if zc is not None else None, _ptr(dst))
+        if st:
+            raise OracleError(st)
+        return dst
     src = np.ascontiguousarray(src, dtype=np.int32)
     d = _abi.RequantDesc(nonline=nonline, has_z=int(z is not None), scale_src=scale_src, scale_z=scale_z,
                          scale_dst=scale_dst, count=src.size)

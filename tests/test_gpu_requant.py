@@ -82,3 +82,28 @@ def test_rejects_bad_arguments():
         ops.requant_exec(x, 1.0, 1.0, nonline="SIGMOID")
     with pytest.raises(Mi355Error):
         ops.requant_exec(x[1:], 1.0, 1.0)     # misaligned int32 view
+
+
+@pytest.mark.parametrize("si", range(len(SCALES)))
+def test_int8_binary_modes_exhaustive(oracle, si):
+    """QADD / QFUSE_ADD_RELU / QFUSE_ADD_H_SWISH on two int8 tensors: every one of the 65536 operand pairs."""
+    s_a, s_dst, s_b = SCALES[si]
+    s_a = s_a * 64.0          # int8 operands: bring the quotient range to a few hundred again
+    a = np.repeat(np.arange(-128, 128, dtype=np.int16), 256).astype(np.int8)
+    b = np.tile(np.arange(-128, 128, dtype=np.int16), 256).astype(np.int8)
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        say("int8 pairs", (s_a, s_b, s_dst), nl)
+        run_case(oracle, a, b, s_a, s_dst, s_b, nl)
+        run_case(oracle, a, None, s_a, s_dst, s_b, nl)    # unary QRELU / QH_SWISH / rescaling TypeCvt
+
+
+def test_int8_tail_and_alignment(oracle):
+    from megengine_amd.lib import Mi355Error
+    rng = np.random.RandomState(3)
+    for n in (1, 15, 16, 17, 4099):
+        a = rng.randint(-128, 128, n).astype(np.int8)
+        b = rng.randint(-128, 128, n).astype(np.int8)
+        run_case(oracle, a, b, 0.031, 0.047, 0.022, "RELU")
+    x = torch.zeros(64, dtype=torch.int8, device="cuda")
+    with pytest.raises(Mi355Error):
+        ops.requant_exec(x[1:33], 1.0, 1.0)

@@ -396,3 +396,30 @@ def test_requant_operator_is_the_epilogue(oracle):
     q = xi.astype(np.int64)
     want = np.clip(np.sign(q) * ((2 * np.abs(q) + 4) // 8), -128, 127).astype(np.int8)   # round-half-away of q / 4
     assert np.array_equal(got, want)
+
+
+def test_requant_int8_operands_closed_forms(oracle):
+    """Binary quantized modes on two int8 tensors: equal unit scales make QADD a saturating integer add and
+    QFUSE_ADD_RELU its positive part; element by element it is the pinned scalar epilogue."""
+    L = oracle.lib()
+    a = np.repeat(np.arange(-128, 128, dtype=np.int16), 256).astype(np.int8)
+    b = np.tile(np.arange(-128, 128, dtype=np.int16), 256).astype(np.int8)
+    s = a.astype(np.int32) + b.astype(np.int32)
+    assert np.array_equal(oracle.requant(a, 1.0, 1.0, 0, z=b, scale_z=1.0), np.clip(s, -128, 127).astype(np.int8))
+    assert np.array_equal(oracle.requant(a, 1.0, 1.0, 1, z=b, scale_z=1.0), np.clip(s, 0, 127).astype(np.int8))
+    # scale 0.5 on dst doubles; scale 2 on one operand weights it
+    assert np.array_equal(oracle.requant(a, 2.0, 0.5, 0, z=b, scale_z=1.0),
+                          np.clip(4 * a.astype(np.int32) + 2 * b.astype(np.int32), -128, 127).astype(np.int8))
+    # h_swish of integers: x * clip(x + 3, 0, 6) / 6 is an integer multiple of 1/6; compare through exact fractions
+    hs = oracle.requant(a, 1.0, 1.0, 3, z=b, scale_z=1.0).astype(np.int32)
+    num = s * np.clip(s + 3, 0, 6)                       # 6 * h_swish(s)
+    want = np.clip(np.sign(num) * ((2 * np.abs(num) + 6) // 12), -128, 127)   # round half away of num / 6
+    # float evaluation of x * t * (1/6) can differ from the exact quotient only where num / 6 sits on a tie
+    tie = (np.abs(num) % 6) == 3
+    assert np.array_equal(hs[~tie], want[~tie])
+    rng = np.random.RandomState(2)
+    idx = rng.randint(0, a.size, 4000)
+    for nl in (0, 1, 3):
+        got = oracle.requant(a[idx], 0.031, 0.047, nl, z=b[idx], scale_z=0.022)
+        ref = np.array([L.oracle_epilogue_s8(int(x), 0.031, 1, int(y), 0.022, nl, 0.047) for x, y in zip(a[idx], b[idx])], np.int8)
+        assert np.array_equal(got, ref)
