@@ -63,7 +63,8 @@ enum {
     MI355_FMT_NCHW32 = 5,
     MI355_FMT_NCHW44 = 7,
     MI355_FMT_NCHW4_NCHW32 = 9,
-    MI355_FMT_NCHW32_NCHW4 = 10
+    MI355_FMT_NCHW32_NCHW4 = 10,
+    MI355_FMT_NCHW4_NCHW = 11
 };
 /* param::ConvBias::NonlineMode (opr_param_defs.py:5-35); SIGMOID (2) is rejected for
  * quantized data exactly as naive does (conv_bias/opr_impl.cpp:79-88). */
@@ -75,7 +76,7 @@ enum { MI355_SPARSE_DENSE = 0, MI355_SPARSE_GROUP = 1 };
 /* ConvBiasForward::BiasMode (nn.h:449-453) */
 enum { MI355_BIAS_NONE = 0, MI355_BIAS_BROADCAST_CHANNEL = 1, MI355_BIAS_FULL = 2 };
 /* dst dtype */
-enum { MI355_DT_QS8 = 0, MI355_DT_QS32 = 1 };
+enum { MI355_DT_QS8 = 0, MI355_DT_QS32 = 1, MI355_DT_F32 = 2 /* Float32 dst: NCHW4_NCHW only */ };
 
 /*
  * One ConvBias problem.  Channel counts are LOGICAL channels (ic = group * icpg,
@@ -91,6 +92,14 @@ enum { MI355_DT_QS8 = 0, MI355_DT_QS32 = 1 };
  *   NCHW44 channel-wise filter layout (g/4, 1, 1, fh, fw, 4); the reference cannot express
  *   icpg < 4 under Format::NCHW4 (dnn/src/common/convolution.cpp:392-407).
  *   NCHW4_NCHW32 / NCHW32_NCHW4: src+filter in the first pack, dst/bias in the second.
+ *   NCHW4_NCHW: src+filter NCHW4, dst/bias/z NCHW (dnn/src/common/convolution.cpp:929-947).  Its dst may also be
+ *   Float32 (MI355_DT_F32; check_or_deduce_dtype_fwd, dnn/src/common/convolution.cpp:1051-1140): then bias and z are
+ *   Float32 too (passed through the typed pointers of exec by a cast, as the int32 z of a QuantizedS32 dst is),
+ *   scale_bias holds the scale of src, scale_z the scale of filter, scale_dst is ignored, and the result is
+ *   act(sum(dequantize(s) * dequantize(f)) + bias + z) in float (StrategyFwd::on for qint8 -> float,
+ *   dnn/src/naive/convolution/helper.h:59-66).  Float accumulation order is not part of the contract: the kernel
+ *   accumulates exactly in int32 and scales once; agreement with the reference's float running sum is to 1e-3
+ *   relative, the tolerance of its own checker.
  *   bias: int32, (1, oc, 1, 1) / (1, oc/p, 1, 1, p) of the dst pack, or the full dst shape.
  *   z:    dst dtype and shape, own scale.
  * src/dst/z may have a non-contiguous batch dimension: *_stride_n are in elements, 0 = dense.

@@ -11,10 +11,10 @@ ABI_VERSION = 1
 OK, ERR_BAD_ARG, ERR_UNSUPPORTED, ERR_SHAPE, ERR_WORKSPACE, ERR_LAUNCH, ERR_NO_DEVICE, ERR_ALGO = range(8)
 
 # param::ConvBias::Format
-FMT_NCHW, FMT_NCHW4, FMT_NCHW32, FMT_NCHW44, FMT_NCHW4_NCHW32, FMT_NCHW32_NCHW4 = 0, 3, 5, 7, 9, 10
+FMT_NCHW, FMT_NCHW4, FMT_NCHW32, FMT_NCHW44, FMT_NCHW4_NCHW32, FMT_NCHW32_NCHW4, FMT_NCHW4_NCHW = 0, 3, 5, 7, 9, 10, 11
 FORMAT_NAMES = {
     "NCHW": FMT_NCHW, "NCHW4": FMT_NCHW4, "NCHW32": FMT_NCHW32, "NCHW44": FMT_NCHW44,
-    "NCHW4_NCHW32": FMT_NCHW4_NCHW32, "NCHW32_NCHW4": FMT_NCHW32_NCHW4,
+    "NCHW4_NCHW32": FMT_NCHW4_NCHW32, "NCHW32_NCHW4": FMT_NCHW32_NCHW4, "NCHW4_NCHW": FMT_NCHW4_NCHW,
 }
 # param::ConvBias::NonlineMode
 NL_IDENTITY, NL_RELU, NL_SIGMOID, NL_H_SWISH = 0, 1, 2, 3
@@ -22,7 +22,7 @@ NONLINE_NAMES = {"IDENTITY": NL_IDENTITY, "RELU": NL_RELU, "SIGMOID": NL_SIGMOID
 MODE_CROSS_CORRELATION, MODE_CONVOLUTION = 0, 1
 SPARSE_DENSE, SPARSE_GROUP = 0, 1
 BIAS_NONE, BIAS_BROADCAST_CHANNEL, BIAS_FULL = 0, 1, 2
-DT_QS8, DT_QS32 = 0, 1
+DT_QS8, DT_QS32, DT_F32 = 0, 1, 2
 
 ALGO_HEURISTIC = -1
 
@@ -82,11 +82,11 @@ class RequantDesc(C.Structure):
 
 
 def in_pack(fmt):
-    return {FMT_NCHW: 1, FMT_NCHW4: 4, FMT_NCHW44: 4, FMT_NCHW4_NCHW32: 4}.get(fmt, 32)
+    return {FMT_NCHW: 1, FMT_NCHW4: 4, FMT_NCHW44: 4, FMT_NCHW4_NCHW32: 4, FMT_NCHW4_NCHW: 4}.get(fmt, 32)
 
 
 def out_pack(fmt):
-    return {FMT_NCHW: 1, FMT_NCHW4: 4, FMT_NCHW44: 4, FMT_NCHW32_NCHW4: 4}.get(fmt, 32)
+    return {FMT_NCHW: 1, FMT_NCHW4_NCHW: 1, FMT_NCHW4: 4, FMT_NCHW44: 4, FMT_NCHW32_NCHW4: 4}.get(fmt, 32)
 
 
 def out_size(i, f, d, s, p):
@@ -129,8 +129,8 @@ def conv_shapes(d):
         bias = (1, d.oc, 1, 1)
     else:
         src = (d.n, d.ic // pi, d.ih, d.iw, pi)
-        dst = (d.n, d.oc // po, oh, ow, po)
-        bias = (1, d.oc // po, 1, 1, po)
+        dst = (d.n, d.oc // po, oh, ow, po) if po > 1 else (d.n, d.oc, oh, ow)
+        bias = (1, d.oc // po, 1, 1, po) if po > 1 else (1, d.oc, 1, 1)
         if dw4:
             flt = (g // 4, 1, 1, d.fh, d.fw, 4)
         elif d.format == FMT_NCHW44:

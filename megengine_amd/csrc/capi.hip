@@ -28,14 +28,14 @@ int fail(int status, const char* fmt, ...) {
 int in_pack(uint32_t fmt) {
     switch (fmt) {
         case MI355_FMT_NCHW: return 1;
-        case MI355_FMT_NCHW4: case MI355_FMT_NCHW44: case MI355_FMT_NCHW4_NCHW32: return 4;
+        case MI355_FMT_NCHW4: case MI355_FMT_NCHW44: case MI355_FMT_NCHW4_NCHW32: case MI355_FMT_NCHW4_NCHW: return 4;
         case MI355_FMT_NCHW32: case MI355_FMT_NCHW32_NCHW4: return 32;
         default: return 0;
     }
 }
 int out_pack(uint32_t fmt) {
     switch (fmt) {
-        case MI355_FMT_NCHW: return 1;
+        case MI355_FMT_NCHW: case MI355_FMT_NCHW4_NCHW: return 1;
         case MI355_FMT_NCHW4: case MI355_FMT_NCHW44: case MI355_FMT_NCHW32_NCHW4: return 4;
         case MI355_FMT_NCHW32: case MI355_FMT_NCHW4_NCHW32: return 32;
         default: return 0;
@@ -90,7 +90,9 @@ int canonize(const mi355_conv_desc* d, ConvProblem* p) {
         return fail(MI355_ERR_UNSUPPORTED, "SIGMOID is not defined for quantized ConvBias");
     if (d->nonline > MI355_NL_H_SWISH) return fail(MI355_ERR_BAD_ARG, "invalid nonlineMode %u", d->nonline);
     if (d->bias_mode > MI355_BIAS_FULL) return fail(MI355_ERR_BAD_ARG, "invalid bias mode");
-    if (d->dst_dtype > MI355_DT_QS32) return fail(MI355_ERR_BAD_ARG, "invalid dst dtype");
+    if (d->dst_dtype > MI355_DT_F32) return fail(MI355_ERR_BAD_ARG, "invalid dst dtype");
+    if (d->dst_dtype == MI355_DT_F32 && d->format != MI355_FMT_NCHW4_NCHW)
+        return fail(MI355_ERR_UNSUPPORTED, "a Float32 dst needs format NCHW4_NCHW");
     if (d->has_z && (d->format == MI355_FMT_NCHW4_NCHW32 || d->format == MI355_FMT_NCHW32_NCHW4))
         return fail(MI355_ERR_SHAPE, "z is not allowed for NCHW4_NCHW32 / NCHW32_NCHW4");
     const uint32_t dfh = (d->fh - 1) * d->dilate_h + 1, dfw = (d->fw - 1) * d->dilate_w + 1;
@@ -105,7 +107,8 @@ int canonize(const mi355_conv_desc* d, ConvProblem* p) {
     p->z_sn = d->z_stride_n ? d->z_stride_n : dst_img;
     if (p->src_sn < src_img || p->dst_sn < dst_img || p->z_sn < dst_img)
         return fail(MI355_ERR_SHAPE, "batch stride smaller than one image");
-    p->epi.s_b = d->scale_bias;
+    // Float32 dst: scale_bias / scale_z carry the scales of src and filter; one factor dequantises the exact sum
+    p->epi.s_b = d->dst_dtype == MI355_DT_F32 ? d->scale_bias * d->scale_z : d->scale_bias;
     p->epi.s_z = d->scale_z;
     p->epi.s_d = d->scale_dst;
     p->epi.nonline = (int)d->nonline;

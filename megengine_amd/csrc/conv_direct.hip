@@ -21,7 +21,7 @@ struct DirectArgs {
     int pin, pout;
     int dw4;
     int bias_mode;
-    int dst_s32;
+    int dst_s32, dst_f32;
     int64_t src_sn, dst_sn, z_sn;
     EpiParams epi;
 };
@@ -95,6 +95,23 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(DirectArgs a) {
             }
         }
     }
+    if (a.dst_f32) {
+        // Float32 dst (NCHW4_NCHW): dequantise the exact sum once, then bias, z and activation in float
+        // (forward_bias and handle_z_inp_and_activation_naive on float tensors)
+        float v = (float)acc * a.epi.s_b;
+        const float* fb = reinterpret_cast<const float*>(a.bias);
+        if (a.bias_mode == MI355_BIAS_BROADCAST_CHANNEL)
+            v = v + fb[oc];
+        else if (a.bias_mode == MI355_BIAS_FULL)
+            v = v + fb[idx];
+        if (a.epi.has_z) v = v + reinterpret_cast<const float*>(a.z)[(int64_t)n * a.z_sn + r];
+        if (a.epi.nonline == NL_RELU)
+            v = v <= 0.f ? 0.f : v;
+        else if (a.epi.nonline == NL_H_SWISH)
+            v = v * fminf(fmaxf(v + 3.f, 0.f), 6.f) * (1.f / 6.f);
+        reinterpret_cast<float*>(a.dst)[(int64_t)n * a.dst_sn + r] = v;
+        return;
+    }
     if (a.bias_mode == MI355_BIAS_BROADCAST_CHANNEL)
         acc += a.bias[oc];
     else if (a.bias_mode == MI355_BIAS_FULL)
@@ -146,6 +163,7 @@ int launch_conv_direct(hipStream_t st, const ConvProblem& p, const int8_t* src, 
     a.pin = p.pin; a.pout = p.pout; a.dw4 = p.dw4 ? 1 : 0;
     a.bias_mode = d.bias_mode;
     a.dst_s32 = d.dst_dtype == MI355_DT_QS32;
+    a.dst_f32 = d.dst_dtype == MI355_DT_F32;
     a.src_sn = p.src_sn; a.dst_sn = p.dst_sn; a.z_sn = p.z_sn;
     a.epi = p.epi;
     const int64_t total = (int64_t)d.n * d.oc * p.oh * p.ow;

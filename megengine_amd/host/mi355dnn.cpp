@@ -36,7 +36,7 @@ using Format = param::ConvBias::Format;
 bool format_supported(Format f) {
     switch (f) {
         case Format::NCHW: case Format::NCHW4: case Format::NCHW32: case Format::NCHW44:
-        case Format::NCHW4_NCHW32: case Format::NCHW32_NCHW4:
+        case Format::NCHW4_NCHW32: case Format::NCHW32_NCHW4: case Format::NCHW4_NCHW:
             return true;
         default:
             return false;
@@ -51,7 +51,7 @@ size_t in_pack(Format f) {
 }
 size_t out_pack(Format f) {
     switch (f) {
-        case Format::NCHW: return 1;
+        case Format::NCHW: case Format::NCHW4_NCHW: return 1;
         case Format::NCHW32: case Format::NCHW4_NCHW32: return 32;
         default: return 4;
     }
@@ -141,6 +141,8 @@ void ConvBiasForward::deduce_dtype(DType src, DType filter, DType, DType, DType&
     HOST_ASSERT(src.enumv == DTypeEnum::QuantizedS8 && filter.enumv == DTypeEnum::QuantizedS8, MI355_ERR_UNSUPPORTED,
                 "this backend implements QuantizedS8 x QuantizedS8 ConvBias only");
     if (dst.enumv == DTypeEnum::QuantizedS8) return;
+    // NCHW4_NCHW may also dequantise into a Float32 dst (convolution.cpp:1051-1140)
+    if (dst.enumv == DTypeEnum::Float32 && m_param.format == Format::NCHW4_NCHW) return;
     dst = dtype::QuantizedS32(src.scale * filter.scale);
 }
 
@@ -213,12 +215,18 @@ void ConvBiasForward::canonize(const TensorLayout& src, const TensorLayout& filt
 
     uint32_t oh = 0, ow = 0;
     check_abi(mi355_convbias_deduce_out(&d, &oh, &ow));
-    out.dst_shape = packed ? TensorShape{d.n, d.oc / po, oh, ow, po} : TensorShape{d.n, d.oc, oh, ow};
+    const bool dst_packed = po != 1;
+    out.dst_shape = dst_packed ? TensorShape{d.n, d.oc / po, oh, ow, po} : TensorShape{d.n, d.oc, oh, ow};
 
     // dtypes and the bias / z rules of dnn/src/common/conv_bias.cpp:8-133
     const float s_acc = src.dtype.scale * filter.dtype.scale;
     d.scale_bias = s_acc;
-    if (bias.dtype.enumv == DTypeEnum::QuantizedS32) {
+    const bool f32 = need_dst && dst.dtype.enumv == DTypeEnum::Float32;
+    if (f32) {
+        HOST_ASSERT(p.format == Format::NCHW4_NCHW, MI355_ERR_UNSUPPORTED, "a Float32 dst needs format NCHW4_NCHW");
+        HOST_ASSERT(bias.ndim == 0 || bias.dtype.enumv == DTypeEnum::Float32, MI355_ERR_BAD_ARG,
+                    "a Float32 dst takes a Float32 bias");
+    } else if (bias.dtype.enumv == DTypeEnum::QuantizedS32) {
         HOST_ASSERT(fabsf(s_acc - bias.dtype.scale) < 1e-6f, MI355_ERR_BAD_ARG,
                     "bias scale %g differs from src scale * filter scale = %g", bias.dtype.scale, s_acc);
         d.scale_bias = bias.dtype.scale;
@@ -229,16 +237,16 @@ void ConvBiasForward::canonize(const TensorLayout& src, const TensorLayout& filt
 
     HOST_ASSERT(dst.eq_shape(out.dst_shape), MI355_ERR_SHAPE, "dst %s, expected %s", dst.to_string().c_str(),
                 out.dst_shape.to_string().c_str());
-    HOST_ASSERT(dst.dtype.enumv == DTypeEnum::QuantizedS8 || dst.dtype.enumv == DTypeEnum::QuantizedS32,
-                MI355_ERR_UNSUPPORTED, "dst must be QuantizedS8 or QuantizedS32");
+    HOST_ASSERT(dst.dtype.enumv == DTypeEnum::QuantizedS8 || dst.dtype.enumv == DTypeEnum::QuantizedS32 || f32,
+                MI355_ERR_UNSUPPORTED, "dst must be QuantizedS8, QuantizedS32 or (NCHW4_NCHW) Float32");
     HOST_ASSERT(dst.is_batch_strided(), MI355_ERR_UNSUPPORTED, "dst must be contiguous within an image");
-    d.dst_dtype = dst.dtype.enumv == DTypeEnum::QuantizedS8 ? MI355_DT_QS8 : MI355_DT_QS32;
+    d.dst_dtype = f32 ? MI355_DT_F32 : dst.dtype.enumv == DTypeEnum::QuantizedS8 ? MI355_DT_QS8 : MI355_DT_QS32;
     d.scale_dst = dst.dtype.scale;
     switch (bias_mode_of(bias, dst)) {
         case BiasMode::NO_BIAS: d.bias_mode = MI355_BIAS_NONE; break;
         case BiasMode::BIAS: d.bias_mode = MI355_BIAS_FULL; break;
         default: {
-            TensorShape want = packed ? TensorShape{1, d.oc / po, 1, 1, po} : TensorShape{1, d.oc, 1, 1};
+            TensorShape want = dst_packed ? TensorShape{1, d.oc / po, 1, 1, po} : TensorShape{1, d.oc, 1, 1};
             HOST_ASSERT(bias.eq_shape(want), MI355_ERR_SHAPE, "bias %s, expected %s or the dst shape",
                         bias.to_string().c_str(), want.to_string().c_str());
             d.bias_mode = MI355_BIAS_BROADCAST_CHANNEL;
@@ -254,6 +262,10 @@ void ConvBiasForward::canonize(const TensorLayout& src, const TensorLayout& filt
         HOST_ASSERT(z.is_batch_strided(), MI355_ERR_UNSUPPORTED, "z must be contiguous within an image");
         d.scale_z = z.dtype.scale;
         d.z_stride_n = z.stride[0];
+    }
+    if (f32) {  // the C ABI carries the scales of src and filter in these two fields for a Float32 dst
+        d.scale_bias = src.dtype.scale;
+        d.scale_z = filter.dtype.scale;
     }
     d.src_stride_n = src.is_contiguous() ? 0 : src.stride[0];
     d.dst_stride_n = dst.is_contiguous() ? 0 : dst.stride[0];

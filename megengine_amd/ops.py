@@ -60,7 +60,7 @@ def conv_bias_exec(desc, src, flt, bias=None, z=None, dst=None, algo=None, works
         ws_bytes = 0
     if dst is None:
         shape = _abi.conv_shapes(desc)[3]
-        dt = torch.int8 if desc.dst_dtype == _abi.DT_QS8 else torch.int32
+        dt = {_abi.DT_QS8: torch.int8, _abi.DT_QS32: torch.int32, _abi.DT_F32: torch.float32}[desc.dst_dtype]
         if desc.dst_stride_n:
             dst = torch.empty((desc.n, desc.dst_stride_n), dtype=dt, device=src.device)
         else:

@@ -129,13 +129,13 @@ static uint32_t out_size(uint32_t i, uint32_t f, uint32_t d, uint32_t s, uint32_
 static int in_pack(uint32_t fmt) {
     switch (fmt) {
         case MI355_FMT_NCHW: return 1;
-        case MI355_FMT_NCHW4: case MI355_FMT_NCHW44: case MI355_FMT_NCHW4_NCHW32: return 4;
+        case MI355_FMT_NCHW4: case MI355_FMT_NCHW44: case MI355_FMT_NCHW4_NCHW32: case MI355_FMT_NCHW4_NCHW: return 4;
         default: return 32;
     }
 }
 static int out_pack(uint32_t fmt) {
     switch (fmt) {
-        case MI355_FMT_NCHW: return 1;
+        case MI355_FMT_NCHW: case MI355_FMT_NCHW4_NCHW: return 1;
         case MI355_FMT_NCHW4: case MI355_FMT_NCHW44: case MI355_FMT_NCHW32_NCHW4: return 4;
         default: return 32;
     }
@@ -309,11 +309,66 @@ int oracle_convbias_s8_points(const mi355_conv_desc* d, const int8_t* src, const
 }
 
 /* full operator: naive::ConvBiasForwardImpl::exec (conv_bias/opr_impl.cpp:211-292) */
+/* Float32 dst (NCHW4_NCHW): StrategyFwd::on for (qint8, qint8) -> float, helper.h:59-66: every product is
+ * dequantize(s) * dequantize(f) in float, added to a float running sum in the loop order of compute2d (fh, fw, ic;
+ * padded taps skipped, helper.h:466-502); then the bias (float add, helper.h:732-760), z (Elemwise ADD) and the float
+ * activation (naive/conv_bias/opr_impl.cpp:21-98).  scale_bias / scale_z of the descriptor hold the scales of src and
+ * filter. */
+static int oracle_convbias_s8_f32(const mi355_conv_desc* d, uint32_t icpg, uint32_t ocpg, const int8_t* src,
+                                  const int8_t* flt, const float* bias, const float* z, float* dst) {
+    if (d->format != MI355_FMT_NCHW4_NCHW) return MI355_ERR_UNSUPPORTED;
+    const uint32_t OH = out_size(d->ih, d->fh, d->dilate_h, d->stride_h, d->pad_h);
+    const uint32_t OW = out_size(d->iw, d->fw, d->dilate_w, d->stride_w, d->pad_w);
+    const int64_t per_n = (int64_t)d->oc * OH * OW;
+    const int64_t dsn = d->dst_stride_n ? d->dst_stride_n : per_n;
+    const int64_t zsn = d->z_stride_n ? d->z_stride_n : per_n;
+    const float ss = d->scale_bias, sf = d->scale_z;
+    int h_offset = -(int)d->pad_h, w_offset = -(int)d->pad_w;
+    int dh = 1, dw = 1;
+    if (d->mode == MI355_MODE_CONVOLUTION) {
+        h_offset += (int)(d->fh - 1);
+        w_offset += (int)(d->fw - 1);
+        dh = dw = -1;
+    }
+#pragma omp parallel for collapse(2) schedule(static)
+    for (uint32_t n = 0; n < d->n; ++n)
+        for (uint32_t oc = 0; oc < d->oc; ++oc) {
+            const uint32_t g = oc / ocpg, oc_in_g = oc % ocpg;
+            for (uint32_t oh = 0; oh < OH; ++oh)
+                for (uint32_t ow = 0; ow < OW; ++ow) {
+                    float dval = 0.f;
+                    for (uint32_t fh = 0; fh < d->fh; ++fh)
+                        for (uint32_t fw = 0; fw < d->fw; ++fw) {
+                            int64_t ih = (int64_t)d->stride_h * oh + (int64_t)fh * dh + h_offset;
+                            int64_t iw = (int64_t)d->stride_w * ow + (int64_t)fw * dw + w_offset;
+                            if (ih < 0 || ih >= (int64_t)d->ih || iw < 0 || iw >= (int64_t)d->iw) continue;
+                            for (uint32_t ic = 0; ic < icpg; ++ic) {
+                                float s = (float)src[act_off(d->src_stride_n, 4, d->ic, d->ih, d->iw, n,
+                                                             (int64_t)g * icpg + ic, ih, iw)] * ss;
+                                float f = (float)flt[flt_off(d, icpg, ocpg, g, oc_in_g, ic, fh, fw)] * sf;
+                                float prod = s * f;
+                                dval = dval + prod;
+                            }
+                        }
+                    const int64_t i = ((int64_t)oc * OH + oh) * OW + ow;
+                    if (d->bias_mode == MI355_BIAS_BROADCAST_CHANNEL)
+                        dval = dval + bias[oc];
+                    else if (d->bias_mode == MI355_BIAS_FULL)
+                        dval = dval + bias[(int64_t)n * per_n + i];
+                    if (d->has_z) dval = dval + z[n * zsn + i];
+                    dst[n * dsn + i] = oracle_activation(dval, (int)d->nonline);
+                }
+        }
+    return MI355_OK;
+}
+
 int oracle_convbias_s8(const mi355_conv_desc* d, const int8_t* src, const int8_t* flt, const int32_t* bias,
                        const void* z, void* dst) {
     uint32_t icpg, ocpg;
     int st = check_desc(d, &icpg, &ocpg);
     if (st) return st;
+    if (d->dst_dtype == MI355_DT_F32)
+        return oracle_convbias_s8_f32(d, icpg, ocpg, src, flt, (const float*)bias, (const float*)z, (float*)dst);
     const int po = out_pack(d->format);
     const uint32_t OH = out_size(d->ih, d->fh, d->dilate_h, d->stride_h, d->pad_h);
     const uint32_t OW = out_size(d->iw, d->fw, d->dilate_w, d->stride_w, d->pad_w);

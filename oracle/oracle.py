@@ -70,7 +70,7 @@ def _ptr(a):
 def conv_bias(desc, src, flt, bias=None, z=None):
     """Full operator.  Arrays are C-contiguous numpy int8/int32 in the reference's layouts."""
     _, _, _, dshape = _abi.conv_shapes(desc)
-    dt = np.int8 if desc.dst_dtype == _abi.DT_QS8 else np.int32
+    dt = {_abi.DT_QS8: np.int8, _abi.DT_QS32: np.int32, _abi.DT_F32: np.float32}[desc.dst_dtype]
     if desc.dst_stride_n:
         per_n = int(np.prod(dshape[1:]))
         dst = np.zeros((desc.n, desc.dst_stride_n), dtype=dt)

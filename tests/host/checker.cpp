@@ -113,6 +113,8 @@ static std::vector<Case> cases() {
          2, 16, 8, 8, 32, 3, 3, 1},
         {"nchw32->nchw4", F::NCHW32_NCHW4, S::DENSE, N::RELU, {2, 1, 8, 8, 32}, {12, 1, 3, 3, 32}, 1, 1, true, false, false,
          2, 32, 8, 8, 12, 3, 3, 1},
+        {"nchw4->nchw", F::NCHW4_NCHW, S::DENSE, N::RELU, {2, 4, 8, 8, 4}, {10, 4, 3, 3, 4}, 1, 1, true, true, false,
+         2, 16, 8, 8, 10, 3, 3, 1},
         {"nchw dense", F::NCHW, S::DENSE, N::RELU, {2, 5, 9, 9}, {7, 5, 3, 3}, 1, 1, true, true, false,
          2, 5, 9, 9, 7, 3, 3, 1},
         {"nchw depthwise", F::NCHW, S::GROUP, N::RELU, {2, 6, 9, 9}, {6, 1, 1, 3, 3}, 1, 2, true, false, false,
@@ -125,7 +127,7 @@ static std::vector<Case> cases() {
 }
 
 static TensorShape bias_shape(const Case& c, const TensorShape& dst) {
-    if (c.fmt == CB::Format::NCHW) return {1, dst[1], 1, 1};
+    if (c.fmt == CB::Format::NCHW || c.fmt == CB::Format::NCHW4_NCHW) return {1, dst[1], 1, 1};
     return {1, dst[1], 1, 1, dst[4]};
 }
 
@@ -157,7 +159,7 @@ static void run_conv_case(Handle* h, const Case& c, bool on_gpu) {
     d.has_z = c.has_z;
     d.scale_bias = s_src * s_flt; d.scale_z = c.dst_s32 ? s_src * s_flt : s_z; d.scale_dst = c.dst_s32 ? s_src * s_flt : s_dst;
     const uint32_t oh = (c.ih + 2 * c.pad - c.fh) / c.stride + 1, ow = (c.iw + 2 * c.pad - c.fw) / c.stride + 1;
-    const bool plain = c.fmt == CB::Format::NCHW;
+    const bool plain = c.fmt == CB::Format::NCHW || c.fmt == CB::Format::NCHW4_NCHW;  // dst layout
     const uint32_t po = plain ? 1 : (c.fmt == CB::Format::NCHW32 || c.fmt == CB::Format::NCHW4_NCHW32) ? 32 : 4;
     TensorShape want = plain ? TensorShape{c.n, c.oc, oh, ow} : TensorShape{c.n, c.oc / po, oh, ow, po};
     EXPECT(dst.eq_shape(want), "deduced dst %s, expected %s", dst.to_string().c_str(), want.to_string().c_str());

@@ -54,6 +54,38 @@ def test_direct_all_formats(oracle, i):
             check_case(oracle, mk(c, nonline=nl, has_z=has_z, **S), seed=i + 1, algo=DIRECT, tag="direct%d" % i)
 
 
+NCHW4_NCHW_CASES = [
+    # shape family of the reference's own test of the format (dnn/test/cuda/conv_bias_int8.cpp:917-958), reduced
+    dict(fmt="NCHW4_NCHW", n=2, ic=16, ih=23, iw=20, oc=20, fh=3, pad=1),
+    dict(fmt="NCHW4_NCHW", n=2, ic=16, ih=12, iw=16, oc=24, fh=3, pad=1, stride=2),
+    dict(fmt="NCHW4_NCHW", n=1, ic=16, ih=9, iw=10, oc=4, fh=3),
+    dict(fmt="NCHW4_NCHW", n=2, ic=24, ih=8, iw=8, oc=6, fh=3, group=2, pad=1),
+]
+
+
+@pytest.mark.parametrize("i", range(len(NCHW4_NCHW_CASES)))
+def test_nchw4_nchw(oracle, i):
+    """NCHW4 activations and filter, NCHW dst: quantized dst bit-exact, Float32 dst to the reference checker's tolerance
+    and exactly where float arithmetic is exact (unit scales, small integers)."""
+    c = NCHW4_NCHW_CASES[i]
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        for has_z in (False, True):
+            check_case(oracle, mk(c, nonline=nl, has_z=has_z, **S), seed=40 + i, algo=DIRECT, tag="nchw4_nchw s8")
+            check_case(oracle, mk(c, nonline=nl, has_z=has_z, dst_dtype=_abi.DT_F32, scale_bias=1.9980618, scale_z=1.9980927),
+                       seed=50 + i, tag="nchw4_nchw f32", src_range=(-3, 3), flt_range=(-3, 3), bias_range=(-200, 200),
+                       z_range=(-128, 127))
+            check_case(oracle, mk(c, nonline=nl, has_z=has_z, dst_dtype=_abi.DT_F32, scale_bias=0.0173, scale_z=0.0041),
+                       seed=60 + i, tag="nchw4_nchw f32 full range")
+    # exact: unit scales, so every float product and partial sum is a small integer
+    d = mk(c, nonline="RELU", has_z=True, dst_dtype=_abi.DT_F32, scale_bias=1.0, scale_z=0.5)
+    src, flt, bias, z = util.make_tensors(d, seed=70 + i, src_range=(-8, 8), flt_range=(-8, 8))
+    want = oracle.conv_bias(d, src, flt, bias, z)
+    got = run_gpu(d, src, flt, bias, z)
+    assert np.array_equal(got, want)
+    check_case(oracle, mk(c, dst_dtype=_abi.DT_QS32, scale_bias=2e-4, scale_dst=2e-4), seed=80 + i, algo=DIRECT,
+               tag="nchw4_nchw s32")
+
+
 def test_direct_s32_dst_and_full_bias(oracle, kats):
     # the reference KAT itself, on the GPU (QuantizedS32 dst and z)
     k = kats["conv_bias_quantized8x8x32"]

@@ -423,3 +423,39 @@ def test_requant_int8_operands_closed_forms(oracle):
         got = oracle.requant(a[idx], 0.031, 0.047, nl, z=b[idx], scale_z=0.022)
         ref = np.array([L.oracle_epilogue_s8(int(x), 0.031, 1, int(y), 0.022, nl, 0.047) for x, y in zip(a[idx], b[idx])], np.int8)
         assert np.array_equal(got, ref)
+
+
+def test_nchw4_nchw_format_and_float_dst(oracle):
+    """NCHW4 in / NCHW out: the quantized result is the NCHW4 result unpacked (the reference's strategy of testing mixed
+    formats, dnn/test/naive/conv_bias.cpp:163-285); the Float32 dst is act(sum + bias + z) in float: with unit scales
+    and small integers every float operation is exact, so it must equal the int32 accumulators of the pinned integer
+    path; power-of-two scales only shift the exponent."""
+    rng = np.random.RandomState(31)
+    kw = dict(pad=1, stride=1)
+    for group in (1, 2):
+        d4 = _abi.make_conv_desc("NCHW4", 2, 16, 7, 9, 12, 3, group=group, has_z=True, nonline="H_SWISH",
+                                 scale_bias=2e-3, scale_z=0.05, scale_dst=0.07, **kw)
+        d1 = _abi.make_conv_desc("NCHW4_NCHW", 2, 16, 7, 9, 12, 3, group=group, has_z=True, nonline="H_SWISH",
+                                 scale_bias=2e-3, scale_z=0.05, scale_dst=0.07, **kw)
+        src, flt, bias, z4 = util.make_tensors(d4, seed=5 + group)
+        out4 = oracle.conv_bias(d4, src, flt, bias, z4)
+        out1 = oracle.conv_bias(d1, src, flt, util.packed_to_nchw(bias), util.packed_to_nchw(z4))
+        assert np.array_equal(out1, util.packed_to_nchw(out4))
+
+        df = _abi.make_conv_desc("NCHW4_NCHW", 2, 16, 7, 9, 12, 3, group=group, has_z=True, nonline="RELU",
+                                 dst_dtype=_abi.DT_F32, scale_bias=1.0, scale_z=1.0, **kw)
+        ss, fs, bs, ds = _abi.conv_shapes(df)
+        s = rng.randint(-9, 10, ss).astype(np.int8)
+        f = rng.randint(-9, 10, fs).astype(np.int8)
+        b = rng.randint(-99, 100, bs).astype(np.float32)
+        zz = rng.randint(-99, 100, ds).astype(np.float32)
+        got = oracle.conv_bias(df, s, f, b, zz)
+        dq = _abi.make_conv_desc("NCHW4", 2, 16, 7, 9, 12, 3, group=group, bias_mode=_abi.BIAS_NONE,
+                                 dst_dtype=_abi.DT_QS32, **kw)
+        acc = util.packed_to_nchw(oracle.conv_acc(dq, s, f, None)).astype(np.float64)
+        want = np.maximum(acc + b.reshape(1, -1, 1, 1) + zz, 0).astype(np.float32)
+        assert got.dtype == np.float32 and np.array_equal(got, want)
+        # scales 2^-3 and 2^2: the same sums times 2^-1, still exact
+        df.scale_bias, df.scale_z = 0.125, 4.0
+        got2 = oracle.conv_bias(df, s, f, b, zz)
+        assert np.array_equal(got2, np.maximum(acc * 0.5 + b.reshape(1, -1, 1, 1) + zz, 0).astype(np.float32))

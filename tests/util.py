@@ -34,6 +34,10 @@ def make_tensors(desc, seed=1, src_range=(-128, 127), flt_range=(-128, 127), bia
     if desc.has_z:
         zdt = np.int8 if desc.dst_dtype == _abi.DT_QS8 else np.int32
         z = uniform_int(seed * 4 + 3, dst_s, *z_range, zdt)
+    if desc.dst_dtype == _abi.DT_F32:
+        # Float32 dst: bias and z are float tensors; quarter-integer values keep them exactly representable
+        bias = None if bias is None else (bias.astype(np.float32) * np.float32(0.25))
+        z = None if z is None else (z.astype(np.float32) * np.float32(0.25))
     return src, flt, bias, z
 
 
