@@ -20,6 +20,7 @@
  *                                 (dnn/src/naive/conv_bias/opr_impl.cpp:211-292)
  *   mi355_convbias_algo_*      <- MultiAlgoOpr::get_all_algorithms / Algorithm::name
  *                                 (dnn/include/megdnn/oprs/base.h:545-615)
+ *   mi355_convbias_s8_profile  <- the timed trial run of the fast-run algorithm chooser (src/rdnn/impl/algo_chooser.cpp)
  *   mi355_requant_s32_s8_exec  <- the ConvBias post-process as its own pass, handle_z_inp_and_activation_naive
  *                                 (dnn/src/naive/conv_bias/opr_impl.cpp:21-98); without z that is the unary
  *                                 ElemwiseMultiType Q<mode> s32 -> s8 (dnn/src/naive/elemwise_multi_type/
@@ -168,6 +169,15 @@ int mi355_convbias_s8_query(const mi355_conv_desc* d, int algo_request, mi355_al
 int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_algo* algo,
                            const int8_t* src, const int8_t* filter, const int32_t* bias,
                            const int8_t* z, void* dst, void* workspace, size_t workspace_bytes);
+
+/* Profiling primitive of a fast-run chooser (the role of rdnn::AlgoChooser's timed trial runs over
+ * get_all_algorithms_info_safe, src/rdnn/impl/algo_chooser.cpp; dnn/include/megdnn/oprs/base.h:545-615): `warmup`
+ * untimed and `iters` timed launches of ONE algorithm, bracketed by HIP events on `stream`; *avg_usec receives the
+ * average time of a launch.  Synchronises the stream and overwrites dst; allocates no device memory. */
+int mi355_convbias_s8_profile(void* stream, const mi355_conv_desc* d, const mi355_algo* algo,
+                              const int8_t* src, const int8_t* filter, const int32_t* bias, const int8_t* z,
+                              void* dst, void* workspace, size_t workspace_bytes, int warmup, int iters,
+                              float* avg_usec);
 
 /* tile configurations of the MFMA implicit-GEMM algorithm (values of mi355_algo.tile_cfg) */
 int mi355_igemm_tile_count(void);

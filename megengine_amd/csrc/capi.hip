@@ -303,6 +303,37 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
     return MI355_OK;
 }
 
+int mi355_convbias_s8_profile(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src,
+                              const int8_t* filter, const int32_t* bias, const int8_t* z, void* dst, void* workspace,
+                              size_t workspace_bytes, int warmup, int iters, float* avg_usec) {
+    if (!avg_usec || iters <= 0 || warmup < 0) return fail(MI355_ERR_BAD_ARG, "profile: bad iteration counts or null result");
+    hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    for (int i = 0; i < warmup; ++i) {
+        int st = mi355_convbias_s8_exec(stream, d, algo, src, filter, bias, z, dst, workspace, workspace_bytes);
+        if (st) return st;
+    }
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess) return fail(MI355_ERR_LAUNCH, "profile: cannot create an event");
+    if (hipEventCreate(&e1) != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return fail(MI355_ERR_LAUNCH, "profile: cannot create an event");
+    }
+    int st = MI355_OK;
+    hipError_t he = hipEventRecord(e0, hs);
+    for (int i = 0; i < iters && st == MI355_OK && he == hipSuccess; ++i)
+        st = mi355_convbias_s8_exec(stream, d, algo, src, filter, bias, z, dst, workspace, workspace_bytes);
+    if (he == hipSuccess) he = hipEventRecord(e1, hs);
+    if (he == hipSuccess) he = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (he == hipSuccess) he = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (st) return st;
+    if (he != hipSuccess) return fail(MI355_ERR_LAUNCH, "profile: %s", hipGetErrorString(he));
+    *avg_usec = ms * 1000.f / (float)iters;
+    return MI355_OK;
+}
+
 int mi355_requant_s32_s8_exec(void* stream, const mi355_requant_desc* d, const int32_t* src, const int8_t* z, int8_t* dst) {
     if (!d) return fail(MI355_ERR_BAD_ARG, "null descriptor");
     if (d->nonline == MI355_NL_SIGMOID || d->nonline > MI355_NL_H_SWISH)

@@ -4,6 +4,13 @@
 
 #include <math.h>
 #include <stdio.h>
+#include <string.h>
+
+#include <algorithm>
+#include <fstream>
+#include <map>
+#include <mutex>
+#include <sstream>
 
 #include "../../include/mi355_convbias.h"
 
@@ -281,7 +288,104 @@ void ConvBiasForward::deduce_layout(const TensorLayout& src, const TensorLayout&
     dst = TensorLayout(c.dst_shape, dt);
 }
 
+// ---------------------------------------------------------------- algorithm cache
+struct AlgorithmCache::Impl {
+    mutable std::mutex mu;
+    std::map<std::string, Result> map;
+    static std::string key_of(const mi355_conv_desc& d) {
+        return std::string(reinterpret_cast<const char*>(&d), sizeof(d));
+    }
+};
+AlgorithmCache& AlgorithmCache::instance() {
+    static AlgorithmCache c;
+    return c;
+}
+AlgorithmCache::Impl& AlgorithmCache::impl() const {
+    static Impl i;
+    return i;
+}
+void AlgorithmCache::put(const mi355_conv_desc& key, const Result& r) {
+    Impl& i = impl();
+    std::lock_guard<std::mutex> lk(i.mu);
+    i.map[Impl::key_of(key)] = r;
+}
+bool AlgorithmCache::get(const mi355_conv_desc& key, Result& r) const {
+    Impl& i = impl();
+    std::lock_guard<std::mutex> lk(i.mu);
+    auto it = i.map.find(Impl::key_of(key));
+    if (it == i.map.end()) return false;
+    r = it->second;
+    return true;
+}
+void AlgorithmCache::clear() {
+    Impl& i = impl();
+    std::lock_guard<std::mutex> lk(i.mu);
+    i.map.clear();
+}
+size_t AlgorithmCache::size() const {
+    Impl& i = impl();
+    std::lock_guard<std::mutex> lk(i.mu);
+    return i.map.size();
+}
+void AlgorithmCache::save(const std::string& path) const {
+    Impl& i = impl();
+    std::lock_guard<std::mutex> lk(i.mu);
+    std::ofstream f(path, std::ios::trunc);
+    if (!f) fail(MI355_ERR_BAD_ARG, "cannot write the algorithm cache to " + path);
+    f << "mi355-algorithm-cache 1 " << sizeof(mi355_conv_desc) << " " << mi355_abi_version() << "\n";
+    static const char* hex = "0123456789abcdef";
+    for (auto& kv : i.map) {
+        for (unsigned char ch : kv.first) f << hex[ch >> 4] << hex[ch & 15];
+        f << ' ' << kv.second.policy.algo.id << ' ' << kv.second.policy.algo.tile_cfg << ' ' << kv.second.workspace << ' '
+          << kv.second.usec << "\n";
+    }
+}
+size_t AlgorithmCache::load(const std::string& path) {
+    std::ifstream f(path);
+    if (!f) fail(MI355_ERR_BAD_ARG, "cannot read the algorithm cache from " + path);
+    std::string magic;
+    size_t ver = 0, desc_bytes = 0;
+    int abi = 0;
+    f >> magic >> ver >> desc_bytes >> abi;
+    // a cache written for another descriptor layout or ABI revision names algorithms this library may not have
+    if (magic != "mi355-algorithm-cache" || ver != 1 || desc_bytes != sizeof(mi355_conv_desc) || abi != mi355_abi_version())
+        return 0;
+    Impl& i = impl();
+    std::lock_guard<std::mutex> lk(i.mu);
+    size_t n = 0;
+    std::string hexkey;
+    Result r;
+    while (f >> hexkey >> r.policy.algo.id >> r.policy.algo.tile_cfg >> r.workspace >> r.usec) {
+        if (hexkey.size() != 2 * sizeof(mi355_conv_desc)) continue;
+        std::string key(sizeof(mi355_conv_desc), '\0');
+        bool ok = true;
+        for (size_t b = 0; b < key.size() && ok; ++b) {
+            auto nib = [&](char ch) -> int {
+                if (ch >= '0' && ch <= '9') return ch - '0';
+                if (ch >= 'a' && ch <= 'f') return ch - 'a' + 10;
+                ok = false;
+                return 0;
+            };
+            key[b] = (char)((nib(hexkey[2 * b]) << 4) | nib(hexkey[2 * b + 1]));
+        }
+        if (!ok || r.policy.algo.id < 0 || r.policy.algo.id >= mi355_convbias_algo_count() ||
+            r.policy.algo.tile_cfg >= mi355_igemm_tile_count())
+            continue;
+        i.map[key] = r;
+        ++n;
+    }
+    return n;
+}
+
 static mi355_algo resolve_algo(const mi355_conv_desc& d, const ExecutionPolicy& pol, size_t* ws) {
+    // fast-run: a recorded winner replaces the heuristic
+    AlgorithmCache::Result hit;
+    if (!pol.valid() && pol.strategy == ExecutionPolicy::Strategy::PROFILE && AlgorithmCache::instance().get(d, hit)) {
+        mi355_algo a;
+        check_abi(mi355_convbias_s8_query(&d, hit.policy.algo.id, &a, ws));
+        if (hit.policy.algo.tile_cfg >= 0) a.tile_cfg = hit.policy.algo.tile_cfg;
+        return a;
+    }
     mi355_algo a;
     check_abi(mi355_convbias_s8_query(&d, pol.valid() ? pol.algo.id : MI355_ALGO_HEURISTIC, &a, ws));
     if (pol.valid() && pol.algo.tile_cfg >= 0) {
@@ -305,10 +409,14 @@ void ConvBiasForward::exec(const TensorND& src, const TensorND& filter, const Te
                            const TensorND& dst, const PreprocessedFilter*, const Workspace& workspace) {
     Canon c;
     canonize(src.layout, filter.layout, bias.layout, z.layout, dst.layout, c, true);
+    HOST_ASSERT(src.raw_ptr && filter.raw_ptr && dst.raw_ptr, MI355_ERR_BAD_ARG, "null tensor pointer");
+    if (!m_policy.valid() && m_policy.strategy == ExecutionPolicy::Strategy::PROFILE) {
+        AlgorithmCache::Result hit;
+        if (!AlgorithmCache::instance().get(c.d, hit)) profile_algorithms(src, filter, bias, z, dst, workspace);
+    }
     size_t ws = 0;
     mi355_algo a = resolve_algo(c.d, m_policy, &ws);
     HOST_ASSERT(workspace.size >= ws, MI355_ERR_WORKSPACE, "workspace of %zu bytes, %zu needed", workspace.size, ws);
-    HOST_ASSERT(src.raw_ptr && filter.raw_ptr && dst.raw_ptr, MI355_ERR_BAD_ARG, "null tensor pointer");
     check_abi(mi355_convbias_s8_exec(m_handle->stream(), &c.d, &a, (const int8_t*)src.raw_ptr,
                                      (const int8_t*)filter.raw_ptr,
                                      bias.layout.ndim ? (const int32_t*)bias.raw_ptr : nullptr,
@@ -331,6 +439,37 @@ std::vector<AlgorithmInfo> ConvBiasForward::get_all_algorithms_info(const Tensor
                 r.push_back(AlgorithmInfo{AlgorithmDesc{id, t}, base + ":" + mi355_igemm_tile_name(t), true});
     }
     return r;
+}
+
+std::vector<std::pair<AlgorithmInfo, float>> ConvBiasForward::profile_algorithms(
+        const TensorND& src, const TensorND& filter, const TensorND& bias, const TensorND& z, const TensorND& dst,
+        const Workspace& workspace, int warmup, int iters) {
+    Canon c;
+    canonize(src.layout, filter.layout, bias.layout, z.layout, dst.layout, c, true);
+    HOST_ASSERT(src.raw_ptr && filter.raw_ptr && dst.raw_ptr, MI355_ERR_BAD_ARG, "null tensor pointer");
+    std::vector<std::pair<AlgorithmInfo, float>> timed;
+    for (auto& info : get_all_algorithms_info(src.layout, filter.layout, bias.layout, z.layout, dst.layout)) {
+        size_t ws = 0;
+        mi355_algo a;
+        if (mi355_convbias_s8_query(&c.d, info.desc.id, &a, &ws) != MI355_OK || ws > workspace.size) continue;
+        if (info.desc.tile_cfg >= 0) a.tile_cfg = info.desc.tile_cfg;
+        float us = 0.f;
+        // an algorithm that cannot take these tensors (alignment) is skipped, not fatal
+        if (mi355_convbias_s8_profile(m_handle->stream(), &c.d, &a, (const int8_t*)src.raw_ptr,
+                                      (const int8_t*)filter.raw_ptr,
+                                      bias.layout.ndim ? (const int32_t*)bias.raw_ptr : nullptr,
+                                      z.layout.ndim ? (const int8_t*)z.raw_ptr : nullptr, dst.raw_ptr, workspace.raw_ptr,
+                                      workspace.size, warmup, iters, &us) != MI355_OK)
+            continue;
+        timed.emplace_back(info, us);
+    }
+    HOST_ASSERT(!timed.empty(), MI355_ERR_ALGO, "no algorithm could be profiled");
+    std::stable_sort(timed.begin(), timed.end(), [](const auto& x, const auto& y) { return x.second < y.second; });
+    AlgorithmCache::Result best;
+    best.policy.algo = timed.front().first.desc;
+    best.usec = timed.front().second;
+    AlgorithmCache::instance().put(c.d, best);
+    return timed;
 }
 
 AlgorithmInfo ConvBiasForward::get_algorithm_info_heuristic(const TensorLayout& src, const TensorLayout& filter,

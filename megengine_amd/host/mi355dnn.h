@@ -23,7 +23,10 @@
 #include <memory>
 #include <stdexcept>
 #include <string>
+#include <utility>
 #include <vector>
+
+struct mi355_conv_desc;  // include/mi355_convbias.h
 
 namespace mi355dnn {
 
@@ -137,8 +140,37 @@ struct AlgorithmInfo {
     bool is_reproducible = true;  // every kernel here is deterministic (no atomics, fixed order)
 };
 struct ExecutionPolicy {
-    AlgorithmDesc algo;  // id < 0: let the heuristic choose
+    // HEURISTIC: the backend's rule table.  PROFILE: fast-run -- the first exec of a problem times every usable
+    // algorithm and tile on the caller's tensors, later ones take the winner from AlgorithmCache.
+    enum class Strategy : uint32_t { HEURISTIC = 0, PROFILE = 1 };
+    AlgorithmDesc algo;  // id >= 0: use exactly this one, whatever the strategy
+    Strategy strategy = Strategy::HEURISTIC;
     bool valid() const { return algo.id >= 0; }
+};
+
+// Winners of profiling runs, keyed by the flat problem descriptor: megdnn::AlgorithmCache
+// (dnn/include/megdnn/algorithm_cache.h:12-80) with the persistence the reference keeps in its PersistentCache
+// (src/core/include/megbrain/utils/persistent_cache.h): one text line per problem.
+class AlgorithmCache {
+public:
+    struct Result {
+        ExecutionPolicy policy;
+        size_t workspace = 0;
+        float usec = 0.f;  // measured time of the winner
+    };
+    static AlgorithmCache& instance();
+    void put(const mi355_conv_desc& key, const Result& r);
+    bool get(const mi355_conv_desc& key, Result& r) const;
+    void clear();
+    size_t size() const;
+    // text file: "<descriptor bytes in hex> <algorithm id> <tile> <workspace> <microseconds>" per line
+    void save(const std::string& path) const;
+    size_t load(const std::string& path);  // returns the number of entries read; unknown lines are skipped
+
+private:
+    AlgorithmCache() = default;
+    struct Impl;
+    Impl& impl() const;
 };
 
 class Handle;
@@ -198,6 +230,12 @@ public:
                                                const TensorLayout& dst,
                                                size_t workspace_limit_in_bytes = SIZE_MAX) const;
     const char* get_algorithm_set_name() const { return "MI355_CONV_BIAS"; }
+    // fast-run: times every usable algorithm (every tile of the implicit-GEMM family) on these tensors, fastest first,
+    // and records the winner in AlgorithmCache.  Overwrites dst; synchronises the handle's stream.
+    std::vector<std::pair<AlgorithmInfo, float>> profile_algorithms(const TensorND& src, const TensorND& filter,
+                                                                    const TensorND& bias, const TensorND& z,
+                                                                    const TensorND& dst, const Workspace& workspace,
+                                                                    int warmup = 2, int iters = 10);
     static BiasMode bias_mode_of(const TensorLayout& bias, const TensorLayout& dst);
 
 private:

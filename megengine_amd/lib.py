@@ -18,7 +18,7 @@ EXPORTS = [
     "mi355_convbias_deduce_out", "mi355_convbias_algo_count", "mi355_convbias_algo_name",
     "mi355_convbias_algo_usable", "mi355_convbias_s8_query", "mi355_convbias_s8_exec",
     "mi355_igemm_tile_count", "mi355_igemm_tile_name",
-    "mi355_relayout_deduce", "mi355_relayout_exec", "mi355_requant_s32_s8_exec", "mi355_requant_s8_s8_exec",
+    "mi355_relayout_deduce", "mi355_relayout_exec", "mi355_requant_s32_s8_exec", "mi355_requant_s8_s8_exec", "mi355_convbias_s8_profile",
 ]
 
 
@@ -55,6 +55,9 @@ def lib():
     L.mi355_convbias_s8_query.argtypes = [P(_abi.ConvDesc), C.c_int, P(_abi.Algo), P(C.c_size_t)]
     L.mi355_convbias_s8_exec.argtypes = [C.c_void_p, P(_abi.ConvDesc), P(_abi.Algo), C.c_void_p, C.c_void_p,
                                          C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    L.mi355_convbias_s8_profile.argtypes = [C.c_void_p, P(_abi.ConvDesc), P(_abi.Algo), C.c_void_p, C.c_void_p,
+                                            C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int,
+                                            P(C.c_float)]
     L.mi355_igemm_tile_count.restype = C.c_int
     L.mi355_igemm_tile_name.restype = C.c_char_p
     L.mi355_igemm_tile_name.argtypes = [C.c_int]

@@ -73,6 +73,15 @@ def conv_bias_exec(desc, src, flt, bias=None, z=None, dst=None, algo=None, works
     return dst
 
 
+def conv_bias_profile(desc, src, flt, bias, z, dst, algo, warmup=2, iters=10, workspace=None):
+    """Average time in microseconds of one launch of `algo` (synchronises the current stream, overwrites dst)."""
+    us = C.c_float()
+    wsn = workspace.numel() if workspace is not None else 0
+    check(lib().mi355_convbias_s8_profile(_stream(), C.byref(desc), C.byref(algo), _ptr(src), _ptr(flt), _ptr(bias),
+                                         _ptr(z), _ptr(dst), _ptr(workspace), wsn, warmup, iters, C.byref(us)))
+    return us.value
+
+
 def conv_bias_bind(desc, src, flt, bias, z, dst, algo, workspace=None, stream=None):
     """Pre-marshals one exec call; the returned callable launches it on the CURRENT torch stream
     when `stream` is None, else on that raw stream handle, and raises on a non-zero status.

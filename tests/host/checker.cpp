@@ -333,6 +333,101 @@ static void run_relayout_gpu(Handle* h) {
     }
 }
 
+// ------------------------------------------------------------------ algorithm cache (no device)
+static void run_cache_roundtrip() {
+    printf("case: algorithm cache save / load\n");
+    AlgorithmCache& c = AlgorithmCache::instance();
+    c.clear();
+    mi355_conv_desc a = mi355_conv_desc(), b = mi355_conv_desc();
+    a.format = MI355_FMT_NCHW32; a.n = 64; a.ic = 256; a.ih = a.iw = 14; a.oc = 256; a.fh = a.fw = 3; a.group = 1;
+    a.pad_h = a.pad_w = 1; a.stride_h = a.stride_w = 1; a.dilate_h = a.dilate_w = 1; a.scale_bias = 2e-4f; a.scale_dst = 0.05f;
+    b = a; b.oc = 512;
+    AlgorithmCache::Result ra, rb, got;
+    ra.policy.algo.id = 1; ra.policy.algo.tile_cfg = 23; ra.workspace = 0; ra.usec = 15.25f;
+    rb.policy.algo.id = 0; rb.policy.algo.tile_cfg = -1; rb.workspace = 64; rb.usec = 99.5f;
+    c.put(a, ra); c.put(b, rb);
+    EXPECT(c.size() == 2, "two entries expected");
+    const std::string path = "/tmp/mi355_algo_cache_test.txt";
+    c.save(path);
+    c.clear();
+    EXPECT(!c.get(a, got), "cleared cache must miss");
+    EXPECT(c.load(path) == 2, "two entries must come back");
+    EXPECT(c.get(a, got) && got.policy.algo.id == 1 && got.policy.algo.tile_cfg == 23 && got.usec == 15.25f, "entry a");
+    EXPECT(c.get(b, got) && got.policy.algo.id == 0 && got.policy.algo.tile_cfg == -1 && got.workspace == 64, "entry b");
+    b.oc = 1024;
+    EXPECT(!c.get(b, got), "a different problem must miss");
+    // a file of another format is ignored, a missing one is an error
+    FILE* f = fopen(path.c_str(), "w");
+    fputs("something else\n", f);
+    fclose(f);
+    c.clear();
+    EXPECT(c.load(path) == 0 && c.size() == 0, "foreign file must load nothing");
+    EXPECT(throws([&] { c.load("/nonexistent/dir/cache.txt"); }, MI355_ERR_BAD_ARG), "missing file");
+    remove(path.c_str());
+    c.clear();
+}
+
+// ------------------------------------------------------------------ fast-run (GPU)
+static void run_fast_run_gpu(Handle* h) {
+    printf("case: fast-run profiling\n");
+    fflush(stdout);
+    AlgorithmCache::instance().clear();
+    auto opr = h->create_operator<ConvBiasForward>();
+    opr->param().format = CB::Format::NCHW32;
+    opr->param().nonlineMode = CB::NonlineMode::RELU;
+    opr->param().pad_h = opr->param().pad_w = 1;
+    const float s_src = 0.02f, s_flt = 0.01f, s_dst = 0.05f;
+    TensorLayout src({4, 4, 14, 14, 32}, dtype::QuantizedS8(s_src)), flt({128, 4, 3, 3, 32}, dtype::QuantizedS8(s_flt));
+    TensorLayout bias({1, 4, 1, 1, 32}, dtype::QuantizedS32(s_src * s_flt)), z, dst;
+    dst.dtype = dtype::QuantizedS8(s_dst);
+    opr->deduce_layout(src, flt, bias, z, dst);
+    std::vector<int8_t> hsrc(src.total_nr_elems()), hflt(flt.total_nr_elems());
+    std::vector<int32_t> hbias(bias.total_nr_elems());
+    fill_s8(hsrc, 21, -128, 127);
+    fill_s8(hflt, 22, -127, 127);
+    fill_s32(hbias, 23, -1000, 1000);
+    mi355_conv_desc d = mi355_conv_desc();
+    d.format = MI355_FMT_NCHW32; d.nonline = MI355_NL_RELU; d.n = 4; d.ic = 128; d.ih = d.iw = 14; d.oc = 128; d.fh = d.fw = 3;
+    d.group = 1; d.pad_h = d.pad_w = 1; d.stride_h = d.stride_w = 1; d.dilate_h = d.dilate_w = 1;
+    d.bias_mode = MI355_BIAS_BROADCAST_CHANNEL; d.scale_bias = s_src * s_flt; d.scale_z = 1.f; d.scale_dst = s_dst;
+    std::vector<int8_t> expect(dst.total_nr_elems()), got(dst.total_nr_elems());
+    EXPECT(oracle_convbias_s8(&d, hsrc.data(), hflt.data(), hbias.data(), nullptr, expect.data()) == 0, "CPU checker");
+    DevBuf dsrc(hsrc.size()), dflt(hflt.size()), dbias(hbias.size() * 4), ddst(got.size()), dws(16);
+    HIP_OK(hipMemcpy(dsrc.p, hsrc.data(), hsrc.size(), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dflt.p, hflt.data(), hflt.size(), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dbias.p, hbias.data(), hbias.size() * 4, hipMemcpyHostToDevice));
+
+    auto timed = opr->profile_algorithms(TensorND(dsrc.p, src), TensorND(dflt.p, flt), TensorND(dbias.p, bias), TensorND(nullptr, z),
+                                         TensorND(ddst.p, dst), Workspace(dws.p, 0), 1, 5);
+    EXPECT(timed.size() >= 2, "several algorithms must have been timed, got %zu", timed.size());
+    for (size_t i = 1; i < timed.size(); ++i) EXPECT(timed[i - 1].second <= timed[i].second, "results must be sorted");
+    printf("  %zu algorithms timed, fastest %s %.2f us, slowest %s %.2f us\n", timed.size(), timed.front().first.name.c_str(),
+           timed.front().second, timed.back().first.name.c_str(), timed.back().second);
+    EXPECT(AlgorithmCache::instance().size() == 1, "the winner must be cached");
+
+    // the PROFILE strategy takes the cached winner and must still be bit-exact
+    opr->execution_policy().strategy = ExecutionPolicy::Strategy::PROFILE;
+    HIP_OK(hipMemset(ddst.p, 0x5a, got.size()));
+    opr->exec(TensorND(dsrc.p, src), TensorND(dflt.p, flt), TensorND(dbias.p, bias), TensorND(nullptr, z), TensorND(ddst.p, dst),
+              nullptr, Workspace(dws.p, 0));
+    HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
+    HIP_OK(hipMemcpy(got.data(), ddst.p, got.size(), hipMemcpyDeviceToHost));
+    size_t bad = 0;
+    for (size_t i = 0; i < got.size(); ++i) bad += got[i] != expect[i];
+    EXPECT(bad == 0, "fast-run exec: %zu bytes differ", bad);
+    // a problem not seen before is profiled on first use
+    AlgorithmCache::instance().clear();
+    opr->exec(TensorND(dsrc.p, src), TensorND(dflt.p, flt), TensorND(dbias.p, bias), TensorND(nullptr, z), TensorND(ddst.p, dst),
+              nullptr, Workspace(dws.p, 0));
+    HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
+    EXPECT(AlgorithmCache::instance().size() == 1, "first use under PROFILE must fill the cache");
+    HIP_OK(hipMemcpy(got.data(), ddst.p, got.size(), hipMemcpyDeviceToHost));
+    bad = 0;
+    for (size_t i = 0; i < got.size(); ++i) bad += got[i] != expect[i];
+    EXPECT(bad == 0, "fast-run first use: %zu bytes differ", bad);
+    AlgorithmCache::instance().clear();
+}
+
 int main(int argc, char** argv) {
     bool gpu = argc > 1 && !strcmp(argv[1], "--gpu");
     bool cpu = argc > 1 && !strcmp(argv[1], "--cpu");
@@ -349,8 +444,10 @@ int main(int argc, char** argv) {
         auto handle = Handle::make(stream, 0);
         if (gpu) handle->check_device();
         run_validation(handle.get());
+        run_cache_roundtrip();
         for (auto& c : cases()) run_conv_case(handle.get(), c, gpu);
         if (gpu) run_relayout_gpu(handle.get());
+        if (gpu) run_fast_run_gpu(handle.get());
     } catch (const Error& e) {
         printf("unexpected mi355dnn::Error %d: %s\n", e.status(), e.what());
         return 1;

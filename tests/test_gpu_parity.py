@@ -304,3 +304,26 @@ def test_first_layer_kernel(oracle, i):
                             bias_mode=_abi.BIAS_NONE, src_stride_n=int(np.prod(ss[1:])) + 20,
                             dst_stride_n=int(np.prod(ds[1:])) + 12, z_stride_n=int(np.prod(ds[1:])) + 36, **S)
     check_case(oracle, d, seed=600 + i, tag="c4-%d-strided" % i)
+
+
+def test_profile_entry_point(oracle):
+    """the timed trial run of a fast-run chooser: times one algorithm, leaves the right result in dst"""
+    d = _abi.make_conv_desc("NCHW32", 8, 128, 14, 14, 128, 3, pad=1, nonline="RELU", **S)
+    src, flt, bias, z = util.make_tensors(d, seed=91)
+    want = oracle.conv_bias(d, src, flt, bias, z)
+    ts, tf, tb = to_dev(src), to_dev(flt), to_dev(bias)
+    dst = torch.zeros(_abi.conv_shapes(d)[3], dtype=torch.int8, device="cuda")
+    times = {}
+    for algo_id in (DIRECT, IGEMM):
+        a, _ = ops.conv_bias_query(d, algo_id)
+        dst.zero_()
+        us = ops.conv_bias_profile(d, ts, tf, tb, None, dst, a, warmup=1, iters=5)
+        say("profile", algo_id, "%.2f us" % us)
+        assert 0.5 < us < 1e5
+        assert np.array_equal(dst.cpu().numpy(), want)
+        times[algo_id] = us
+    assert times[IGEMM] < times[DIRECT]       # the MFMA kernel must beat one-thread-per-output
+    from megengine_amd.lib import Mi355Error
+    a, _ = ops.conv_bias_query(d, IGEMM)
+    with pytest.raises(Mi355Error):
+        ops.conv_bias_profile(d, ts, tf, tb, None, dst, a, warmup=0, iters=0)
