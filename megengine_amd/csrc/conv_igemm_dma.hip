@@ -16,6 +16,10 @@
 //     stricter, never too weak; and because the compiler does not see the copies, it cannot serialise them.
 //   * before the workgroup ends it waits for every copy (vmcnt(0)): a copy landing after the LDS allocation
 //     has been handed to another workgroup would corrupt it.
+//   * the stages of a tile split into a steady loop, whose refills stay inside the tile (no tile bookkeeping: with 16
+//     waves on a CU the one scalar unit paces a loop that carries it), and the last NS stages, whose refills cross
+//     into the workgroup's next tile.  The bias of the workgroup's channel tile sits in LDS, written once: tiles of
+//     one workgroup are a multiple of the channel-tile count apart whenever that count is a power of two.
 #include "igemm_shared.h"
 
 namespace mi355 {
@@ -62,7 +66,7 @@ struct DmaKernel {
     static constexpr int UA = BM / (RPL * NW);     // copies per wave per stage
     static constexpr int UB = BN / (RPL * NW);
     static constexpr int U = UA + UB;
-    static constexpr int BIAS_BYTES = 2 * BM * 4;  // flat schedule: bias of the current and the next tile
+    static constexpr int BIAS_BYTES = BM * 4;  // bias of the workgroup's channel tile
     static constexpr int RING_BYTES = NS * STG + BIAS_BYTES;
     static_assert(NW == 4 || NW == 8, "4 or 8 waves");
     static_assert(UA >= 1 && UB >= 1 && BM % (RPL * NW) == 0 && BN % (RPL * NW) == 0, "tile vs copy granularity");
@@ -154,34 +158,6 @@ struct DmaKernel {
         }
     }
 
-    // Bias of one wave tile in accumulator order (lane l, register v of a 32x32 block: channel 8 (v / 4) + 4 (l / 32) +
-    // v % 4), straight from global memory: 4 x 16 bytes per 32 channels.  A buffer of zero size (no bias) and channels
-    // past OC read as zeros.  Requested a tile ahead, so that its latency runs under the previous tile's last stage.
-    struct BiasRegs {
-        v4i v[MT][4];
-    };
-    __device__ static __forceinline__ void load_bias(const IgemmArgs& a, BiasRegs& b, int oc_w, int lh) {
-        const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.bias, a.has_bias ? (uint32_t)a.OC * 4u : 0u);
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                b.v[i][q] = __builtin_amdgcn_raw_buffer_load_b128(rs, (oc_w + i * 32 + 8 * q + 4 * lh) * 4, 0, 0);
-    }
-    __device__ static __forceinline__ void init_acc(v16i (&acc)[MT][NT], const BiasRegs& b) {
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            v16i init;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                init[4 * q + 0] = b.v[i][q][0]; init[4 * q + 1] = b.v[i][q][1];
-                init[4 * q + 2] = b.v[i][q][2]; init[4 * q + 3] = b.v[i][q][3];
-            }
-#pragma unroll
-            for (int j = 0; j < NT; ++j) acc[i][j] = init;
-        }
-    }
-
     __device__ static __forceinline__ void init_acc_lds(v16i (&acc)[MT][NT], const int* sBias, int wm, int lh) {
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
@@ -201,184 +177,10 @@ struct DmaKernel {
         return (a.has_bias && t < BM && oc < a.OC) ? a.bias[oc] : 0;
     }
 
-    // Flat schedule: one loop over all (tile, stage) pairs of the workgroup.  Used when workgroups own several tiles.
-    __device__ static __forceinline__ void run_flat(const IgemmArgs& a) {
-        extern __shared__ __attribute__((aligned(16))) int8_t lds[];
-        int* sBias = reinterpret_cast<int*>(lds + NS * STG);  // 2 x BM
-        KEntry* tab = reinterpret_cast<KEntry*>(lds + RING_BYTES);
-        const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)lds);
-
-        const int t = threadIdx.x;
-        const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
-        const int l32 = lane & 31, lh = lane >> 5;
-        const int wm = wave / WN, wn = wave % WN;
-
-        // this workgroup's tile sequence (XCD-contiguous ranges, see conv_igemm.hip)
-        int first, step, last;
-        {
-            const int G = gridDim.x, b = blockIdx.x;
-            if ((G & 7) == 0) {
-                const int x = b & 7, j = b >> 3, gx = G >> 3;
-                const int per = a.tiles >> 3, rem = a.tiles & 7;
-                const int t0 = x * per + (x < rem ? x : rem);
-                last = t0 + per + (x < rem ? 1 : 0);
-                first = t0 + j;
-                step = gx;
-            } else {
-                first = b; step = G; last = a.tiles;
-            }
-        }
-        const int my_tiles = first < last ? (last - first + step - 1) / step : 0;
-        const int total = my_tiles * a.nstages;
-
-        if (!PW) {
-            const int cap = a.nstages * KCH;
-            for (int e = t; e < cap; e += THREADS) {
-                KEntry k;
-                if (e < a.entries) {
-                    const uint32_t cb = fdiv(e, a.div_t), tap = e - cb * a.T;
-                    const uint32_t fh = fdiv(tap, a.div_fw), fw = tap - fh * a.FW;
-                    k.off = (int)cb * a.src_scb + ((int)fh * a.IW + (int)fw) * 32;
-                    k.fhfw = (int)(fh | (fw << 16));
-                } else {
-                    k.off = 0;
-                    k.fhfw = 0x4000;
-                }
-                tab[e] = k;
-            }
-        }
-        if (total == 0) return;
-
-        const v4i rs_src = uniform_rsrc(a.src, a.src_bytes);
-        const v4i rs_flt = uniform_rsrc(a.flt, a.flt_bytes);
-
-        Loader L;
-        L.tile = first;
-        L.stage = 0;
-        L.kc0 = 0;
-        loader_enter_tile(a, L, first, wave, lane);
-        int issued = 0;
-        auto advance = [&]() __attribute__((always_inline)) {
-            ++issued;
-            L.kc0 += KCH;
-            if (++L.stage == a.nstages) {
-                L.stage = 0;
-                L.kc0 = 0;
-                L.tile += step;
-                if (issued < total) loader_enter_tile(a, L, L.tile, wave, lane);
-            }
-            if (issued >= total) loader_kill(L);
-        };
-
-        int c_tile = first, c_stage = 0, c_oc0, c_pix0;
-        tile_coords(a, c_tile, c_oc0, c_pix0);
-        int c_par = 0;
-        int bias_next = 0;
-        if (t < BM) sBias[t] = fetch_bias(a, c_oc0, t);
-        __syncthreads();  // table and bias ready
-
-        // prologue: stages 0 .. NS - 2 go to buffers 0 .. NS - 2
-#pragma unroll
-        for (int s = 0; s < NS - 1; ++s) {
-            issue(a, L, tab, rs_src, rs_flt, lds0 + (uint32_t)(s * STG), wave, lane);
-            advance();
-        }
-        int rd = 0, wr = NS - 1;  // ring positions of the stage being multiplied / refilled
-
-        v16i acc[MT][NT];
-        constexpr bool DUAL = MT * NT == 1;
-        v16i alt;
-
-        for (int it = 0; it < total; ++it) {
-            // stage `it` of this wave has landed once at most the NS - 2 younger stages are in flight
-            wait_vmcnt<(NS - 2) * U>();
-            __syncthreads();  // ... of every wave; and every wave is done reading the buffer refilled next
-            // the residual of a tile is requested at the start of its last stage -- before this iteration's copies, so
-            // that waiting for it in the epilogue does not also wait for them
-            const bool last_stage = c_stage + 1 == a.nstages;
-            ZRegs<MT, NT> zr;
-            if (last_stage && a.epi.has_z) igemm_load_z<POUT, MT, NT>(a, zr, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh);
-            issue(a, L, tab, rs_src, rs_flt, lds0 + (uint32_t)(wr * STG), wave, lane);
-            advance();
-
-            if (c_stage == 0) {
-                init_acc_lds(acc, sBias + c_par * BM, wm, lh);
-                if (DUAL) alt = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            }
-            int n_oc0 = c_oc0, n_pix0 = c_pix0;
-            if (last_stage && it + 1 < total) {
-                tile_coords(a, c_tile + step, n_oc0, n_pix0);
-                if (a.tiles_m > 1) bias_next = fetch_bias(a, n_oc0, t);  // lands during the MFMAs + epilogue
-            }
-
-            const int8_t* pA = lds + rd * STG;
-            const int8_t* pB = pA + A_BYTES;
-            constexpr int FD = KCH * (MT + NT) <= 12 ? KCH : 2;
-            v4i fa[FD][MT], fb[FD][NT];
-            auto frags = [&](int c, v4i (&xa)[MT], v4i (&xb)[NT]) __attribute__((always_inline)) {
-#pragma unroll
-                for (int i = 0; i < MT; ++i) {
-                    const int row = wm * WTM + i * 32 + l32;
-                    const int slot = (c * 2 + lh) ^ swz<S>(row);
-                    xa[i] = *reinterpret_cast<const v4i*>(pA + row * ROWB + slot * 16);
-                }
-#pragma unroll
-                for (int j = 0; j < NT; ++j) {
-                    const int row = wn * WTN + j * 32 + l32;
-                    const int slot = (c * 2 + lh) ^ swz<S>(row);
-                    xb[j] = *reinterpret_cast<const v4i*>(pB + row * ROWB + slot * 16);
-                }
-            };
-            auto mfmas = [&](int c, const v4i (&xa)[MT], const v4i (&xb)[NT]) __attribute__((always_inline)) {
-#pragma unroll
-                for (int i = 0; i < MT; ++i)
-#pragma unroll
-                    for (int j = 0; j < NT; ++j) {
-                        if (DUAL && (c & 1))
-                            alt = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa[i], xb[j], alt, 0, 0, 0);
-                        else
-                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xa[i], xb[j], acc[i][j], 0, 0, 0);
-                    }
-            };
-            if (FD == KCH) {
-#pragma unroll
-                for (int c = 0; c < KCH; ++c) frags(c, fa[c], fb[c]);
-#pragma unroll
-                for (int c = 0; c < KCH; ++c) mfmas(c, fa[c], fb[c]);
-            } else {
-                frags(0, fa[0], fb[0]);
-#pragma unroll
-                for (int c = 0; c < KCH; ++c) {
-                    if (c + 1 < KCH) frags(c + 1, fa[(c + 1) & 1], fb[(c + 1) & 1]);
-                    mfmas(c, fa[c & 1], fb[c & 1]);
-                }
-            }
-
-            if (last_stage) {
-                if (DUAL) acc[0][0] += alt;
-                igemm_run_epilogue<POUT, MT, NT, true>(a, acc, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh, &zr);
-                c_stage = 0;
-                c_tile += step;
-                if (a.tiles_m > 1) {
-                    c_par ^= 1;
-                    if (t < BM) sBias[c_par * BM + t] = bias_next;
-                }
-                c_oc0 = n_oc0;
-                c_pix0 = n_pix0;
-            } else {
-                ++c_stage;
-            }
-            rd = rd + 1 == NS ? 0 : rd + 1;
-            wr = wr + 1 == NS ? 0 : wr + 1;
-        }
-        // the trailing (out-of-range, zero-filling) copies must land before this workgroup's LDS is released
-        wait_vmcnt<0>();
-    }
-
-    // Nested schedule: per tile a steady loop whose refills stay inside the tile (the loader only steps along k: no
-    // tile bookkeeping, a third of the scalar instructions of the flat loop) and the last NS stages, whose refills
-    // cross into the next tile.  Used when every workgroup owns one tile and the reduction is long.
-    __device__ static __forceinline__ void run_nested(const IgemmArgs& a) {
+    // Per tile: a steady loop whose refills stay inside the tile -- the loader only steps along k, so the loop carries no
+    // tile bookkeeping (with 16 waves on a CU its one scalar unit paces a loop that does) -- then the last NS stages, whose
+    // refills cross into the next tile and which carry the residual prefetch and the next tile's coordinates.
+    __device__ static __forceinline__ void run(const IgemmArgs& a) {
         extern __shared__ __attribute__((aligned(16))) int8_t lds[];
         KEntry* tab = reinterpret_cast<KEntry*>(lds + RING_BYTES);
         const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)lds);
@@ -406,11 +208,13 @@ struct DmaKernel {
         const int my_tiles = first < last ? (last - first + step - 1) / step : 0;
         const int total = my_tiles * a.nstages;
 
-        // the first tile's bias is requested before anything else, so that it lands while the table is built
+        // The bias of the workgroup's channel tile lives in LDS, written once before the first barrier: workgroups
+        // mostly stay on one channel tile (their tile stride is a multiple of the number of channel tiles whenever
+        // that is a power of two), so the copy is read at every tile start and almost never rewritten.
+        int* sBias = reinterpret_cast<int*>(lds + NS * STG);
         int c_tile = first, c_oc0, c_pix0;
         tile_coords(a, c_tile, c_oc0, c_pix0);
-        BiasRegs bias;
-        load_bias(a, bias, c_oc0 + wm * WTM, lh);
+        if (t < BM) sBias[t] = fetch_bias(a, c_oc0, t);
 
         if (!PW) {
             const int cap = a.nstages * KCH;
@@ -459,9 +263,8 @@ struct DmaKernel {
             issue(a, L, tab, rs_src, rs_flt, lds0 + (uint32_t)(s * STG), wave, lane);
             advance();
         }
-        // behind the first copies: the bias, often cold in HBM like the first filter stage, then lands alongside them
         v16i acc[MT][NT];
-        init_acc(acc, bias);
+        init_acc_lds(acc, sBias, wm, lh);
         int rd_off = 0;                                     // byte offset of the stage being multiplied
         uint32_t wr_addr = lds0 + (uint32_t)((NS - 1) * STG);  // LDS address of the stage buffer refilled next
 
@@ -545,16 +348,22 @@ struct DmaKernel {
                 advance();
                 if (last_stage && ti + 1 < my_tiles) {
                     tile_coords(a, c_tile + step, n_oc0, n_pix0);
-                    // workgroups mostly stay on one channel tile (their tile stride is a multiple of the number of
-                    // channel tiles whenever that is a power of two), so this reload is rare
-                    if (n_oc0 != c_oc0) load_bias(a, bias, n_oc0 + wm * WTM, lh);
                 }
                 multiply();
             }
             if (DUAL) acc[0][0] += alt;
             igemm_run_epilogue<POUT, MT, NT, true>(a, acc, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh, &zr);
             c_tile += step;
-            if (ti + 1 < my_tiles) init_acc(acc, bias);
+            if (ti + 1 < my_tiles) {
+                if (n_oc0 != c_oc0) {
+                    // rare: another channel tile.  Everyone is done with the old copy before it is replaced, and
+                    // sees the new one before it is read (a workgroup-uniform branch: barriers are safe here)
+                    __syncthreads();
+                    if (t < BM) sBias[t] = fetch_bias(a, n_oc0, t);
+                    __syncthreads();
+                }
+                init_acc_lds(acc, sBias, wm, lh);
+            }
             c_oc0 = n_oc0;
             c_pix0 = n_pix0;
         }
@@ -563,12 +372,9 @@ struct DmaKernel {
     }
 };
 
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, bool NESTED>
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW>
 __global__ __launch_bounds__(WM * WN * 64, MINW) void igemm_dma_kernel(IgemmArgs a) {
-    if (NESTED)
-        DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW>::run_nested(a);
-    else
-        DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW>::run_flat(a);
+    DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW>::run(a);
 }
 
 struct DmaCfg {
@@ -599,23 +405,24 @@ const DmaCfg kDma[] = {
 };
 constexpr int kNumDma = sizeof(kDma) / sizeof(kDma[0]);
 
-// Launch with one of the two schedules.  The nested one declines (returns false, launches nothing) unless every
-// workgroup gets one tile, give or take the few left over when the grid is rounded to a multiple of 8.
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, bool NESTED>
-bool launch_sched(hipStream_t st, const IgemmArgs& a, int cu_count, int* rc) {
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW>
+int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
     using K = DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW>;
+    a.tiles_m = (a.OC + BM - 1) / BM;
+    a.tiles_n = (a.M + BN - 1) / BN;
+    const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
+    if (tiles <= 0 || tiles > 0x3fffffff) return (int)hipErrorInvalidValue;
+    a.tiles = (int)tiles;
+    a.nstages = (a.KC + KCH - 1) / KCH;
     const int tab_entries = PW ? 0 : a.nstages * KCH;
     const int lds = K::RING_BYTES + tab_entries * 8;
-    auto kern = igemm_dma_kernel<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW, NESTED>;
+    auto kern = igemm_dma_kernel<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW>;
     static int max_lds_set = 0;
     if (lds > max_lds_set) {
         const int want = K::RING_BYTES + IG_MAX_ENTRIES * 8;
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, want);
-        if (e != hipSuccess) {
-            *rc = (int)e;
-            return true;
-        }
+        if (e != hipSuccess) return (int)e;
         max_lds_set = want;
     }
     static int occ_lds = -1, occ_val = 0;
@@ -632,28 +439,10 @@ bool launch_sched(hipStream_t st, const IgemmArgs& a, int cu_count, int* rc) {
     }
     if (cu_count <= 0) cu_count = 256;
     int64_t grid = (int64_t)occ * cu_count;
-    if (grid > a.tiles) grid = a.tiles;
+    if (grid > tiles) grid = tiles;
     if (grid >= 8) grid &= ~(int64_t)7;
-    if (NESTED && a.tiles > grid + 7) return false;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(K::THREADS), lds, st, a);
-    *rc = (int)hipGetLastError();
-    return true;
-}
-
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW>
-int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
-    a.tiles_m = (a.OC + BM - 1) / BM;
-    a.tiles_n = (a.M + BN - 1) / BN;
-    const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
-    if (tiles <= 0 || tiles > 0x3fffffff) return (int)hipErrorInvalidValue;
-    a.tiles = (int)tiles;
-    a.nstages = (a.KC + KCH - 1) / KCH;
-    int rc = 0;
-    // long reductions (3x3 filters over 256 channels and more) on one tile per workgroup: the nested schedule, which
-    // measured 5 - 15 % faster there inside a network; shorter ones measured no gain: the flat one
-    if (a.nstages > NS && a.kbytes >= 2304 && launch_sched<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW, true>(st, a, cu_count, &rc)) return rc;
-    launch_sched<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW, false>(st, a, cu_count, &rc);
-    return rc;
+    return (int)hipGetLastError();
 }
 
 template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW>
@@ -682,7 +471,7 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
         case 13: return launch_one<POUT, 64, 128, 2, 2, 4, 2, 2>(st, a, cu);
         case 14: return launch_one<POUT, 128, 128, 2, 4, 2, 3, 2>(st, a, cu);
         case 15: return launch_one<POUT, 128, 64, 4, 2, 4, 3, 2>(st, a, cu);
-        case 16: return launch_one<POUT, 256, 128, 4, 2, 2, 3, 1>(st, a, cu);
+        case 16: return launch_one<POUT, 256, 128, 4, 2, 2, 3, 4>(st, a, cu);
         case 17: return launch_one<POUT, 128, 128, 2, 4, 4, 2, 2>(st, a, cu);
         case 18: return launch_one<POUT, 64, 128, 2, 4, 4, 3, 2>(st, a, cu);
         default: return (int)hipErrorInvalidValue;

@@ -52,6 +52,8 @@ FULL_CASES = [
     ("stem", "NCHW4", 16, 4, 224, 64, 7, 2, 3, "RELU", False),             # config 2 stem (batch 16)
     ("mbv2_expand", "NCHW4", 64, 24, 56, 144, 1, 1, 0, "RELU", False),     # config 3
     ("mbv2_project", "NCHW4", 64, 144, 56, 24, 1, 1, 0, "IDENTITY", True),
+    # three / six channel tiles: successive tiles of a workgroup change channel tile, so the bias copy is rewritten
+    ("oc384_3x3", "NCHW32", 16, 64, 56, 384, 3, 1, 1, "RELU", True),
     ("large_hswish", "NCHW32", 16, 256, 64, 256, 3, 1, 1, "H_SWISH", True),  # config 4a at batch 16
     ("large_5x5", "NCHW32", 8, 128, 80, 128, 5, 1, 2, "H_SWISH", True),      # config 4c at batch 8
 ]
