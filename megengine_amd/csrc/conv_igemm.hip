@@ -512,15 +512,18 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
         enum {
             D128x128x64 = kNumCfgs + 0, D64x64x128 = kNumCfgs + 1, D128x128x128r2 = kNumCfgs + 7, D64x64x64r4 = kNumCfgs + 10,
             D128x64x128r2 = kNumCfgs + 11, D64x128x128r2 = kNumCfgs + 13, D128x128x64w8 = kNumCfgs + 14,
-            D128x64x128w8 = kNumCfgs + 15, D256x128x64w8 = kNumCfgs + 16, D128x128x128r2w8 = kNumCfgs + 17
+            D128x64x128w8 = kNumCfgs + 15, D256x128x64w8 = kNumCfgs + 16, D128x128x128r2w8 = kNumCfgs + 17,
+            D64x64x128r2 = kNumCfgs + 6, D64x128x128w8 = kNumCfgs + 18
         };
-        if (OC <= 64) return kbytes <= 64 ? D64x64x64r4 : D64x128x128r2;
+        if (OC <= 64) return kbytes <= 64 ? D128x128x64w8 : kbytes <= 256 ? D64x64x128r2 : D64x128x128r2;
         const int64_t t128 = tiles(0);
         if (t128 >= 4 * cu_count)
             return kbytes >= 1024 ? (OC >= 256 ? D256x128x64w8 : D128x128x128r2) : (kbytes <= 128 ? D128x128x64w8 : 0);
         if (t128 >= 2 * cu_count) return D128x64x128r2;
         if (2 * t128 >= 3 * cu_count) return kbytes >= 512 ? D128x128x128r2w8 : D128x128x64;
-        // few tiles, long reductions: the deeper ring hides the cold first touch of every weight byte
+        // few tiles, long reductions: the deeper ring hides the cold first touch of every weight byte; the longest
+        // ones (3x3 over 256 channels) run best with more pixels than channels per tile
+        if (kbytes >= 2304 && tiles(6) >= cu_count) return D64x128x128w8;
         return tiles(7) >= cu_count ? D128x64x128w8 : D64x64x128;
     }
     if (OC <= 64) return tiles(1) >= cu_count ? 1 : 3;
