@@ -15,6 +15,8 @@
 // v_mfma_i32_32x32x32_i8: A = 32 output channels, B = 32 pixels (2 output rows x 16 columns of the
 // tile), accumulator layout as in conv_igemm.hip; epilogue per lane: 4 consecutive channels of one
 // pixel = one dword of the NCHW4 output.
+#include <atomic>
+
 #include "common.h"
 
 namespace mi355 {
@@ -295,9 +297,9 @@ int launch_conv_c4(hipStream_t st, const ConvProblem& p, int cu_count, const int
     if (cu_count <= 0) cu_count = 256;
     // persistent grid: exactly as many workgroups as are resident at once (a workgroup that had to wait for a
     // slot would start its whole share of tiles late)
-    static int occ[2] = {0, 0};
+    static std::atomic<int> occ[2];  // zero-initialised; several threads may launch
     const int si = d.stride_h == 2 ? 1 : 0;
-    if (!occ[si]) {
+    if (!occ[si].load(std::memory_order_relaxed)) {
         int o = 0;
         hipError_t e = si ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&o, reinterpret_cast<const void*>(c4_kernel<2>), C4_THREADS, 0)
                           : hipOccupancyMaxActiveBlocksPerMultiprocessor(&o, reinterpret_cast<const void*>(c4_kernel<1>), C4_THREADS, 0);
@@ -305,9 +307,9 @@ int launch_conv_c4(hipStream_t st, const ConvProblem& p, int cu_count, const int
             (void)hipGetLastError();
             o = 1;
         }
-        occ[si] = o;
+        occ[si].store(o, std::memory_order_relaxed);
     }
-    int64_t grid = (int64_t)occ[si] * cu_count;
+    int64_t grid = (int64_t)occ[si].load(std::memory_order_relaxed) * cu_count;
     if (grid > a.tiles) grid = a.tiles;
     if (si)
         hipLaunchKernelGGL((c4_kernel<2>), dim3((unsigned)grid), dim3(C4_THREADS), 0, st, a);

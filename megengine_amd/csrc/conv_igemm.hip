@@ -21,6 +21,8 @@
 // oc = 8*(v/4) + 4*(l/32) + v%4.  NCHW4 output stores one dword (4 channels) per register quad;
 // NCHW32 output first exchanges quads between lanes l and l+32 (v_permlane32_swap) so that each
 // lane owns 16 consecutive channels of one pixel and stores 16 bytes.
+#include <atomic>
+
 #include "igemm_shared.h"
 
 namespace mi355 {
@@ -413,26 +415,27 @@ int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
     const int tab_entries = PW ? 0 : a.nstages * KCH * (PIN == 32 ? 1 : 8);
     const int lds = K::STAGE_BYTES + tab_entries * 8;
     auto kern = igemm_kernel<PIN, POUT, BM, BN, WM, WN, KCH, MINW, PW>;
-    static int max_lds_set = 0;
-    if (lds > max_lds_set) {
+    // per-instantiation caches; atomics, because operators on different streams may launch from several threads
+    static std::atomic<int> max_lds_set{0};
+    if (lds > max_lds_set.load(std::memory_order_relaxed)) {
         const int want = K::STAGE_BYTES + IG_MAX_ENTRIES * 8;
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, want);
         if (e != hipSuccess) return (int)e;
-        max_lds_set = want;
+        max_lds_set.store(want, std::memory_order_relaxed);
     }
     // persistent grid: as many workgroups as fit on the device at once
-    static int occ_lds = -1, occ_val = 0;  // last query of this instantiation
-    int occ = occ_val;
-    if (occ_lds != lds) {
+    static std::atomic<uint64_t> occ_cache{0};  // LDS bytes of the last query << 32 | its result
+    const uint64_t cached = occ_cache.load(std::memory_order_relaxed);
+    int occ = (int)(uint32_t)cached;
+    if ((cached >> 32) != (uint64_t)lds || occ < 1) {
         hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(kern),
                                                                     IG_THREADS, (size_t)lds);
         if (e != hipSuccess || occ < 1) {
             (void)hipGetLastError();
             occ = 1;
         }
-        occ_lds = lds;
-        occ_val = occ;
+        occ_cache.store(((uint64_t)lds << 32) | (uint32_t)occ, std::memory_order_relaxed);
     }
     if (cu_count <= 0) cu_count = 256;
     int64_t grid = (int64_t)occ * cu_count;

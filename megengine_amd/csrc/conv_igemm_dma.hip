@@ -20,6 +20,8 @@
 //     waves on a CU the one scalar unit paces a loop that carries it), and the last NS stages, whose refills cross
 //     into the workgroup's next tile.  The bias of the workgroup's channel tile sits in LDS, written once: tiles of
 //     one workgroup are a multiple of the channel-tile count apart whenever that count is a power of two.
+#include <atomic>
+
 #include "igemm_shared.h"
 
 namespace mi355 {
@@ -417,25 +419,26 @@ int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
     const int tab_entries = PW ? 0 : a.nstages * KCH;
     const int lds = K::RING_BYTES + tab_entries * 8;
     auto kern = igemm_dma_kernel<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW>;
-    static int max_lds_set = 0;
-    if (lds > max_lds_set) {
+    // per-instantiation caches; atomics, because operators on different streams may launch from several threads
+    static std::atomic<int> max_lds_set{0};
+    if (lds > max_lds_set.load(std::memory_order_relaxed)) {
         const int want = K::RING_BYTES + IG_MAX_ENTRIES * 8;
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, want);
         if (e != hipSuccess) return (int)e;
-        max_lds_set = want;
+        max_lds_set.store(want, std::memory_order_relaxed);
     }
-    static int occ_lds = -1, occ_val = 0;
-    int occ = occ_val;
-    if (occ_lds != lds) {
+    static std::atomic<uint64_t> occ_cache{0};  // LDS bytes of the last query << 32 | its result
+    const uint64_t cached = occ_cache.load(std::memory_order_relaxed);
+    int occ = (int)(uint32_t)cached;
+    if ((cached >> 32) != (uint64_t)lds || occ < 1) {
         hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(kern),
                                                                     K::THREADS, (size_t)lds);
         if (e != hipSuccess || occ < 1) {
             (void)hipGetLastError();
             occ = 1;
         }
-        occ_lds = lds;
-        occ_val = occ;
+        occ_cache.store(((uint64_t)lds << 32) | (uint32_t)occ, std::memory_order_relaxed);
     }
     if (cu_count <= 0) cu_count = 256;
     int64_t grid = (int64_t)occ * cu_count;
