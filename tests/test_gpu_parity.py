@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from megengine_amd import _abi, ops
+from megengine_amd import _abi, lib, ops
 from tests import util
 from tests.gpu_util import check_case, run_gpu, say, to_dev
 
@@ -327,3 +327,43 @@ def test_profile_entry_point(oracle):
     a, _ = ops.conv_bias_query(d, IGEMM)
     with pytest.raises(Mi355Error):
         ops.conv_bias_profile(d, ts, tf, tb, None, dst, a, warmup=0, iters=0)
+
+
+def test_random_descriptors_every_kernel_family(oracle):
+    """Seeded random descriptors (formats, channel counts that leave ragged tiles, filter sizes, strides, paddings,
+    residual, activation): MFMA tiles drawn at random and the heuristic against the generic kernel, bit for bit; the
+    generic kernel itself against the CPU checker on every fifth case."""
+    import random
+    rnd = random.Random(2025)
+    names = lib.tile_names()
+    for it in range(120):
+        fmt = rnd.choice(["NCHW32", "NCHW32", "NCHW32", "NCHW32_NCHW4", "NCHW4", "NCHW4_NCHW32"])
+        pin = 32 if fmt.startswith("NCHW32") else 4
+        pout = 32 if fmt in ("NCHW32", "NCHW4_NCHW32") else 4
+        n = rnd.randint(1, 9)
+        ic = rnd.choice([32, 64, 96, 128, 256, 512]) if pin == 32 else rnd.choice([4, 8, 16, 32, 64])
+        f = rnd.choice([1, 1, 3, 3, 5])
+        s = rnd.choice([1, 1, 2])
+        pad = rnd.randint(0, f // 2 + (1 if f > 1 else 0))
+        ih = rnd.randint(max(f - 2 * pad, 1) + 1, 40)
+        iw = rnd.randint(max(f - 2 * pad, 1) + 1, 40)
+        oc = rnd.randint(1, 20) * 32 if pout == 32 else rnd.randint(1, 80) * 4
+        has_z = rnd.random() < 0.5 and fmt in ("NCHW32", "NCHW4")
+        nl = rnd.choice(["IDENTITY", "RELU", "H_SWISH"])
+        d = _abi.make_conv_desc(fmt, n, ic, ih, iw, oc, f, pad=pad, stride=s, nonline=nl, has_z=has_z,
+                                scale_bias=rnd.choice([2e-4, 3.3e-5, 1e-3]), scale_z=rnd.choice([0.05, 0.013]),
+                                scale_dst=rnd.choice([0.05, 0.021, 0.2]))
+        say("random case", it, fmt, "n", n, "ic", ic, "hw", ih, iw, "oc", oc, "f", f, "s", s, "pad", pad, "z", has_z, nl)
+        src, flt, bias, z = util.make_tensors(d, seed=300 + it, bias_range=(-20000, 20000))
+        ts, tf, tb, tz = to_dev(src), to_dev(flt), to_dev(bias), to_dev(z)
+        ref = ops.conv_bias_exec(d, ts, tf, tb, tz, algo=DIRECT)
+        if it % 5 == 0:
+            torch.cuda.synchronize()
+            assert np.array_equal(ref.cpu().numpy(), oracle.conv_bias(d, src, flt, bias, z))
+        for tile in rnd.sample(range(len(names)), 4) + [None]:
+            a, _ = ops.conv_bias_query(d, IGEMM)
+            if tile is not None:
+                a.tile_cfg = tile
+            out = ops.conv_bias_exec(d, ts, tf, tb, tz, algo=a)
+            torch.cuda.synchronize()
+            assert torch.equal(out, ref), "tile %s" % (names[tile] if tile is not None else "heuristic")
