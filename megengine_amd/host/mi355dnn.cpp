@@ -530,4 +530,53 @@ void RelayoutFormat::exec(const TensorND& src, const TensorND& dst, const Worksp
     check_abi(mi355_relayout_exec(m_handle->stream(), &d, src.raw_ptr, dst.raw_ptr));
 }
 
+// ---------------------------------------------------------------- elementwise requantisation
+static void requant_exec(Handle* h, uint32_t nonline, const TensorND& a, const TensorND* b, const TensorND& dst) {
+    HOST_ASSERT(dst.layout.dtype.enumv == DTypeEnum::QuantizedS8, MI355_ERR_UNSUPPORTED, "dst must be QuantizedS8");
+    HOST_ASSERT(a.layout.dtype.enumv == DTypeEnum::QuantizedS8 || a.layout.dtype.enumv == DTypeEnum::QuantizedS32,
+                MI355_ERR_UNSUPPORTED, "the first operand must be QuantizedS8 or QuantizedS32");
+    HOST_ASSERT(a.layout.eq_shape(dst.layout) && a.layout.is_contiguous() && dst.layout.is_contiguous(), MI355_ERR_SHAPE,
+                "operands must be contiguous and of the dst shape %s", dst.layout.to_string().c_str());
+    mi355_requant_desc d = mi355_requant_desc();
+    d.nonline = nonline;
+    d.scale_src = a.layout.dtype.scale;
+    d.scale_dst = dst.layout.dtype.scale;
+    d.scale_z = 1.f;
+    d.count = dst.layout.total_nr_elems();
+    const int8_t* zp = nullptr;
+    if (b) {
+        HOST_ASSERT(b->layout.dtype.enumv == DTypeEnum::QuantizedS8, MI355_ERR_UNSUPPORTED,
+                    "the second operand must be QuantizedS8");
+        HOST_ASSERT(b->layout.eq_shape(dst.layout) && b->layout.is_contiguous(), MI355_ERR_SHAPE,
+                    "operands must be contiguous and of the dst shape %s", dst.layout.to_string().c_str());
+        d.has_z = 1;
+        d.scale_z = b->layout.dtype.scale;
+        zp = (const int8_t*)b->raw_ptr;
+        HOST_ASSERT(zp, MI355_ERR_BAD_ARG, "null tensor pointer");
+    }
+    HOST_ASSERT(a.raw_ptr && dst.raw_ptr, MI355_ERR_BAD_ARG, "null tensor pointer");
+    if (a.layout.dtype.enumv == DTypeEnum::QuantizedS32)
+        check_abi(mi355_requant_s32_s8_exec(h->stream(), &d, (const int32_t*)a.raw_ptr, zp, (int8_t*)dst.raw_ptr));
+    else
+        check_abi(mi355_requant_s8_s8_exec(h->stream(), &d, (const int8_t*)a.raw_ptr, zp, (int8_t*)dst.raw_ptr));
+}
+
+void ElemwiseMultiType::exec(const std::vector<TensorND>& src, const TensorND& dst) {
+    using Mode = Param::Mode;
+    uint32_t nl = MI355_NL_IDENTITY;
+    size_t arity = 2;
+    switch (m_param.mode) {
+        case Mode::QADD: break;
+        case Mode::QFUSE_ADD_RELU: nl = MI355_NL_RELU; break;
+        case Mode::QFUSE_ADD_H_SWISH: nl = MI355_NL_H_SWISH; break;
+        case Mode::QRELU: nl = MI355_NL_RELU; arity = 1; break;
+        case Mode::QH_SWISH: nl = MI355_NL_H_SWISH; arity = 1; break;
+        default: fail(MI355_ERR_UNSUPPORTED, "ElemwiseMultiType mode " + std::to_string((unsigned)m_param.mode) + " is not implemented");
+    }
+    HOST_ASSERT(src.size() == arity, MI355_ERR_BAD_ARG, "mode takes %zu operands, got %zu", arity, src.size());
+    requant_exec(m_handle, nl, src[0], arity == 2 ? &src[1] : nullptr, dst);
+}
+
+void TypeCvt::exec(const TensorND& src, const TensorND& dst) { requant_exec(m_handle, MI355_NL_IDENTITY, src, nullptr, dst); }
+
 }  // namespace mi355dnn

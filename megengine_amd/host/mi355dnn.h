@@ -261,6 +261,33 @@ private:
     Param m_param;
 };
 
+// The quantized modes of megdnn::ElemwiseMultiType (dnn/include/megdnn/oprs/nn_int.h:12) that sit around ConvBias in
+// an int8 network: dst = quantize(mode(dequantize(a) [, dequantize(b)])).  First operand QuantizedS8 or QuantizedS32,
+// second (binary modes) QuantizedS8, dst QuantizedS8; contiguous tensors of one shape.
+class ElemwiseMultiType : public OperatorBase {
+public:
+    struct Param {
+        // values of param::ElemwiseMultiType::Mode (dnn/scripts/opr_param_defs.py:479-529)
+        enum class Mode : uint32_t { QADD = 6, QFUSE_ADD_RELU = 7, QRELU = 15, QH_SWISH = 51, QFUSE_ADD_H_SWISH = 52 };
+        Mode mode = Mode::QADD;
+    };
+    explicit ElemwiseMultiType(Handle* h) : OperatorBase(h) {}
+    Param& param() { return m_param; }
+    const Param& param() const { return m_param; }
+    // src: one tensor for QRELU / QH_SWISH, two for the QADD family
+    void exec(const std::vector<TensorND>& src, const TensorND& dst);
+
+private:
+    Param m_param;
+};
+
+// megdnn::TypeCvt (dnn/include/megdnn/oprs/general.h:890) for QuantizedS32 / QuantizedS8 -> QuantizedS8
+class TypeCvt : public OperatorBase {
+public:
+    explicit TypeCvt(Handle* h) : OperatorBase(h) {}
+    void exec(const TensorND& src, const TensorND& dst);
+};
+
 // One handle <-> one device and one stream; the caller keeps ownership of the stream.
 class Handle {
 public:

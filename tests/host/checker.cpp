@@ -367,6 +367,68 @@ static void run_cache_roundtrip() {
     c.clear();
 }
 
+// ------------------------------------------------------------------ elementwise requantisation (GPU)
+extern "C" int oracle_requant_s32_s8(const mi355_requant_desc* d, const int32_t* src, const int8_t* z, int8_t* dst);
+extern "C" int oracle_requant_s8_s8(const mi355_requant_desc* d, const int8_t* src, const int8_t* z, int8_t* dst);
+
+static void run_elemwise_gpu(Handle* h) {
+    printf("case: ElemwiseMultiType quantized modes and TypeCvt\n");
+    fflush(stdout);
+    using EM = ElemwiseMultiType::Param::Mode;
+    const size_t n = 100003;  // ragged tail
+    const TensorShape shp{n};
+    std::vector<int8_t> ha(n), hb(n), expect(n), got(n);
+    std::vector<int32_t> ha32(n);
+    fill_s8(ha, 31, -128, 127);
+    fill_s8(hb, 32, -128, 127);
+    fill_s32(ha32, 33, -60000, 60000);
+    DevBuf da(n), db(n), da32(n * 4), dd(n);
+    HIP_OK(hipMemcpy(da.p, ha.data(), n, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(db.p, hb.data(), n, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(da32.p, ha32.data(), n * 4, hipMemcpyHostToDevice));
+    const float s_a = 0.031f, s_b = 0.022f, s_d = 0.047f, s_acc = 2e-4f;
+    TensorLayout la(shp, dtype::QuantizedS8(s_a)), lb(shp, dtype::QuantizedS8(s_b)), ld(shp, dtype::QuantizedS8(s_d));
+    TensorLayout la32(shp, dtype::QuantizedS32(s_acc));
+    auto opr = h->create_operator<ElemwiseMultiType>();
+    struct M { EM mode; uint32_t nl; bool binary; const char* name; };
+    const M modes[] = {{EM::QADD, MI355_NL_IDENTITY, true, "QADD"}, {EM::QFUSE_ADD_RELU, MI355_NL_RELU, true, "QFUSE_ADD_RELU"},
+                       {EM::QFUSE_ADD_H_SWISH, MI355_NL_H_SWISH, true, "QFUSE_ADD_H_SWISH"}, {EM::QRELU, MI355_NL_RELU, false, "QRELU"},
+                       {EM::QH_SWISH, MI355_NL_H_SWISH, false, "QH_SWISH"}};
+    for (int s32 = 0; s32 < 2; ++s32)
+        for (auto& m : modes) {
+            mi355_requant_desc d = mi355_requant_desc();
+            d.nonline = m.nl; d.has_z = m.binary; d.scale_src = s32 ? s_acc : s_a; d.scale_z = s_b; d.scale_dst = s_d; d.count = n;
+            int st = s32 ? oracle_requant_s32_s8(&d, ha32.data(), m.binary ? hb.data() : nullptr, expect.data())
+                         : oracle_requant_s8_s8(&d, ha.data(), m.binary ? hb.data() : nullptr, expect.data());
+            EXPECT(st == 0, "CPU checker refused %s", m.name);
+            opr->param().mode = m.mode;
+            std::vector<TensorND> src{s32 ? TensorND(da32.p, la32) : TensorND(da.p, la)};
+            if (m.binary) src.push_back(TensorND(db.p, lb));
+            HIP_OK(hipMemset(dd.p, 0x5a, n));
+            opr->exec(src, TensorND(dd.p, ld));
+            HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
+            HIP_OK(hipMemcpy(got.data(), dd.p, n, hipMemcpyDeviceToHost));
+            size_t bad = 0;
+            for (size_t i = 0; i < n; ++i) bad += got[i] != expect[i];
+            EXPECT(bad == 0, "%s (%s first operand): %zu of %zu bytes differ", m.name, s32 ? "s32" : "s8", bad, n);
+        }
+    // TypeCvt s32 -> s8 and the wrong arity
+    {
+        mi355_requant_desc d = mi355_requant_desc();
+        d.nonline = MI355_NL_IDENTITY; d.scale_src = s_acc; d.scale_z = 1.f; d.scale_dst = s_d; d.count = n;
+        EXPECT(oracle_requant_s32_s8(&d, ha32.data(), nullptr, expect.data()) == 0, "CPU checker refused TypeCvt");
+        auto cvt = h->create_operator<TypeCvt>();
+        cvt->exec(TensorND(da32.p, la32), TensorND(dd.p, ld));
+        HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
+        HIP_OK(hipMemcpy(got.data(), dd.p, n, hipMemcpyDeviceToHost));
+        size_t bad = 0;
+        for (size_t i = 0; i < n; ++i) bad += got[i] != expect[i];
+        EXPECT(bad == 0, "TypeCvt: %zu bytes differ", bad);
+        opr->param().mode = EM::QADD;
+        EXPECT(throws([&] { opr->exec({TensorND(da.p, la)}, TensorND(dd.p, ld)); }, MI355_ERR_BAD_ARG), "QADD with one operand");
+    }
+}
+
 // ------------------------------------------------------------------ fast-run (GPU)
 static void run_fast_run_gpu(Handle* h) {
     printf("case: fast-run profiling\n");
@@ -447,6 +509,7 @@ int main(int argc, char** argv) {
         run_cache_roundtrip();
         for (auto& c : cases()) run_conv_case(handle.get(), c, gpu);
         if (gpu) run_relayout_gpu(handle.get());
+        if (gpu) run_elemwise_gpu(handle.get());
         if (gpu) run_fast_run_gpu(handle.get());
     } catch (const Error& e) {
         printf("unexpected mi355dnn::Error %d: %s\n", e.status(), e.what());
