@@ -521,7 +521,7 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
         if (OC <= 64) return kbytes <= 64 ? D128x128x64w8 : kbytes <= 256 ? D64x64x128r2 : D64x128x128r2;
         const int64_t t128 = tiles(0);
         if (t128 >= 4 * cu_count)
-            return kbytes >= 1024 ? (OC >= 256 ? D256x128x64w8 : D128x128x128r2) : (kbytes <= 128 ? D128x128x64w8 : 0);
+            return kbytes >= 1024 ? (OC >= 256 ? D256x128x64w8 : D128x128x128r2) : (kbytes <= 128 ? D128x128x64w8 : D128x128x128r2w8);
         if (t128 >= 2 * cu_count) return D128x64x128r2;
         if (2 * t128 >= 3 * cu_count) return kbytes >= 512 ? D128x128x128r2w8 : D128x128x64;
         // few tiles, long reductions: the deeper ring hides the cold first touch of every weight byte; the longest
