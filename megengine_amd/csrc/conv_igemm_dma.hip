@@ -44,6 +44,18 @@ __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+// a dword load the compiler does not wait for: the value is valid only after wait_vmcnt_for on it
+__device__ __forceinline__ int load_dword_async(int voff, const v4i& rsrc) {
+    int v;
+    asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=v"(v) : "v"(voff), "s"(rsrc) : "memory");
+    return v;
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_for(int& v) {
+    static_assert(N >= 0 && N < 64, "vmcnt range");
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N) : "memory");
+}
+
 __device__ __forceinline__ v4i uniform_rsrc(const void* p, uint32_t bytes) {
     const uint64_t a = (uint64_t)(uintptr_t)p;
     v4i r;
@@ -133,9 +145,12 @@ struct DmaKernel {
         L.kc0 = 0;
     }
 
-    // copies of one stage into ring buffer `buf` (LDS byte address lds0 + buf * STG); always U copies per wave
+    // copies of one stage into ring buffer `buf` (LDS byte address lds0 + buf * STG); always U copies per wave.
+    // PF: the caller already holds this lane's table entry (*pk), read one iteration ahead
+    template <bool PF = false>
     __device__ static __forceinline__ void issue(const IgemmArgs& a, const Loader& L, const KEntry* tab, const v4i& rs_src,
-                                                 const v4i& rs_flt, uint32_t stage_addr, int w, int lane) {
+                                                 const v4i& rs_flt, uint32_t stage_addr, int w, int lane,
+                                                 const KEntry* pk = nullptr) {
         const int a_k = L.kc0 * 32;
 #pragma unroll
         for (int j = 0; j < UA; ++j) {
@@ -149,7 +164,7 @@ struct DmaKernel {
                 lds_copy64x16(stage_addr + (uint32_t)(A_BYTES + (NW * j + w) * 1024), L.b_off[j] + b_k, rs_src);
             }
         } else {
-            const KEntry k = tab[L.kc0 + (slot_of(w, lane) >> 1)];  // this lane's k-chunk: channel block and tap
+            const KEntry k = PF ? *pk : tab[L.kc0 + (slot_of(w, lane) >> 1)];  // this lane's k-chunk: channel block and tap
             const int fh = k.fhfw & 0xffff, fw = k.fhfw >> 16;
 #pragma unroll
             for (int j = 0; j < UB; ++j) {
@@ -210,13 +225,16 @@ struct DmaKernel {
         const int my_tiles = first < last ? (last - first + step - 1) / step : 0;
         const int total = my_tiles * a.nstages;
 
-        // The bias of the workgroup's channel tile lives in LDS, written once before the first barrier: workgroups
+        // The bias of the workgroup's channel tile lives in LDS, written once after the prologue's copies are issued: workgroups
         // mostly stay on one channel tile (their tile stride is a multiple of the number of channel tiles whenever
         // that is a power of two), so the copy is read at every tile start and almost never rewritten.
         int* sBias = reinterpret_cast<int*>(lds + NS * STG);
         int c_tile = first, c_oc0, c_pix0;
         tile_coords(a, c_tile, c_oc0, c_pix0);
-        if (t < BM) sBias[t] = fetch_bias(a, c_oc0, t);
+        // requested now, written to LDS only after the prologue's copies are on their way: the first touch of the bias
+        // (a cold miss) overlaps theirs instead of preceding it.  Without a bias the buffer has no bytes: every lane reads 0
+        const v4i rs_bias = uniform_rsrc(a.bias, a.has_bias ? (uint32_t)a.OC * 4u : 0u);
+        int bias_reg = load_dword_async(t < BM ? (c_oc0 + t) * 4 : SENT, rs_bias);
 
         if (!PW) {
             const int cap = a.nstages * KCH;
@@ -257,7 +275,7 @@ struct DmaKernel {
             if (issued >= total) loader_kill(L);
         };
 
-        __syncthreads();  // table ready
+        if (!PW) __syncthreads();  // table ready
 
         // prologue: stages 0 .. NS - 2 go to buffers 0 .. NS - 2
 #pragma unroll
@@ -266,6 +284,9 @@ struct DmaKernel {
             advance();
         }
         v16i acc[MT][NT];
+        wait_vmcnt_for<(NS - 1) * U>(bias_reg);  // older than every copy of the prologue
+        if (t < BM) sBias[t] = bias_reg;
+        __syncthreads();
         init_acc_lds(acc, sBias, wm, lh);
         int rd_off = 0;                                     // byte offset of the stage being multiplied
         uint32_t wr_addr = lds0 + (uint32_t)((NS - 1) * STG);  // LDS address of the stage buffer refilled next
@@ -326,14 +347,17 @@ struct DmaKernel {
         const int steady = a.nstages > NS ? a.nstages - NS : 0;
         for (int ti = 0; ti < my_tiles; ++ti) {
             if (DUAL) alt = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            KEntry nk;  // the table entry of the next refill, read while the current stage multiplies
+            if (!PW && steady > 0) nk = tab[L.kc0 + (slot_of(wave, lane) >> 1)];
             for (int s = 0; s < steady; ++s) {
                 // this wave's copies of the stage have landed once at most the NS - 2 younger stages are in flight
                 wait_vmcnt<(NS - 2) * U>();
                 __syncthreads();  // ... of every wave; and every wave is done reading the buffer refilled next
-                issue(a, L, tab, rs_src, rs_flt, wr_addr, wave, lane);
+                issue<!PW>(a, L, tab, rs_src, rs_flt, wr_addr, wave, lane, &nk);
                 ++issued;
                 ++L.stage;
                 L.kc0 += KCH;
+                if (!PW) nk = tab[L.kc0 + (slot_of(wave, lane) >> 1)];
                 multiply();
             }
             ZRegs<MT, NT> zr;
