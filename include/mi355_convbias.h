@@ -237,6 +237,25 @@ int mi355_requant_s32_s8_exec(void* stream, const mi355_requant_desc* d, const i
  * All three tensors need 16-byte alignment. */
 int mi355_requant_s8_s8_exec(void* stream, const mi355_requant_desc* d, const int8_t* src, const int8_t* z, int8_t* dst);
 
+/* ---- Pooling forward on QuantizedS8 (src and dst share one scale: the stored bytes are pooled) ----
+ * megdnn::PoolingForward (dnn/include/megdnn/oprs/nn.h PoolingForward::exec; param::Pooling,
+ * dnn/scripts/opr_param_defs.py:233-254) with the naive arithmetic (dnn/src/naive/pooling/opr_impl.cpp:16-36,
+ * :107-127, :237-289): MAX over the part of the window inside the image; AVERAGE = roundf(float(sum) / (window_h *
+ * window_w)), padding counted as zeros; AVERAGE_COUNT_EXCLUDE_PADDING = roundf(float(sum) / float(elements inside)).
+ * format: MI355_FMT_NCHW, MI355_FMT_NCHW4, MI355_FMT_NCHW44 or MI355_FMT_NCHW32 (c a multiple of the pack).
+ * Output size (dnn/src/common/pooling.cpp:7-125): (i + 2 * pad - window) / stride + 1.  A window that lies outside
+ * the image completely is an error for MAX and AVERAGE_COUNT_EXCLUDE_PADDING, as in the reference (its message:
+ * "The pooling window lies outside completely").  NCHW4 tensors need 4-byte, NCHW32 tensors 16-byte alignment. */
+enum { MI355_POOL_MAX = 0, MI355_POOL_AVERAGE = 1, MI355_POOL_AVERAGE_COUNT_EXCLUDE_PADDING = 2 };
+typedef struct mi355_pooling_desc {
+    uint32_t mode;     /* MI355_POOL_* */
+    uint32_t format;   /* MI355_FMT_* */
+    uint32_t n, c, ih, iw;
+    uint32_t pad_h, pad_w, stride_h, stride_w, window_h, window_w;
+} mi355_pooling_desc;
+int mi355_pooling_deduce_out(const mi355_pooling_desc* d, uint32_t* oh, uint32_t* ow);
+int mi355_pooling_s8_exec(void* stream, const mi355_pooling_desc* d, const int8_t* src, int8_t* dst);
+
 #ifdef __cplusplus
 }
 #endif

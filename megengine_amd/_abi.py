@@ -81,6 +81,36 @@ class RequantDesc(C.Structure):
     ]
 
 
+# param::Pooling::Mode
+POOL_MAX, POOL_AVERAGE, POOL_AVERAGE_COUNT_EXCLUDE_PADDING = 0, 1, 2
+POOL_NAMES = {"MAX": POOL_MAX, "AVERAGE": POOL_AVERAGE, "AVERAGE_COUNT_EXCLUDE_PADDING": POOL_AVERAGE_COUNT_EXCLUDE_PADDING}
+
+
+class PoolingDesc(C.Structure):
+    _fields_ = [
+        ("mode", C.c_uint32), ("format", C.c_uint32),
+        ("n", C.c_uint32), ("c", C.c_uint32), ("ih", C.c_uint32), ("iw", C.c_uint32),
+        ("pad_h", C.c_uint32), ("pad_w", C.c_uint32), ("stride_h", C.c_uint32), ("stride_w", C.c_uint32),
+        ("window_h", C.c_uint32), ("window_w", C.c_uint32),
+    ]
+
+
+def make_pooling_desc(mode, fmt, n, c, ih, iw, window, stride=None, pad=0):
+    """window / stride / pad: an int or an (h, w) pair; stride defaults to the window (param::Pooling defaults are 2, 2)."""
+    two = lambda v: (v, v) if isinstance(v, int) else tuple(v)
+    wh, ww = two(window)
+    sh, sw = two(window if stride is None else stride)
+    ph, pw = two(pad)
+    return PoolingDesc(mode=POOL_NAMES.get(mode, mode), format=FORMAT_NAMES.get(fmt, fmt), n=n, c=c, ih=ih, iw=iw,
+                       pad_h=ph, pad_w=pw, stride_h=sh, stride_w=sw, window_h=wh, window_w=ww)
+
+
+def packed_shape(fmt, n, c, h, w):
+    """Tensor shape of (n, c, h, w) activations in a ConvBias / Pooling format."""
+    p = {FMT_NCHW: 1, FMT_NCHW4: 4, FMT_NCHW44: 4, FMT_NCHW32: 32}[FORMAT_NAMES.get(fmt, fmt)]
+    return (n, c, h, w) if p == 1 else (n, c // p, h, w, p)
+
+
 def in_pack(fmt):
     return {FMT_NCHW: 1, FMT_NCHW4: 4, FMT_NCHW44: 4, FMT_NCHW4_NCHW32: 4, FMT_NCHW4_NCHW: 4}.get(fmt, 32)
 

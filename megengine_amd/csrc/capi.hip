@@ -374,6 +374,59 @@ int mi355_requant_s8_s8_exec(void* stream, const mi355_requant_desc* d, const in
     return MI355_OK;
 }
 
+// ---- Pooling ----
+static int pooling_check(const mi355_pooling_desc* d, int* pack, uint32_t* oh, uint32_t* ow) {
+    if (!d) return fail(MI355_ERR_BAD_ARG, "null descriptor");
+    if (d->mode > MI355_POOL_AVERAGE_COUNT_EXCLUDE_PADDING) return fail(MI355_ERR_UNSUPPORTED, "pooling mode %u", d->mode);
+    switch (d->format) {
+        case MI355_FMT_NCHW: *pack = 1; break;
+        case MI355_FMT_NCHW4:
+        case MI355_FMT_NCHW44: *pack = 4; break;
+        case MI355_FMT_NCHW32: *pack = 32; break;
+        default: return fail(MI355_ERR_UNSUPPORTED, "invalid pooling format %u", d->format);
+    }
+    if (d->c % (uint32_t)*pack) return fail(MI355_ERR_SHAPE, "channels %u not a multiple of %d", d->c, *pack);
+    if (!d->window_h || !d->window_w || !d->stride_h || !d->stride_w) return fail(MI355_ERR_SHAPE, "zero window or stride");
+    if ((uint64_t)d->ih + 2ull * d->pad_h < d->window_h || (uint64_t)d->iw + 2ull * d->pad_w < d->window_w)
+        return fail(MI355_ERR_SHAPE, "window %ux%u larger than the padded input %ux%u", d->window_h, d->window_w,
+                    d->ih + 2 * d->pad_h, d->iw + 2 * d->pad_w);
+    if (d->ih > (1u << 24) || d->iw > (1u << 24) || d->pad_h > (1u << 24) || d->pad_w > (1u << 24) ||
+        (uint64_t)d->window_h * d->window_w > 65535)
+        return fail(MI355_ERR_SHAPE, "pooling geometry out of range");
+    *oh = (d->ih + 2 * d->pad_h - d->window_h) / d->stride_h + 1;
+    *ow = (d->iw + 2 * d->pad_w - d->window_w) / d->stride_w + 1;
+    return MI355_OK;
+}
+
+int mi355_pooling_deduce_out(const mi355_pooling_desc* d, uint32_t* oh, uint32_t* ow) {
+    if (!oh || !ow) return fail(MI355_ERR_BAD_ARG, "null argument");
+    int pack;
+    return pooling_check(d, &pack, oh, ow);
+}
+
+int mi355_pooling_s8_exec(void* stream, const mi355_pooling_desc* d, const int8_t* src, int8_t* dst) {
+    int pack;
+    uint32_t oh, ow;
+    int rc = pooling_check(d, &pack, &oh, &ow);
+    if (rc) return rc;
+    const uint64_t out_elems = (uint64_t)d->n * d->c * oh * ow;
+    if (out_elems == 0) return MI355_OK;
+    if ((uint64_t)d->n * d->c * d->ih * d->iw == 0) return fail(MI355_ERR_SHAPE, "empty input with a non-empty output");
+    if (out_elems / (pack == 32 ? 16 : pack) >= (1ull << 31)) return fail(MI355_ERR_SHAPE, "pooling output too large");
+    if (!src || !dst) return fail(MI355_ERR_BAD_ARG, "null tensor pointer");
+    const uintptr_t al = pack == 32 ? 15 : pack == 4 ? 3 : 0;
+    if (((uintptr_t)src & al) || ((uintptr_t)dst & al)) return fail(MI355_ERR_BAD_ARG, "src and dst need %d-byte alignment", (int)al + 1);
+    if (d->mode != MI355_POOL_AVERAGE) {
+        // the last window along an axis starts at (o - 1) * stride - pad; the first ends at window - pad
+        const bool out_h = d->pad_h >= d->window_h || (uint64_t)(oh - 1) * d->stride_h >= (uint64_t)d->ih + d->pad_h;
+        const bool out_w = d->pad_w >= d->window_w || (uint64_t)(ow - 1) * d->stride_w >= (uint64_t)d->iw + d->pad_w;
+        if (out_h || out_w) return fail(MI355_ERR_SHAPE, "The pooling window lies outside completely");
+    }
+    rc = launch_pooling(reinterpret_cast<hipStream_t>(stream), *d, pack, oh, ow, src, dst, cu_count());
+    if (rc) return fail(MI355_ERR_LAUNCH, "pooling: %s", hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
+}
+
 int mi355_igemm_tile_count(void) { return igemm_num_cfgs(); }
 const char* mi355_igemm_tile_name(int cfg) { return igemm_cfg_name(cfg); }
 

@@ -136,3 +136,22 @@ def requant_exec(src, scale_src, scale_dst, nonline="IDENTITY", z=None, scale_z=
     fn = lib().mi355_requant_s32_s8_exec if src.dtype == torch.int32 else lib().mi355_requant_s8_s8_exec
     check(fn(_stream(), C.byref(d), _ptr(src), _ptr(z), _ptr(dst)))
     return dst
+
+
+def pooling_deduce_layout(d):
+    """Output shape of megdnn::PoolingForward for the descriptor (dnn/src/common/pooling.cpp:7-125)."""
+    oh, ow = C.c_uint32(), C.c_uint32()
+    check(lib().mi355_pooling_deduce_out(C.byref(d), C.byref(oh), C.byref(ow)))
+    return _abi.packed_shape(d.format, d.n, d.c, oh.value, ow.value)
+
+
+def pooling_exec(d, src, dst=None):
+    """megdnn::PoolingForward::exec on a QuantizedS8 tensor (dst carries the scale of src)."""
+    if src.dtype != torch.int8:
+        raise RuntimeError("pooling_exec takes an int8 tensor")
+    if tuple(src.shape) != _abi.packed_shape(d.format, d.n, d.c, d.ih, d.iw):
+        raise RuntimeError("src shape %s does not match the descriptor" % (tuple(src.shape),))
+    if dst is None:
+        dst = torch.empty(pooling_deduce_layout(d), dtype=torch.int8, device=src.device)
+    check(lib().mi355_pooling_s8_exec(_stream(), C.byref(d), _ptr(src), _ptr(dst)))
+    return dst

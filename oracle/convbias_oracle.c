@@ -1,6 +1,6 @@
 /*
- * convbias_oracle.c -- CPU restatement of MegDNN's naive quantized ConvBias and
- * RelayoutFormat.  TEST INFRASTRUCTURE ONLY: the parity checker for tests/, the smoke
+ * convbias_oracle.c -- CPU restatement of MegDNN's naive quantized ConvBias,
+ * RelayoutFormat, the requantising elementwise operators and QuantizedS8 Pooling.  TEST INFRASTRUCTURE ONLY: the parity checker for tests/, the smoke
  * check and the bench's cpu_baseline leg.  Nothing in the product library links, calls
  * or falls back to this file.
  *
@@ -114,6 +114,72 @@ int oracle_requant_s8_s8(const mi355_requant_desc* d, const int8_t* src, const i
         dst[i] = oracle_epilogue_s8((int32_t)src[i], d->scale_src, d->has_z != 0, d->has_z ? z[i] : 0, d->scale_z,
                                     (int)d->nonline, d->scale_dst);
     return MI355_OK;
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* Pooling forward on dt_qint8                                                           */
+/* ------------------------------------------------------------------------------------ */
+
+/* element index of (n, c, h, w): the IdxGetters of dnn/src/naive/pooling/opr_impl.cpp:129-186
+ * (NCHW :129-135, NCHW4 :153-159, NCHW44 :168-175, NCHW32 :185-191) */
+static size_t pool_idx(int pack, size_t n, size_t c, size_t h, size_t w, size_t C, size_t H, size_t W) {
+    if (pack == 1) return ((n * C + c) * H + h) * W + w;
+    return (((n * (C / (size_t)pack) + c / (size_t)pack) * H + h) * W + w) * (size_t)pack + c % (size_t)pack;
+}
+
+/* pooling_forward_impl (naive/pooling/opr_impl.cpp:270-289) with the dt_qint8 poolers: MaxPooler (:16-36),
+ * MeanIncludePooler<dt_qint8> = MeanIncludeRoundedPooler (:107-127: round(float(sum) / count), count = window),
+ * MeanExcludePooler<dt_qint8> = MeanExcludeRoundedPooler (:237-268: count = elements fed).  The bounds test uses the
+ * reference's unsigned wrap-around (ih = -PH + oh * SH + fh as size_t, valid when < IH).  A window without a
+ * valid element makes MAX and the excluding mean throw: status MI355_ERR_SHAPE here. */
+int oracle_pooling_s8(const mi355_pooling_desc* d, const int8_t* src, int8_t* dst) {
+    int pack;
+    switch (d->format) {
+        case MI355_FMT_NCHW: pack = 1; break;
+        case MI355_FMT_NCHW4:
+        case MI355_FMT_NCHW44: pack = 4; break;
+        case MI355_FMT_NCHW32: pack = 32; break;
+        default: return MI355_ERR_UNSUPPORTED;
+    }
+    if (d->mode > MI355_POOL_AVERAGE_COUNT_EXCLUDE_PADDING) return MI355_ERR_UNSUPPORTED;
+    const size_t N = d->n, C = d->c, IH = d->ih, IW = d->iw;
+    const size_t PH = d->pad_h, PW = d->pad_w, SH = d->stride_h, SW = d->stride_w, FH = d->window_h, FW = d->window_w;
+    if (C % (size_t)pack || !FH || !FW || !SH || !SW || IH + 2 * PH < FH || IW + 2 * PW < FW) return MI355_ERR_SHAPE;
+    const size_t OH = (IH + 2 * PH - FH) / SH + 1, OW = (IW + 2 * PW - FW) / SW + 1;
+    int status = MI355_OK;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (size_t n = 0; n < N; ++n)
+        for (size_t c = 0; c < C; ++c)
+            for (size_t oh = 0; oh < OH; ++oh)
+                for (size_t ow = 0; ow < OW; ++ow) {
+                    int8_t best = INT8_MIN;
+                    int32_t sum = 0;
+                    size_t fed = 0;
+                    for (size_t fh = 0; fh < FH; ++fh)
+                        for (size_t fw = 0; fw < FW; ++fw) {
+                            const size_t ih = -PH + oh * SH + fh, iw = -PW + ow * SW + fw;
+                            if (ih < IH && iw < IW) {
+                                const int8_t x = src[pool_idx(pack, n, c, ih, iw, C, IH, IW)];
+                                best = best > x ? best : x;
+                                sum += (int32_t)x;
+                                ++fed;
+                            }
+                        }
+                    int8_t r;
+                    if (d->mode == MI355_POOL_AVERAGE) {
+                        const int32_t count = (int32_t)(FH * FW);
+                        r = (int8_t)roundf((float)sum / count);
+                    } else if (!fed) {
+                        status = MI355_ERR_SHAPE;
+                        r = 0;
+                    } else if (d->mode == MI355_POOL_MAX) {
+                        r = best;
+                    } else {
+                        r = (int8_t)roundf((float)sum / fed);
+                    }
+                    dst[pool_idx(pack, n, c, oh, ow, C, OH, OW)] = r;
+                }
+    return status;
 }
 
 /* infer_conv_shape, dnn/src/common/utils.cpp:130-138 */

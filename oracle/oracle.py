@@ -53,6 +53,8 @@ def lib():
         L.oracle_fastdiv_sweep.argtypes = [C.c_float, C.c_uint32, C.c_uint32, C.c_uint64, P(C.c_float)]
         L.oracle_round_sweep.restype = C.c_uint64
         L.oracle_round_sweep.argtypes = [C.c_uint32, C.c_uint32, P(C.c_float)]
+        L.oracle_pooling_s8.restype = C.c_int
+        L.oracle_pooling_s8.argtypes = [P(_abi.PoolingDesc), C.c_void_p, C.c_void_p]
         _LIB = L
     return _LIB
 
@@ -150,6 +152,19 @@ def requant(src, scale_src, scale_dst, nonline=0, z=None, scale_z=1.0):
     dst = np.empty(src.shape, np.int8)
     zc = None if z is None else np.ascontiguousarray(z, dtype=np.int8)
     st = lib().oracle_requant_s32_s8(C.byref(d), _ptr(src), _ptr(zc) if zc is not None else None, _ptr(dst))
+    if st:
+        raise OracleError(st)
+    return dst
+
+
+def pooling(d, src):
+    """QuantizedS8 Pooling forward of an int8 array laid out in d.format; returns the int8 result"""
+    src = np.ascontiguousarray(src, dtype=np.int8)
+    assert src.shape == _abi.packed_shape(d.format, d.n, d.c, d.ih, d.iw), (src.shape, d.format)
+    oh = (d.ih + 2 * d.pad_h - d.window_h) // d.stride_h + 1
+    ow = (d.iw + 2 * d.pad_w - d.window_w) // d.stride_w + 1
+    dst = np.zeros(_abi.packed_shape(d.format, d.n, d.c, oh, ow), np.int8)
+    st = lib().oracle_pooling_s8(C.byref(d), _ptr(src), _ptr(dst))
     if st:
         raise OracleError(st)
     return dst

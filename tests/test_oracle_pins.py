@@ -459,3 +459,83 @@ def test_nchw4_nchw_format_and_float_dst(oracle):
         df.scale_bias, df.scale_z = 0.125, 4.0
         got2 = oracle.conv_bias(df, s, f, b, zz)
         assert np.array_equal(got2, np.maximum(acc * 0.5 + b.reshape(1, -1, 1, 1) + zz, 0).astype(np.float32))
+
+
+def _pool_brute(mode, x, window, stride, pad):
+    """NCHW pooling from the definition, in Python integers: the mean is the exact rational sum / count rounded half
+    away from zero by integer arithmetic (no float division)."""
+    n, c, ih, iw = x.shape
+    (fh, fw), (sh, sw), (ph, pw) = window, stride, pad
+    oh, ow = (ih + 2 * ph - fh) // sh + 1, (iw + 2 * pw - fw) // sw + 1
+    out = np.zeros((n, c, oh, ow), np.int8)
+    for a in range(oh):
+        for b in range(ow):
+            h0, w0 = a * sh - ph, b * sw - pw
+            win = x[:, :, max(h0, 0):min(h0 + fh, ih), max(w0, 0):min(w0 + fw, iw)].astype(np.int64)
+            if mode == "MAX":
+                out[:, :, a, b] = win.max(axis=(2, 3))
+                continue
+            s = win.sum(axis=(2, 3))
+            cnt = fh * fw if mode == "AVERAGE" else win.shape[2] * win.shape[3]
+            out[:, :, a, b] = np.sign(s) * ((2 * np.abs(s) + cnt) // (2 * cnt))
+    return out
+
+
+def _to_packed(x, p):
+    n, c, h, w = x.shape
+    return x if p == 1 else np.ascontiguousarray(x.reshape(n, c // p, p, h, w).transpose(0, 1, 3, 4, 2))
+
+
+def test_pooling_reference_vectors(oracle, kats):
+    """The reference's pooling known-answer tests.  Its quantized vectors are Quantized8Asymm with zero point 128: x - 128
+    is the same problem in QuantizedS8 (padding = zero point = 0) for MAX, and for the means wherever sum / count is not
+    a tie -- the unsigned pooler rounds (sum + 128 count) / count half up, the signed one rounds sum / count half away
+    from zero (naive/pooling/opr_impl.cpp:88-95 vs :107-127), so a negative tie lands one lower."""
+    k = kats["pooling_quantized8asymm"]
+    x = (np.array(k["src"], np.int32) - 128).astype(np.int8).reshape(1, 1, 3, 3)
+    ties = {"MAX": [0, 0, 0, 0], "AVERAGE": [1, 0, 1, 0], "AVERAGE_COUNT_EXCLUDE_PADDING": [0, 1, 0, 0]}
+    for mode in ("MAX", "AVERAGE", "AVERAGE_COUNT_EXCLUDE_PADDING"):
+        d = _abi.make_pooling_desc(mode, "NCHW", 1, 1, 3, 3, k["window"], k["stride"], k["pad"])
+        got = oracle.pooling(d, x).ravel().astype(np.int32)
+        want = np.array(k[mode], np.int32) - 128 - np.array(ties[mode])
+        assert np.array_equal(got, want), (mode, got, want)
+        # the ties are where twice the window sum is an odd multiple of the count, and they are negative
+        assert np.array_equal(got, _pool_brute(mode, x, (2, 2), (2, 2), (1, 1)).ravel())
+    k = kats["pooling_int8_average"]
+    for mode in ("AVERAGE", "AVERAGE_COUNT_EXCLUDE_PADDING"):
+        d = _abi.make_pooling_desc(mode, "NCHW", 1, 1, 3, 3, k["window"], k["stride"], k["pad"])
+        for sign in ("positive", "negative"):
+            x = np.array(k["src_" + sign], np.int8).reshape(1, 1, 3, 3)
+            assert np.array_equal(oracle.pooling(d, x).ravel(), np.array(k["dst_" + sign], np.int8))
+
+
+def test_pooling_vs_definition_and_formats(oracle):
+    """Windows, strides and padding against the definition evaluated with exact integer rounding (for windows of fewer
+    than 65536 elements the float quotient cannot reach a tie that the rational misses); packed formats are the NCHW
+    problem repacked; MAX also against torch's max_pool2d."""
+    import torch
+    rng = np.random.RandomState(77)
+    cases = [((3, 3), (2, 2), (1, 1), 12, 13), ((2, 2), (2, 2), (0, 0), 8, 10), ((3, 2), (1, 2), (1, 0), 7, 9),
+             ((5, 5), (3, 3), (2, 2), 11, 11), ((7, 7), (7, 7), (0, 0), 7, 7), ((1, 1), (1, 1), (0, 0), 4, 5),
+             ((3, 3), (1, 1), (2, 2), 6, 6)]
+    for window, stride, pad, ih, iw in cases:
+        x = rng.randint(-128, 128, (2, 64, ih, iw)).astype(np.int8)
+        x[0, 0] = -128
+        x[0, 1] = 127
+        for mode in ("MAX", "AVERAGE", "AVERAGE_COUNT_EXCLUDE_PADDING"):
+            want = _pool_brute(mode, x, window, stride, pad)
+            for fmt, p in (("NCHW", 1), ("NCHW4", 4), ("NCHW44", 4), ("NCHW32", 32)):
+                d = _abi.make_pooling_desc(mode, fmt, 2, 64, ih, iw, window, stride, pad)
+                got = oracle.pooling(d, _to_packed(x, p))
+                assert np.array_equal(got, _to_packed(want, p)), (mode, fmt, window, stride, pad)
+        if pad[0] * 2 <= window[0] and pad[1] * 2 <= window[1]:
+            t = torch.nn.functional.max_pool2d(torch.from_numpy(x.astype(np.float32)), window, stride, pad)
+            assert np.array_equal(_pool_brute("MAX", x, window, stride, pad), t.numpy().astype(np.int8))
+    # a window that lies in the padding completely: an error for MAX and the excluding mean, zero for AVERAGE
+    x = rng.randint(-128, 128, (1, 4, 4, 4)).astype(np.int8)
+    d = _abi.make_pooling_desc("AVERAGE", "NCHW", 1, 4, 4, 4, 2, 2, 2)
+    assert np.all(oracle.pooling(d, x)[:, :, 0, :] == 0)
+    for mode in ("MAX", "AVERAGE_COUNT_EXCLUDE_PADDING"):
+        d = _abi.make_pooling_desc(mode, "NCHW", 1, 4, 4, 4, 2, 2, 2)
+        with pytest.raises(oracle.OracleError):
+            oracle.pooling(d, x)
