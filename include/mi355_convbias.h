@@ -237,6 +237,13 @@ int mi355_requant_s32_s8_exec(void* stream, const mi355_requant_desc* d, const i
  * All three tensors need 16-byte alignment. */
 int mi355_requant_s8_s8_exec(void* stream, const mi355_requant_desc* d, const int8_t* src, const int8_t* z, int8_t* dst);
 
+/* TypeCvt between Float32 and QuantizedS8, the quantize / dequantize at the two ends of an int8 network
+ * (dnn/src/naive/type_cvt/opr_impl.cpp:24-56): Float32 -> QuantizedS8 is DTypeParamImpl<dt_qint8>::quantize =
+ * saturate(roundf(x / scale)) (dnn/include/megdnn/dtype.h:845-853; NaN -> -128), QuantizedS8 -> Float32 is
+ * float(x) * scale (dtype.h:854).  Contiguous tensors; the float side needs 16-byte, the int8 side 4-byte alignment. */
+int mi355_typecvt_f32_s8_exec(void* stream, uint64_t count, float scale_dst, const float* src, int8_t* dst);
+int mi355_typecvt_s8_f32_exec(void* stream, uint64_t count, float scale_src, const int8_t* src, float* dst);
+
 /* ---- Pooling forward on QuantizedS8 (src and dst share one scale: the stored bytes are pooled) ----
  * megdnn::PoolingForward (dnn/include/megdnn/oprs/nn.h PoolingForward::exec; param::Pooling,
  * dnn/scripts/opr_param_defs.py:233-254) with the naive arithmetic (dnn/src/naive/pooling/opr_impl.cpp:16-36,

@@ -374,6 +374,24 @@ int mi355_requant_s8_s8_exec(void* stream, const mi355_requant_desc* d, const in
     return MI355_OK;
 }
 
+int mi355_typecvt_f32_s8_exec(void* stream, uint64_t count, float scale_dst, const float* src, int8_t* dst) {
+    if (count == 0) return MI355_OK;
+    if (!src || !dst) return fail(MI355_ERR_BAD_ARG, "null tensor pointer");
+    if (!aligned16(src) || ((uintptr_t)dst & 3)) return fail(MI355_ERR_BAD_ARG, "src needs 16-byte, dst 4-byte alignment");
+    int rc = launch_cvt_f32_s8(reinterpret_cast<hipStream_t>(stream), scale_dst, src, dst, count, cu_count());
+    if (rc) return fail(MI355_ERR_LAUNCH, "typecvt: %s", hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
+}
+
+int mi355_typecvt_s8_f32_exec(void* stream, uint64_t count, float scale_src, const int8_t* src, float* dst) {
+    if (count == 0) return MI355_OK;
+    if (!src || !dst) return fail(MI355_ERR_BAD_ARG, "null tensor pointer");
+    if (((uintptr_t)src & 3) || !aligned16(dst)) return fail(MI355_ERR_BAD_ARG, "src needs 4-byte, dst 16-byte alignment");
+    int rc = launch_cvt_s8_f32(reinterpret_cast<hipStream_t>(stream), scale_src, src, dst, count, cu_count());
+    if (rc) return fail(MI355_ERR_LAUNCH, "typecvt: %s", hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
+}
+
 // ---- Pooling ----
 static int pooling_check(const mi355_pooling_desc* d, int* pack, uint32_t* oh, uint32_t* ow) {
     if (!d) return fail(MI355_ERR_BAD_ARG, "null descriptor");

@@ -54,6 +54,9 @@ int launch_requant(hipStream_t st, const EpiParams& e, const int32_t* src, const
 int launch_requant8(hipStream_t st, const EpiParams& e, const int8_t* src, const int8_t* z, int8_t* dst, uint64_t count,
                     int cu_count);
 
+int launch_cvt_f32_s8(hipStream_t st, float scale, const float* src, int8_t* dst, uint64_t count, int cu_count);
+int launch_cvt_s8_f32(hipStream_t st, float scale, const int8_t* src, float* dst, uint64_t count, int cu_count);
+
 int launch_pooling(hipStream_t st, const mi355_pooling_desc& d, int pack, uint32_t oh, uint32_t ow, const int8_t* src,
                    int8_t* dst, int cu_count);
 

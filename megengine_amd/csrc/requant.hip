@@ -1,5 +1,6 @@
 // Stand-alone requantisation QuantizedS32 | QuantizedS8 (+ QuantizedS8) -> QuantizedS8 with the ConvBias epilogue arithmetic
-// (epilogue.h): the reference's post-process pass, unary quantized ElemwiseMultiType modes and TypeCvt s32 -> s8.  Pure streaming:
+// (epilogue.h): the reference's post-process pass, unary quantized ElemwiseMultiType modes and TypeCvt s32 -> s8; and
+// TypeCvt between Float32 and QuantizedS8 (the quantize / dequantize at the edges of an int8 network).  Pure streaming:
 // 16 bytes in (+ 4), 4 bytes out per thread step; bound by HBM (5-6 bytes per element) and by the ~10 VALU operations
 // per element of the bit-exact requantisation.
 #include "common.h"
@@ -46,7 +47,69 @@ __global__ __launch_bounds__(256) void requant8_kernel(const int8_t* __restrict_
     }
 }
 
+// TypeCvt Float32 -> QuantizedS8: quantize = saturate(roundf(x / scale)), the literal divide -- the input is any float
+// (infinities, NaN -> -128 through fmaxf), so the divide-free form of the epilogue has no range guarantee to stand on
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int quantize_s8(float x, float scale) {
+    float v = x / scale;
+    v = __builtin_roundf(v);
+    v = fminf(fmaxf(-128.f, v), 127.f);
+    return (int)v;
+}
+
+__global__ __launch_bounds__(256) void cvt_f32_s8_kernel(const float* __restrict__ src, int8_t* __restrict__ dst,
+                                                         uint64_t quads, uint64_t count, float scale) {
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < quads; i += stride) {
+        const v4f x = reinterpret_cast<const v4f*>(src)[i];
+        reinterpret_cast<uint32_t*>(dst)[i] =
+                pack4(quantize_s8(x[0], scale), quantize_s8(x[1], scale), quantize_s8(x[2], scale), quantize_s8(x[3], scale));
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        for (uint64_t j = quads * 4; j < count; ++j) dst[j] = (int8_t)quantize_s8(src[j], scale);
+}
+
+// TypeCvt QuantizedS8 -> Float32: dequantize = float(x) * scale
+__global__ __launch_bounds__(256) void cvt_s8_f32_kernel(const int8_t* __restrict__ src, float* __restrict__ dst,
+                                                         uint64_t quads, uint64_t count, float scale) {
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < quads; i += stride) {
+        const int w = reinterpret_cast<const int*>(src)[i];
+        v4f o;
+        o[0] = (float)((w << 24) >> 24) * scale;
+        o[1] = (float)((w << 16) >> 24) * scale;
+        o[2] = (float)((w << 8) >> 24) * scale;
+        o[3] = (float)(w >> 24) * scale;
+        reinterpret_cast<v4f*>(dst)[i] = o;
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        for (uint64_t j = quads * 4; j < count; ++j) dst[j] = (float)src[j] * scale;
+}
+
+unsigned stream_blocks(uint64_t steps, int cu_count) {
+    if (cu_count <= 0) cu_count = 256;
+    uint64_t blocks = (steps + 255) / 256;
+    const uint64_t cap = (uint64_t)cu_count * 16;
+    if (blocks > cap) blocks = cap;
+    return blocks ? (unsigned)blocks : 1u;
+}
+
 }  // namespace
+
+int launch_cvt_f32_s8(hipStream_t st, float scale, const float* src, int8_t* dst, uint64_t count, int cu_count) {
+    if (count == 0) return 0;
+    hipLaunchKernelGGL(cvt_f32_s8_kernel, dim3(stream_blocks(count / 4, cu_count)), dim3(256), 0, st, src, dst, count / 4,
+                       count, scale);
+    return (int)hipGetLastError();
+}
+
+int launch_cvt_s8_f32(hipStream_t st, float scale, const int8_t* src, float* dst, uint64_t count, int cu_count) {
+    if (count == 0) return 0;
+    hipLaunchKernelGGL(cvt_s8_f32_kernel, dim3(stream_blocks(count / 4, cu_count)), dim3(256), 0, st, src, dst, count / 4,
+                       count, scale);
+    return (int)hipGetLastError();
+}
 
 int launch_requant8(hipStream_t st, const EpiParams& e, const int8_t* src, const int8_t* z, int8_t* dst, uint64_t count,
                     int cu_count) {

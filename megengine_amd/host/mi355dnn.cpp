@@ -577,6 +577,70 @@ void ElemwiseMultiType::exec(const std::vector<TensorND>& src, const TensorND& d
     requant_exec(m_handle, nl, src[0], arity == 2 ? &src[1] : nullptr, dst);
 }
 
-void TypeCvt::exec(const TensorND& src, const TensorND& dst) { requant_exec(m_handle, MI355_NL_IDENTITY, src, nullptr, dst); }
+void TypeCvt::exec(const TensorND& src, const TensorND& dst) {
+    const DTypeEnum se = src.layout.dtype.enumv, de = dst.layout.dtype.enumv;
+    const bool quantize = se == DTypeEnum::Float32 && de == DTypeEnum::QuantizedS8;
+    const bool dequantize = se == DTypeEnum::QuantizedS8 && de == DTypeEnum::Float32;
+    if (!quantize && !dequantize) return requant_exec(m_handle, MI355_NL_IDENTITY, src, nullptr, dst);
+    HOST_ASSERT(src.layout.eq_shape(dst.layout) && src.layout.is_contiguous() && dst.layout.is_contiguous(), MI355_ERR_SHAPE,
+                "operands must be contiguous and of the dst shape %s", dst.layout.to_string().c_str());
+    HOST_ASSERT(src.raw_ptr && dst.raw_ptr, MI355_ERR_BAD_ARG, "null tensor pointer");
+    const uint64_t n = dst.layout.total_nr_elems();
+    if (quantize)
+        check_abi(mi355_typecvt_f32_s8_exec(m_handle->stream(), n, dst.layout.dtype.scale,
+                                            static_cast<const float*>(src.raw_ptr), static_cast<int8_t*>(dst.raw_ptr)));
+    else
+        check_abi(mi355_typecvt_s8_f32_exec(m_handle->stream(), n, src.layout.dtype.scale,
+                                            static_cast<const int8_t*>(src.raw_ptr), static_cast<float*>(dst.raw_ptr)));
+}
+
+// ---------------------------------------------------------------- pooling
+static mi355_pooling_desc pooling_desc(const param::Pooling& p, const TensorLayout& src) {
+    using F = param::Pooling::Format;
+    uint32_t pack = 0;
+    switch (p.format) {
+        case F::NCHW: pack = 1; break;
+        case F::NCHW4:
+        case F::NCHW44: pack = 4; break;
+        case F::NCHW32: pack = 32; break;
+        default: HOST_ASSERT(false, MI355_ERR_UNSUPPORTED, "invalid pooling format %u", (unsigned)p.format);
+    }
+    HOST_ASSERT(src.ndim == (pack == 1 ? 4u : 5u), MI355_ERR_SHAPE, "src %s does not fit the format", src.to_string().c_str());
+    HOST_ASSERT(pack == 1 || src[4] == pack, MI355_ERR_SHAPE, "src %s: innermost axis must be %u", src.to_string().c_str(), pack);
+    mi355_pooling_desc d = mi355_pooling_desc();
+    d.mode = (uint32_t)p.mode;
+    d.format = (uint32_t)p.format;
+    d.n = (uint32_t)src[0];
+    d.c = (uint32_t)(src[1] * pack);
+    d.ih = (uint32_t)src[2];
+    d.iw = (uint32_t)src[3];
+    d.pad_h = p.pad_h; d.pad_w = p.pad_w; d.stride_h = p.stride_h; d.stride_w = p.stride_w;
+    d.window_h = p.window_h; d.window_w = p.window_w;
+    return d;
+}
+
+void PoolingForward::deduce_layout(const TensorLayout& src, TensorLayout& dst) const {
+    const mi355_pooling_desc d = pooling_desc(m_param, src);
+    uint32_t oh = 0, ow = 0;
+    check_abi(mi355_pooling_deduce_out(&d, &oh, &ow));
+    TensorShape s = src;
+    s.shape[2] = oh;
+    s.shape[3] = ow;
+    dst = TensorLayout(s, src.dtype);
+}
+
+void PoolingForward::exec(const TensorND& src, const TensorND& dst, const Workspace&) {
+    HOST_ASSERT(src.layout.dtype.enumv == DTypeEnum::QuantizedS8, MI355_ERR_UNSUPPORTED, "pooling takes QuantizedS8 tensors");
+    HOST_ASSERT(src.layout.dtype == dst.layout.dtype, MI355_ERR_BAD_ARG, "src and dst dtypes differ");
+    HOST_ASSERT(src.layout.is_contiguous() && dst.layout.is_contiguous(), MI355_ERR_UNSUPPORTED, "pooling takes contiguous tensors");
+    TensorLayout want;
+    deduce_layout(src.layout, want);
+    HOST_ASSERT(dst.layout.eq_shape(want), MI355_ERR_SHAPE, "dst %s, expected %s", dst.layout.to_string().c_str(),
+                want.to_string().c_str());
+    HOST_ASSERT(src.raw_ptr && dst.raw_ptr, MI355_ERR_BAD_ARG, "null tensor pointer");
+    const mi355_pooling_desc d = pooling_desc(m_param, src.layout);
+    check_abi(mi355_pooling_s8_exec(m_handle->stream(), &d, static_cast<const int8_t*>(src.raw_ptr),
+                                    static_cast<int8_t*>(dst.raw_ptr)));
+}
 
 }  // namespace mi355dnn

@@ -126,6 +126,14 @@ struct RelayoutFormat {
     uint32_t oc = 0;
     uint32_t group = 1;
 };
+// param::Pooling (dnn/scripts/opr_param_defs.py:233-254); Format shares the ConvBias enumerators
+struct Pooling {
+    enum class Mode : uint32_t { MAX = 0, AVERAGE = 1, AVERAGE_COUNT_EXCLUDE_PADDING = 2 };
+    using Format = ConvBias::Format;
+    Mode mode = Mode::MAX;
+    uint32_t pad_h = 0, pad_w = 0, stride_h = 2, stride_w = 2, window_h = 2, window_w = 2;
+    Format format = Format::NCHW;
+};
 }  // namespace param
 
 // ---- algorithms
@@ -281,7 +289,26 @@ private:
     Param m_param;
 };
 
-// megdnn::TypeCvt (dnn/include/megdnn/oprs/general.h:890) for QuantizedS32 / QuantizedS8 -> QuantizedS8
+// megdnn::PoolingForward (dnn/include/megdnn/oprs/nn.h, class PoolingForward) on QuantizedS8 tensors in NCHW, NCHW4,
+// NCHW44 or NCHW32; dst has the dtype of src (dnn/src/common/pooling.cpp:129-140).
+class PoolingForward : public OperatorBase {
+public:
+    using Param = param::Pooling;
+    using Mode = Param::Mode;
+    explicit PoolingForward(Handle* h) : OperatorBase(h) {}
+    Param& param() { return m_param; }
+    const Param& param() const { return m_param; }
+    void deduce_layout(const TensorLayout& src, TensorLayout& dst) const;
+    size_t get_workspace_in_bytes(const TensorLayout&, const TensorLayout&) const { return 0; }
+    void exec(const TensorND& src, const TensorND& dst, const Workspace& workspace);
+
+private:
+    Param m_param;
+};
+using Pooling = PoolingForward;
+
+// megdnn::TypeCvt (dnn/include/megdnn/oprs/general.h:890) for QuantizedS32 / QuantizedS8 -> QuantizedS8 and between
+// Float32 and QuantizedS8
 class TypeCvt : public OperatorBase {
 public:
     explicit TypeCvt(Handle* h) : OperatorBase(h) {}

@@ -19,7 +19,7 @@ EXPORTS = [
     "mi355_convbias_algo_usable", "mi355_convbias_s8_query", "mi355_convbias_s8_exec",
     "mi355_igemm_tile_count", "mi355_igemm_tile_name",
     "mi355_relayout_deduce", "mi355_relayout_exec", "mi355_requant_s32_s8_exec", "mi355_requant_s8_s8_exec", "mi355_convbias_s8_profile",
-    "mi355_pooling_deduce_out", "mi355_pooling_s8_exec",
+    "mi355_pooling_deduce_out", "mi355_pooling_s8_exec", "mi355_typecvt_f32_s8_exec", "mi355_typecvt_s8_f32_exec",
 ]
 
 
@@ -68,6 +68,8 @@ def lib():
     L.mi355_requant_s8_s8_exec.argtypes = [C.c_void_p, P(_abi.RequantDesc), C.c_void_p, C.c_void_p, C.c_void_p]
     L.mi355_pooling_deduce_out.argtypes = [P(_abi.PoolingDesc), P(C.c_uint32), P(C.c_uint32)]
     L.mi355_pooling_s8_exec.argtypes = [C.c_void_p, P(_abi.PoolingDesc), C.c_void_p, C.c_void_p]
+    L.mi355_typecvt_f32_s8_exec.argtypes = [C.c_void_p, C.c_uint64, C.c_float, C.c_void_p, C.c_void_p]
+    L.mi355_typecvt_s8_f32_exec.argtypes = [C.c_void_p, C.c_uint64, C.c_float, C.c_void_p, C.c_void_p]
     if L.mi355_abi_version() != _abi.ABI_VERSION:
         raise RuntimeError("ABI version mismatch: library %d, binding %d" % (L.mi355_abi_version(), _abi.ABI_VERSION))
     _LIB = L

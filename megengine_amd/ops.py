@@ -155,3 +155,19 @@ def pooling_exec(d, src, dst=None):
         dst = torch.empty(pooling_deduce_layout(d), dtype=torch.int8, device=src.device)
     check(lib().mi355_pooling_s8_exec(_stream(), C.byref(d), _ptr(src), _ptr(dst)))
     return dst
+
+
+def typecvt_exec(src, scale, dst=None):
+    """megdnn::TypeCvt between Float32 and QuantizedS8: a float32 tensor is quantized with `scale`, an int8 tensor is
+    dequantized with it."""
+    if src.dtype == torch.float32:
+        if dst is None:
+            dst = torch.empty(src.shape, dtype=torch.int8, device=src.device)
+        check(lib().mi355_typecvt_f32_s8_exec(_stream(), src.numel(), scale, _ptr(src), _ptr(dst)))
+    elif src.dtype == torch.int8:
+        if dst is None:
+            dst = torch.empty(src.shape, dtype=torch.float32, device=src.device)
+        check(lib().mi355_typecvt_s8_f32_exec(_stream(), src.numel(), scale, _ptr(src), _ptr(dst)))
+    else:
+        raise RuntimeError("typecvt_exec takes a float32 or an int8 tensor")
+    return dst

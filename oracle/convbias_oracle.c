@@ -116,6 +116,15 @@ int oracle_requant_s8_s8(const mi355_requant_desc* d, const int8_t* src, const i
     return MI355_OK;
 }
 
+/* TypeCvt Float32 <-> QuantizedS8 over n elements (naive/type_cvt/opr_impl.cpp:24-56: quantize / dequantize of
+ * dtype.h:845-854, the scalar functions above) */
+void oracle_typecvt_f32_s8(uint64_t n, float scale, const float* src, int8_t* dst) {
+    for (uint64_t i = 0; i < n; ++i) dst[i] = oracle_quantize_s8(src[i], scale);
+}
+void oracle_typecvt_s8_f32(uint64_t n, float scale, const int8_t* src, float* dst) {
+    for (uint64_t i = 0; i < n; ++i) dst[i] = oracle_dequantize_s8(src[i], scale);
+}
+
 /* ------------------------------------------------------------------------------------ */
 /* Pooling forward on dt_qint8                                                           */
 /* ------------------------------------------------------------------------------------ */

@@ -55,6 +55,10 @@ def lib():
         L.oracle_round_sweep.argtypes = [C.c_uint32, C.c_uint32, P(C.c_float)]
         L.oracle_pooling_s8.restype = C.c_int
         L.oracle_pooling_s8.argtypes = [P(_abi.PoolingDesc), C.c_void_p, C.c_void_p]
+        L.oracle_typecvt_f32_s8.restype = None
+        L.oracle_typecvt_f32_s8.argtypes = [C.c_uint64, C.c_float, C.c_void_p, C.c_void_p]
+        L.oracle_typecvt_s8_f32.restype = None
+        L.oracle_typecvt_s8_f32.argtypes = [C.c_uint64, C.c_float, C.c_void_p, C.c_void_p]
         _LIB = L
     return _LIB
 
@@ -167,4 +171,17 @@ def pooling(d, src):
     st = lib().oracle_pooling_s8(C.byref(d), _ptr(src), _ptr(dst))
     if st:
         raise OracleError(st)
+    return dst
+
+
+def typecvt(src, scale):
+    """float32 array -> int8 (quantize) or int8 array -> float32 (dequantize)"""
+    src = np.ascontiguousarray(src)
+    if src.dtype == np.float32:
+        dst = np.empty(src.shape, np.int8)
+        lib().oracle_typecvt_f32_s8(src.size, scale, _ptr(src), _ptr(dst))
+    else:
+        assert src.dtype == np.int8
+        dst = np.empty(src.shape, np.float32)
+        lib().oracle_typecvt_s8_f32(src.size, scale, _ptr(src), _ptr(dst))
     return dst

@@ -8,6 +8,7 @@
 //
 // Prints one line per case and "ALL OK" at the end; exit status 0 only when everything passed.
 #include <hip/hip_runtime_api.h>
+#include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -429,6 +430,76 @@ static void run_elemwise_gpu(Handle* h) {
     }
 }
 
+// ------------------------------------------------------------------ Pooling and float TypeCvt (GPU)
+extern "C" int oracle_pooling_s8(const mi355_pooling_desc* d, const int8_t* src, int8_t* dst);
+extern "C" void oracle_typecvt_f32_s8(uint64_t n, float scale, const float* src, int8_t* dst);
+extern "C" void oracle_typecvt_s8_f32(uint64_t n, float scale, const int8_t* src, float* dst);
+static void run_pooling_gpu(Handle* h) {
+    printf("case: PoolingForward and TypeCvt Float32 <-> QuantizedS8\n");
+    fflush(stdout);
+    using PM = PoolingForward::Mode;
+    auto opr = h->create_operator<PoolingForward>();
+    opr->param().format = param::Pooling::Format::NCHW32;
+    opr->param().window_h = opr->param().window_w = 3;
+    opr->param().stride_h = opr->param().stride_w = 2;
+    opr->param().pad_h = opr->param().pad_w = 1;
+    TensorLayout src({3, 2, 15, 17, 32}, dtype::QuantizedS8(0.05f)), dst;
+    opr->deduce_layout(src, dst);
+    EXPECT(dst.eq_shape(TensorShape{3, 2, 8, 9, 32}) && dst.dtype == src.dtype, "pooling deduce_layout: %s", dst.to_string().c_str());
+    const size_t ns = src.total_nr_elems(), nd = dst.total_nr_elems();
+    std::vector<int8_t> hs(ns), expect(nd), got(nd);
+    fill_s8(hs, 41, -128, 127);
+    DevBuf ds(ns), dd(nd);
+    HIP_OK(hipMemcpy(ds.p, hs.data(), ns, hipMemcpyHostToDevice));
+    for (PM mode : {PM::MAX, PM::AVERAGE, PM::AVERAGE_COUNT_EXCLUDE_PADDING}) {
+        opr->param().mode = mode;
+        mi355_pooling_desc d = mi355_pooling_desc();
+        d.mode = (uint32_t)mode; d.format = MI355_FMT_NCHW32; d.n = 3; d.c = 64; d.ih = 15; d.iw = 17;
+        d.pad_h = d.pad_w = 1; d.stride_h = d.stride_w = 2; d.window_h = d.window_w = 3;
+        EXPECT(oracle_pooling_s8(&d, hs.data(), expect.data()) == 0, "CPU checker refused pooling mode %u", (unsigned)mode);
+        HIP_OK(hipMemset(dd.p, 0x5a, nd));
+        opr->exec(TensorND(ds.p, src), TensorND(dd.p, dst), Workspace());
+        HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
+        HIP_OK(hipMemcpy(got.data(), dd.p, nd, hipMemcpyDeviceToHost));
+        size_t bad = 0;
+        for (size_t i = 0; i < nd; ++i) bad += got[i] != expect[i];
+        EXPECT(bad == 0, "pooling mode %u: %zu of %zu bytes differ", (unsigned)mode, bad, nd);
+    }
+    // a window in the padding only; a dst of another dtype
+    opr->param().mode = PM::MAX;
+    opr->param().pad_h = 3;
+    TensorLayout far;
+    opr->deduce_layout(src, far);
+    DevBuf dfar(far.total_nr_elems());
+    EXPECT(throws([&] { opr->exec(TensorND(ds.p, src), TensorND(dfar.p, far), Workspace()); }, MI355_ERR_SHAPE),
+           "window outside the image completely");
+    opr->param().pad_h = 1;
+    TensorLayout other(dst, dtype::QuantizedS8(0.07f));
+    EXPECT(throws([&] { opr->exec(TensorND(ds.p, src), TensorND(dd.p, other), Workspace()); }, MI355_ERR_BAD_ARG), "dst scale differs");
+
+    // TypeCvt Float32 -> QuantizedS8 -> Float32
+    const size_t n = 100003;
+    std::vector<float> hf(n), backf(n), expf(n);
+    std::vector<int8_t> q(n), expq(n);
+    for (size_t i = 0; i < n; ++i) hf[i] = ((float)((i * 2654435761u) % 20001u) - 10000.f) * 7e-4f;
+    hf[0] = INFINITY; hf[1] = -INFINITY; hf[2] = NAN; hf[3] = 0.5f * 0.05f; hf[4] = -0.5f * 0.05f;
+    DevBuf df(n * 4), dq(n), db(n * 4);
+    HIP_OK(hipMemcpy(df.p, hf.data(), n * 4, hipMemcpyHostToDevice));
+    const TensorShape shp{n};
+    TensorLayout lf(shp, dtype::Float32()), lq(shp, dtype::QuantizedS8(0.05f));
+    auto cvt = h->create_operator<TypeCvt>();
+    cvt->exec(TensorND(df.p, lf), TensorND(dq.p, lq));
+    cvt->exec(TensorND(dq.p, lq), TensorND(db.p, lf));
+    HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
+    HIP_OK(hipMemcpy(q.data(), dq.p, n, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(backf.data(), db.p, n * 4, hipMemcpyDeviceToHost));
+    oracle_typecvt_f32_s8(n, 0.05f, hf.data(), expq.data());
+    oracle_typecvt_s8_f32(n, 0.05f, expq.data(), expf.data());
+    size_t bad = 0;
+    for (size_t i = 0; i < n; ++i) bad += q[i] != expq[i] || memcmp(&backf[i], &expf[i], 4) != 0;
+    EXPECT(bad == 0, "TypeCvt float: %zu of %zu elements differ", bad, n);
+}
+
 // ------------------------------------------------------------------ fast-run (GPU)
 static void run_fast_run_gpu(Handle* h) {
     printf("case: fast-run profiling\n");
@@ -510,6 +581,7 @@ int main(int argc, char** argv) {
         for (auto& c : cases()) run_conv_case(handle.get(), c, gpu);
         if (gpu) run_relayout_gpu(handle.get());
         if (gpu) run_elemwise_gpu(handle.get());
+        if (gpu) run_pooling_gpu(handle.get());
         if (gpu) run_fast_run_gpu(handle.get());
     } catch (const Error& e) {
         printf("unexpected mi355dnn::Error %d: %s\n", e.status(), e.what());

@@ -107,3 +107,31 @@ def test_int8_tail_and_alignment(oracle):
     x = torch.zeros(64, dtype=torch.int8, device="cuda")
     with pytest.raises(Mi355Error):
         ops.requant_exec(x[1:33], 1.0, 1.0)
+
+
+def test_typecvt_float32_to_int8_and_back(oracle):
+    """TypeCvt Float32 <-> QuantizedS8: dense sweeps through every rounding boundary, random bit patterns (NaN,
+    infinities, denormals included), ragged lengths, and the round trip."""
+    rng = np.random.RandomState(21)
+    for scale in (1.0, 0.25, 0.037, 3.3e-3, 17.5):
+        s = np.float32(scale)
+        x = (np.arange(-140 * 4096, 140 * 4096 + 1, dtype=np.float32) / np.float32(4096)) * s
+        bits = rng.randint(0, 2 ** 32, 1 << 20, dtype=np.uint64).astype(np.uint32).view(np.float32)
+        for arr in (x, bits, x[:1], x[:5], x[:1023]):
+            say("typecvt f32->s8", scale, arr.size)
+            got = ops.typecvt_exec(torch.from_numpy(arr).cuda(), scale)
+            torch.cuda.synchronize()
+            want = oracle.typecvt(arr, scale)
+            g = got.cpu().numpy()
+            if not np.array_equal(g, want):
+                bad = np.nonzero(g != want)[0]
+                raise AssertionError("%d mismatches, first: x=%r got %d want %d (scale %r)" % (
+                    len(bad), arr[bad[0]], g[bad[0]], want[bad[0]], scale))
+        q = rng.randint(-128, 128, 100003).astype(np.int8)
+        f = ops.typecvt_exec(torch.from_numpy(q).cuda(), scale)
+        assert np.array_equal(f.cpu().numpy(), oracle.typecvt(q, scale))
+        assert np.array_equal(ops.typecvt_exec(f, scale).cpu().numpy(), q)
+    from megengine_amd.lib import Mi355Error
+    buf = torch.zeros(64, dtype=torch.float32).cuda()
+    with pytest.raises(Mi355Error, match="alignment"):
+        ops.typecvt_exec(buf[1:33], 1.0)

@@ -539,3 +539,24 @@ def test_pooling_vs_definition_and_formats(oracle):
         d = _abi.make_pooling_desc(mode, "NCHW", 1, 4, 4, 4, 2, 2, 2)
         with pytest.raises(oracle.OracleError):
             oracle.pooling(d, x)
+
+
+def test_typecvt_float_int8_closed_forms(oracle):
+    """TypeCvt Float32 <-> QuantizedS8 is the pinned scalar quantize / dequantize applied element by element: with a
+    power-of-two scale the quotient is exact, so the result is round-half-away of the scaled input with saturation;
+    infinities saturate and NaN gives -128 (fmax before fmin); dequantize of every int8 is exact for such scales."""
+    x = np.array([0.0, -0.0, 0.5, -0.5, 1.5, -1.5, 2.5, 126.5, 127.49, 127.5, 1e9, -128.5, -129.0, -1e9,
+                  np.inf, -np.inf, np.nan, 0.49999997, -0.49999997], np.float32)
+    want = np.array([0, 0, 1, -1, 2, -2, 3, 127, 127, 127, 127, -128, -128, -128, 127, -128, -128, 0, 0], np.int8)
+    assert np.array_equal(oracle.typecvt(x, 1.0), want)
+    assert np.array_equal(oracle.typecvt(x * np.float32(0.25), 0.25), want)
+    rng = np.random.RandomState(8)
+    y = (rng.randn(5000) * 3).astype(np.float32)
+    s = np.float32(0.037)
+    L = oracle.lib()
+    assert np.array_equal(oracle.typecvt(y, float(s)), np.array([L.oracle_quantize_s8(float(v), float(s)) for v in y], np.int8))
+    q = np.arange(-128, 128, dtype=np.int16).astype(np.int8)
+    assert np.array_equal(oracle.typecvt(q, 0.5), q.astype(np.float32) / 2)
+    assert np.array_equal(oracle.typecvt(q, float(s)), q.astype(np.float32) * s)
+    # round trip: quantize(dequantize(q)) = q for any positive normal scale
+    assert np.array_equal(oracle.typecvt(oracle.typecvt(q, float(s)), float(s)), q)
