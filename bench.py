@@ -2,7 +2,7 @@
 """Benchmark of the int8 ConvBias hot path on one MI355X.
 
 A "step" is one pass over the 53 ConvBias layers of the ResNet-50 int8 conv stack at batch 64
-(BASELINE config 2) on synthetic, HBM-resident tensors; activations are requantised between
+(workload "config 2" of megengine_amd/workloads.py) on synthetic, HBM-resident tensors; activations are requantised between
 layers and the residual z tensors are the real producer outputs.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
@@ -310,7 +310,7 @@ def time_launches(torch, fn, iters=20, warm=3):
 
 
 def run_extras(torch, np, util, _abi, lib, ops, workloads):
-    """Side measurements for the other BASELINE configs (not the headline value)."""
+    """Side measurements for the other workload configurations (not the headline value)."""
     res = {}
 
     def measure(layers, seed):

@@ -1,4 +1,4 @@
-"""The BASELINE workloads as lists of ConvBias descriptors (shapes only; no model code).
+"""The benchmark workloads as lists of ConvBias descriptors (shapes only; no model code).
 
 config 2: the 53 ConvBias layers of ResNet-50 v1.5 at batch 64 (stem in NCHW4 with the input
           padded to 4 channels, everything after the max-pool in NCHW32);

@@ -1,4 +1,4 @@
-"""Parity at BASELINE sizes, where the CPU checker cannot finish the whole tensor in seconds:
+"""Parity at the benchmark workloads' full sizes, where the CPU checker cannot finish the whole tensor in seconds:
   * the checker evaluates the operator at tens of thousands of seeded random output positions;
   * the tiled kernel must agree with the generic direct kernel (checked against the checker on small
     shapes) on EVERY output element;

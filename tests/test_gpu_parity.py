@@ -181,7 +181,7 @@ def test_igemm_strided_batch(oracle):
 
 
 def test_config0_full_size(oracle):
-    """BASELINE config 0: NCHW4 N16 64->64 56x56 3x3 s1 p1, bias U[-1000,1000], RELU, scales .02*.01 -> .05."""
+    """Workload config 0: NCHW4 N16 64->64 56x56 3x3 s1 p1, bias U[-1000,1000], RELU, scales .02*.01 -> .05."""
     sb = float(np.float32(0.02) * np.float32(0.01))
     d = _abi.make_conv_desc("NCHW4", 16, 64, 56, 56, 64, 3, pad=1, nonline="RELU", scale_bias=sb,
                             scale_dst=float(np.float32(0.05)))

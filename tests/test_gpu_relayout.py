@@ -70,7 +70,7 @@ def test_relayout_requant(oracle):
 
 
 def test_roundtrip_full_size():
-    """BASELINE config 4 sized tensors: NCHW -> NCHW32 -> NCHW is the identity and agrees with the
+    """Tensors of the large-shape workload (config 4): NCHW -> NCHW32 -> NCHW is the identity and agrees with the
     closed-form numpy permutation."""
     for shape in ((8, 256, 64, 64), (4, 128, 80, 80)):
         x = util.uniform_int(5, shape, -128, 127, np.int8)
