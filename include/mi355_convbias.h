@@ -183,6 +183,15 @@ int mi355_convbias_s8_profile(void* stream, const mi355_conv_desc* d, const mi35
 int mi355_igemm_tile_count(void);
 const char* mi355_igemm_tile_name(int tile_cfg);
 
+/* The requantisation without z, dst = quantize_s8(act(float(sfb) * scale_bias)) with act IDENTITY or RELU
+ * (dnn/src/naive/conv_bias/opr_impl.cpp:52,69-73,89-93; dnn/include/megdnn/dtype.h:845-853), is a step
+ * function of the integer sfb.  When the library has proved that one fused multiply-add reproduces it on
+ * every int32, dst = floor(min(max(fma(float(sfb), c, d), lo), 127.5)) with lo = 0 (RELU) or -128, its
+ * kernels use that form.  Returns 1 and writes (c, d) if it has such a proof for these scales, 0 if not
+ * (the kernels then run the multi-step form), a negative mi355_status on a bad argument.  Diagnostic:
+ * no counterpart in the reference. */
+int mi355_epilogue_linear_form(float scale_bias, float scale_dst, uint32_t nonline, float* c, float* d);
+
 /* ---- RelayoutFormat ---- */
 /* param::RelayoutFormat::Mode values (opr_param_defs.py:1069-1111); 32/33 and 34/35 are
  * extensions of this backend (the reference has no NCHW32 relayout mode). */

@@ -53,6 +53,127 @@ bool epi_fast_ok(float s_b, float s_z, float s_d, bool has_z) {
     return true;
 }
 
+// ---- linear epilogue form (epilogue.h): host-side search and proof ---------------------------------
+// The contract without z, as a function of the integer sfb (every operation a separately rounded
+// binary32 operation; this host code is compiled without contraction and without fast-math):
+int epi_contract(int t, float s_b, float s_d, bool relu) {
+    float r = (float)t * s_b;
+    if (relu) r = r <= 0.f ? 0.f : r;
+    float v = roundf(r / s_d);
+    v = fminf(fmaxf(-128.f, v), 127.f);
+    return (int)v;
+}
+// The device's linear form on the same integer: one fused multiply-add, clamp, floor.
+int epi_linear(int t, float c, float d, float lo) {
+    float x = fmaf((float)t, c, d);
+    x = fminf(fmaxf(x, lo), 127.5f);
+    return (int)floorf(x);
+}
+
+// Finds (c, d) such that epi_linear == epi_contract on EVERY int32, or reports that it found none.
+// Both are non-decreasing step functions of t (s_b, s_d, c > 0).  T[k] = the smallest t with contract(t) >= k is
+// found by bisection inside [-2^24, 2^24], where float(t) is exact; a candidate is accepted only if
+// linear(T[k]) >= k and linear(T[k] - 1) <= k - 1 for every k, which by monotonicity gives equality on all
+// of [T[kmin] - 1, T[127]], and on both sides of that range the two functions sit at the same clamp.
+bool epi_solve_linear(float s_b, float s_d, bool relu, float* c_out, float* d_out) {
+    const int LIM = 1 << 24;
+    const int kmin = relu ? 1 : -127, kmax = 127;
+    int T[255];
+    if (epi_contract(LIM, s_b, s_d, relu) < kmax) return false;
+    if (epi_contract(-LIM, s_b, s_d, relu) >= kmin) return false;
+    for (int k = kmin; k <= kmax; ++k) {
+        int lo = -LIM, hi = LIM;  // contract(lo) < k <= contract(hi)
+        while (hi - lo > 1) {
+            const int m = lo + (hi - lo) / 2;
+            if (epi_contract(m, s_b, s_d, relu) >= k) hi = m; else lo = m;
+        }
+        T[k - kmin] = hi;
+    }
+    const float lo_clamp = relu ? 0.f : -128.f;
+    const float c0 = (float)((double)s_b / (double)s_d);
+    if (!(c0 > 0.f) || !(c0 < 0x1p20f)) return false;
+    for (int u = 0; u <= 16; ++u) {
+        for (int sgn = -1; sgn <= 1; sgn += 2) {
+            if (u == 0 && sgn == 1) continue;
+            float c = c0;
+            for (int i = 0; i < u; ++i) c = nextafterf(c, sgn > 0 ? INFINITY : 0.f);
+            if (!(c > 0.f)) continue;
+            // in real arithmetic step k sits at T[k] iff  k - T[k] c <= d < k - (T[k] - 1) c
+            double dlo = -1e300, dhi = 1e300;
+            for (int k = kmin; k <= kmax; ++k) {
+                const double a = (double)k - (double)T[k - kmin] * (double)c;
+                if (a > dlo) dlo = a;
+                if (a + (double)c < dhi) dhi = a + (double)c;
+            }
+            if (!(dlo < dhi)) continue;
+            for (int j = 1; j <= 3; ++j) {
+                const float d = (float)(dlo + (dhi - dlo) * j / 4.0);
+                bool ok = true;
+                for (int k = kmin; k <= kmax && ok; ++k) {
+                    const int t = T[k - kmin];
+                    ok = epi_linear(t, c, d, lo_clamp) >= k && epi_linear(t - 1, c, d, lo_clamp) <= k - 1;
+                }
+                if (ok) {
+                    *c_out = c;
+                    *d_out = d;
+                    return true;
+                }
+            }
+        }
+    }
+    return false;
+}
+
+// Results are kept per (s_b, s_d, activation): a search is ~0.1 ms of host time, a hit a few dozen ns.
+struct LinEntry {
+    uint32_t kb, kd;
+    int relu, state;  // state: 0 empty, 1 solved, 2 no solution
+    float c, d;
+};
+LinEntry g_lin[256];
+std::mutex g_lin_mu;
+
+bool epi_linear_cached(float s_b, float s_d, bool relu, float* c, float* d) {
+    uint32_t kb, kd;
+    memcpy(&kb, &s_b, 4);
+    memcpy(&kd, &s_d, 4);
+    const uint32_t slot = ((kb * 2654435761u) ^ (kd * 40503u) ^ (uint32_t)relu) >> 5 & 255u;
+    {
+        std::lock_guard<std::mutex> lk(g_lin_mu);
+        const LinEntry& e = g_lin[slot];
+        if (e.state && e.kb == kb && e.kd == kd && e.relu == (int)relu) {
+            *c = e.c;
+            *d = e.d;
+            return e.state == 1;
+        }
+    }
+    LinEntry n;
+    n.kb = kb; n.kd = kd; n.relu = relu; n.c = n.d = 0.f;
+    n.state = epi_solve_linear(s_b, s_d, relu, &n.c, &n.d) ? 1 : 2;
+    std::lock_guard<std::mutex> lk(g_lin_mu);
+    g_lin[slot] = n;
+    *c = n.c;
+    *d = n.d;
+    return n.state == 1;
+}
+
+// All epilogue parameters of one launch.  qs8: the destination is QuantizedS8 (the only dtype with the fast forms).
+void epi_fill(EpiParams* e, float s_b, float s_z, float s_d, uint32_t nonline, bool has_z, bool qs8) {
+    e->s_b = s_b;
+    e->s_z = s_z;
+    e->s_d = s_d;
+    e->nonline = (int)nonline;
+    e->has_z = has_z ? 1 : 0;
+    e->fast = qs8 && epi_fast_ok(s_b, s_z, s_d, has_z);
+    e->y_hi = 1.0f / s_d;
+    e->y_lo = (float)(1.0 / (double)s_d - (double)e->y_hi);
+    e->lin = 0;
+    e->lin_c = e->lin_d = 0.f;
+    e->lin_lo = nonline == MI355_NL_RELU ? 0.f : -128.f;
+    if (e->fast && !has_z && (nonline == MI355_NL_IDENTITY || nonline == MI355_NL_RELU))
+        e->lin = epi_linear_cached(s_b, s_d, nonline == MI355_NL_RELU, &e->lin_c, &e->lin_d) ? 1 : 0;
+}
+
 // Validation of a descriptor: the checks of ConvolutionBase::deduce_layout_fwd
 // (dnn/src/common/convolution.cpp:633-1049) and do_check_exec_common
 // (dnn/src/common/conv_bias.cpp:8-133) that survive the translation to a flat descriptor.
@@ -108,14 +229,8 @@ int canonize(const mi355_conv_desc* d, ConvProblem* p) {
     if (p->src_sn < src_img || p->dst_sn < dst_img || p->z_sn < dst_img)
         return fail(MI355_ERR_SHAPE, "batch stride smaller than one image");
     // Float32 dst: scale_bias / scale_z carry the scales of src and filter; one factor dequantises the exact sum
-    p->epi.s_b = d->dst_dtype == MI355_DT_F32 ? d->scale_bias * d->scale_z : d->scale_bias;
-    p->epi.s_z = d->scale_z;
-    p->epi.s_d = d->scale_dst;
-    p->epi.nonline = (int)d->nonline;
-    p->epi.has_z = d->has_z ? 1 : 0;
-    p->epi.fast = d->dst_dtype == MI355_DT_QS8 && epi_fast_ok(d->scale_bias, d->scale_z, d->scale_dst, d->has_z != 0);
-    p->epi.y_hi = 1.0f / d->scale_dst;
-    p->epi.y_lo = (float)(1.0 / (double)d->scale_dst - (double)p->epi.y_hi);
+    epi_fill(&p->epi, d->scale_bias, d->scale_z, d->scale_dst, d->nonline, d->has_z != 0, d->dst_dtype == MI355_DT_QS8);
+    if (d->dst_dtype == MI355_DT_F32) p->epi.s_b = d->scale_bias * d->scale_z;
     return MI355_OK;
 }
 
@@ -344,11 +459,7 @@ int mi355_requant_s32_s8_exec(void* stream, const mi355_requant_desc* d, const i
     if (!aligned16(src) || (reinterpret_cast<uintptr_t>(dst) & 3) || (d->has_z && (reinterpret_cast<uintptr_t>(z) & 3)))
         return fail(MI355_ERR_BAD_ARG, "src needs 16-byte, z and dst 4-byte alignment");
     EpiParams e;
-    e.s_b = d->scale_src; e.s_z = d->scale_z; e.s_d = d->scale_dst;
-    e.nonline = (int)d->nonline; e.has_z = d->has_z != 0;
-    e.fast = epi_fast_ok(d->scale_src, d->scale_z, d->scale_dst, d->has_z != 0);
-    e.y_hi = 1.0f / d->scale_dst;
-    e.y_lo = (float)(1.0 / (double)d->scale_dst - (double)e.y_hi);
+    epi_fill(&e, d->scale_src, d->scale_z, d->scale_dst, d->nonline, d->has_z != 0, true);
     int rc = launch_requant(reinterpret_cast<hipStream_t>(stream), e, src, z, dst, d->count, cu_count());
     if (rc) return fail(MI355_ERR_LAUNCH, "requant: %s", hipGetErrorString((hipError_t)rc));
     return MI355_OK;
@@ -364,11 +475,7 @@ int mi355_requant_s8_s8_exec(void* stream, const mi355_requant_desc* d, const in
     if (!aligned16(src) || !aligned16(dst) || (d->has_z && !aligned16(z)))
         return fail(MI355_ERR_BAD_ARG, "src, z and dst need 16-byte alignment");
     EpiParams e;
-    e.s_b = d->scale_src; e.s_z = d->scale_z; e.s_d = d->scale_dst;
-    e.nonline = (int)d->nonline; e.has_z = d->has_z != 0;
-    e.fast = epi_fast_ok(d->scale_src, d->scale_z, d->scale_dst, d->has_z != 0);
-    e.y_hi = 1.0f / d->scale_dst;
-    e.y_lo = (float)(1.0 / (double)d->scale_dst - (double)e.y_hi);
+    epi_fill(&e, d->scale_src, d->scale_z, d->scale_dst, d->nonline, d->has_z != 0, true);
     int rc = launch_requant8(reinterpret_cast<hipStream_t>(stream), e, src, z, dst, d->count, cu_count());
     if (rc) return fail(MI355_ERR_LAUNCH, "requant: %s", hipGetErrorString((hipError_t)rc));
     return MI355_OK;
@@ -447,6 +554,17 @@ int mi355_pooling_s8_exec(void* stream, const mi355_pooling_desc* d, const int8_
 
 int mi355_igemm_tile_count(void) { return igemm_num_cfgs(); }
 const char* mi355_igemm_tile_name(int cfg) { return igemm_cfg_name(cfg); }
+
+int mi355_epilogue_linear_form(float scale_bias, float scale_dst, uint32_t nonline, float* c, float* d) {
+    if (!c || !d) return -fail(MI355_ERR_BAD_ARG, "null argument");
+    if (nonline != MI355_NL_IDENTITY && nonline != MI355_NL_RELU)
+        return -fail(MI355_ERR_BAD_ARG, "the linear form exists for IDENTITY and RELU only");
+    EpiParams e;
+    epi_fill(&e, scale_bias, 1.f, scale_dst, nonline, false, true);
+    *c = e.lin_c;
+    *d = e.lin_d;
+    return e.lin;
+}
 
 // ---- RelayoutFormat ----
 static uint32_t cdiv(uint32_t a, uint32_t b) { return (a + b - 1) / b; }

@@ -231,7 +231,9 @@ __global__ __launch_bounds__(C4_THREADS, 3) void c4_kernel(C4Args a) {
             }
         }
 
-        if (a.epi.has_z) {
+        if (a.epi.lin) {
+            c4_epilogue<NL_LIN, false>(a, acc, zr, doff, rs_dst);
+        } else if (a.epi.has_z) {
             switch (a.epi.nonline) {
                 case NL_RELU: c4_epilogue<NL_RELU, true>(a, acc, zr, doff, rs_dst); break;
                 case NL_H_SWISH: c4_epilogue<NL_H_SWISH, true>(a, acc, zr, doff, rs_dst); break;

@@ -340,6 +340,8 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(Dw3Args a) {
 
     if (!a.epi.fast) {
         dw3_store<R, 0, false, false>(a, acc, n, cg, oh0, ow0);
+    } else if (a.epi.lin) {
+        dw3_store<R, NL_LIN, false, true>(a, acc, n, cg, oh0, ow0);
     } else if (a.epi.has_z) {
         switch (a.epi.nonline) {
             case NL_RELU: dw3_store<R, NL_RELU, true, true>(a, acc, n, cg, oh0, ow0); break;

@@ -21,6 +21,16 @@
 // The host only selects the fast form when the scales are positive, normal and small enough
 // that no intermediate overflows (see epi_fast_ok in capi.hip); otherwise kernels run the
 // literal form with the IEEE divide.
+//
+// The "linear" form (NL_LIN; IDENTITY or RELU without z) is one fused multiply-add:
+//     dst = floor(min(max(fma(float(sfb), c, d), lo), 127.5))
+// Without z the contract above is a non-decreasing step function of the integer sfb with at most 255
+// steps, and so is this form for c > 0.  Two non-decreasing step functions are equal on every integer
+// iff each step of one sits at the same integer as the corresponding step of the other, so the host
+// finds the 255 step positions of the contract by bisection, chooses (c, d) from them and then
+// checks every step of the candidate against them with the device's own arithmetic (epi_solve_linear
+// in capi.hip).  Only a pair (c, d) that passes is ever handed to a kernel; when none passes, the
+// fast form runs.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -33,9 +43,12 @@ struct EpiParams {
     int nonline;  // MI355_NL_*
     int has_z;
     int fast;     // 1: fast form allowed
+    int lin;      // 1: linear form verified for (s_b, s_d, nonline); implies fast && !has_z
+    float lin_c, lin_d, lin_lo;
 };
 
-enum { NL_IDENTITY = 0, NL_RELU = 1, NL_H_SWISH = 3 };
+// NL_LIN is not an activation of the interface: it selects the linear form in the kernels' epilogue templates
+enum { NL_IDENTITY = 0, NL_RELU = 1, NL_H_SWISH = 3, NL_LIN = 4 };
 
 __device__ __forceinline__ float act_f32(float r, int nl) {
     if (nl == NL_RELU) return r <= 0.f ? 0.f : r;
@@ -78,6 +91,13 @@ __device__ __forceinline__ int requant_s32_exact(int sfb, bool has_z, int z, con
 // fast form; NL and HAS_Z are compile-time so the inner loops carry no branches
 template <int NL, bool HAS_Z>
 __device__ __forceinline__ int requant_s8_fast(int sfb, int z, const EpiParams& e) {
+    if (NL == NL_LIN) {
+        float x = __builtin_fmaf((float)sfb, e.lin_c, e.lin_d);
+        x = __builtin_amdgcn_fmed3f(x, e.lin_lo, 127.5f);
+        int o;
+        asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(o) : "v"(x));  // (int)floor(x): x is finite and inside [-128, 127.5]
+        return o;
+    }
     float r = (float)sfb * e.s_b;
     if (HAS_Z) {
         float zf = (float)z * e.s_z;
@@ -144,6 +164,7 @@ __device__ __forceinline__ uint32_t requant4_exact(int a0, int a1, int a2, int a
 // runtime dispatch used by the bandwidth-bound kernels (one uniform branch per call site)
 __device__ __forceinline__ uint32_t requant4(int a0, int a1, int a2, int a3, uint32_t zw, const EpiParams& e) {
     if (!e.fast) return requant4_exact(a0, a1, a2, a3, zw, e);
+    if (e.lin) return requant4_fast<NL_LIN, false>(a0, a1, a2, a3, zw, e);
     if (e.has_z) {
         switch (e.nonline) {
             case NL_RELU: return requant4_fast<NL_RELU, true>(a0, a1, a2, a3, zw, e);

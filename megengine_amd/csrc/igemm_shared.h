@@ -161,7 +161,9 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
 template <int POUT, int MT, int NT, bool ZPRE = false>
 __device__ __forceinline__ void igemm_run_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w, int l32,
                                                    int lh, const ZRegs<MT, NT>* zr = nullptr) {
-    if (a.epi.has_z) {
+    if (a.epi.lin) {
+        igemm_epilogue<POUT, MT, NT, NL_LIN, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh);
+    } else if (a.epi.has_z) {
         switch (a.epi.nonline) {
             case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
             case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;

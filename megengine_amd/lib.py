@@ -17,7 +17,7 @@ EXPORTS = [
     "mi355_abi_version", "mi355_status_string", "mi355_last_error", "mi355_get_device_info",
     "mi355_convbias_deduce_out", "mi355_convbias_algo_count", "mi355_convbias_algo_name",
     "mi355_convbias_algo_usable", "mi355_convbias_s8_query", "mi355_convbias_s8_exec",
-    "mi355_igemm_tile_count", "mi355_igemm_tile_name",
+    "mi355_igemm_tile_count", "mi355_igemm_tile_name", "mi355_epilogue_linear_form",
     "mi355_relayout_deduce", "mi355_relayout_exec", "mi355_requant_s32_s8_exec", "mi355_requant_s8_s8_exec", "mi355_convbias_s8_profile",
     "mi355_pooling_deduce_out", "mi355_pooling_s8_exec", "mi355_typecvt_f32_s8_exec", "mi355_typecvt_s8_f32_exec",
 ]
@@ -62,6 +62,8 @@ def lib():
     L.mi355_igemm_tile_count.restype = C.c_int
     L.mi355_igemm_tile_name.restype = C.c_char_p
     L.mi355_igemm_tile_name.argtypes = [C.c_int]
+    L.mi355_epilogue_linear_form.restype = C.c_int
+    L.mi355_epilogue_linear_form.argtypes = [C.c_float, C.c_float, C.c_uint32, P(C.c_float), P(C.c_float)]
     L.mi355_relayout_deduce.argtypes = [P(_abi.RelayoutDesc), P(C.c_uint32), P(C.c_uint32)]
     L.mi355_relayout_exec.argtypes = [C.c_void_p, P(_abi.RelayoutDesc), C.c_void_p, C.c_void_p]
     L.mi355_requant_s32_s8_exec.argtypes = [C.c_void_p, P(_abi.RequantDesc), C.c_void_p, C.c_void_p, C.c_void_p]
