@@ -367,3 +367,44 @@ def test_random_descriptors_every_kernel_family(oracle):
             out = ops.conv_bias_exec(d, ts, tf, tb, tz, algo=a)
             torch.cuda.synchronize()
             assert torch.equal(out, ref), "tile %s" % (names[tile] if tile is not None else "heuristic")
+
+
+# ---------------------------------------------------------------------------------------------
+# the one-instruction (linear) epilogue form in every kernel family that carries it
+# ---------------------------------------------------------------------------------------------
+
+# scale pairs for which the library has a proved linear form (asserted below, so the test cannot pass vacuously);
+# accumulator ranges are chosen so that the outputs cover every int8 value and both clamps
+LIN_SCALES = [(1.3e-3, 0.0271), (0.5, 1.0), (1e-3, 1.0)]
+
+LIN_CASES = [
+    # tag, expected algorithm, descriptor arguments
+    ("dma 1x1", IGEMM, dict(fmt="NCHW32", n=2, ic=64, ih=9, iw=7, oc=96, fh=1)),
+    ("dma 3x3", IGEMM, dict(fmt="NCHW32", n=2, ic=64, ih=9, iw=11, oc=64, fh=3, pad=1)),
+    ("staged nchw4", IGEMM, dict(fmt="NCHW4", n=2, ic=24, ih=9, iw=9, oc=48, fh=3, pad=1)),
+    ("mixed 4->32", IGEMM, dict(fmt="NCHW4_NCHW32", n=2, ic=16, ih=8, iw=8, oc=64, fh=3, pad=1)),
+    ("first layer", C4, dict(fmt="NCHW4", n=2, ic=4, ih=30, iw=30, oc=64, fh=7, pad=3, stride=2)),
+    ("dw3x3 s1", DW, dict(fmt="NCHW4", n=2, ic=32, ih=14, iw=14, oc=32, fh=3, pad=1, group=32)),
+    ("dw3x3 s2", DW, dict(fmt="NCHW4", n=2, ic=24, ih=15, iw=13, oc=24, fh=3, pad=1, stride=2, group=24)),
+    ("dw 5x5", DW, dict(fmt="NCHW4", n=1, ic=8, ih=12, iw=12, oc=8, fh=5, pad=2, group=8)),
+]
+
+
+@pytest.mark.parametrize("i", range(len(LIN_CASES)))
+def test_linear_epilogue_form(oracle, i):
+    import ctypes as C
+    tag, want_algo, c = LIN_CASES[i]
+    for sb, sd in LIN_SCALES:
+        for nl in ("IDENTITY", "RELU"):
+            cc, dd = C.c_float(), C.c_float()
+            assert lib.lib().mi355_epilogue_linear_form(sb, sd, getattr(_abi, "NL_" + nl), C.byref(cc), C.byref(dd)) == 1
+            d = mk(c, nonline=nl, scale_bias=sb, scale_dst=sd)
+            assert ops.conv_bias_query(d)[0].id == want_algo
+            # accumulators spread over about +-200 / (sb / sd): all 256 outputs and both saturation edges occur
+            span = 200.0 * sd / sb
+            taps = d.fh * d.fw * (d.ic // d.group)
+            amp = int(max(1, min(127, (1.5 * span / taps ** 0.5) ** 0.5)))
+            b = int(min(2 ** 30, span))
+            want = check_case(oracle, d, seed=400 + i, tag="lin " + tag, src_range=(-amp, amp), flt_range=(-amp, amp),
+                              bias_range=(-b, b))
+            assert len(np.unique(want)) >= (100 if nl == "RELU" else 200), len(np.unique(want))
