@@ -28,7 +28,7 @@
 namespace mi355 {
 namespace {
 
-// PW = pointwise fast path: 1x1 filter, no padding, K a multiple of the stage depth.  Its loaders need no
+// PW = pointwise fast path: 1x1 filter, no padding.  Its loaders need no
 // bounds tests and no k-unit table: every address is a per-row base plus a wave-uniform term.
 template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH, bool PW>
 struct IgemmKernel {
@@ -128,13 +128,17 @@ struct IgemmKernel {
             const int r = j % RB;
             const int kc = L.kc0 + cb + CSB * (j / RB);  // wave-uniform
             if (PW) {
+                // channel blocks past the last one (K not a whole number of stages) read as zeros
                 if (PIN == 32) {
-                    R.b[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_src, L.b_base[r] + kc * a.src_scb, 0, 0);
+                    R.b[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_src, kc < a.KC ? L.b_base[r] + kc * a.src_scb : SENT, 0, 0);
                 } else {
+                    const int lim = (a.kbytes >> 2) - (t & 1) * 4;  // this lane's half starts 4 blocks further on
                     v4i x;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        x[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_src, L.b_base[r] + (kc * 8 + i) * a.src_scb, 0, 0);
+                    for (int i = 0; i < 4; ++i) {
+                        const int cbi = kc * 8 + i;
+                        x[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_src, cbi < lim ? L.b_base[r] + cbi * a.src_scb : SENT, 0, 0);
+                    }
                     R.b[j] = x;
                 }
             } else if (PIN == 32) {
@@ -447,8 +451,8 @@ int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
 
 template <int PIN, int POUT, int BM, int BN, int WM, int WN, int KCH, int MINW>
 int launch_one(hipStream_t st, IgemmArgs& a, int cu_count) {
-    // pointwise fast path: 1x1, no padding, whole stages of K
-    const bool pw = a.T == 1 && a.ph == 0 && a.pw == 0 && a.kbytes % (32 * KCH) == 0;
+    // pointwise fast path: 1x1, no padding (any K: the loaders zero the channel blocks past the last one)
+    const bool pw = a.T == 1 && a.ph == 0 && a.pw == 0;
     if (pw) return launch_pw<PIN, POUT, BM, BN, WM, WN, KCH, MINW, true>(st, a, cu_count);
     return launch_pw<PIN, POUT, BM, BN, WM, WN, KCH, MINW, false>(st, a, cu_count);
 }
