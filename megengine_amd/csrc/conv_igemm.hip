@@ -512,7 +512,12 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
     if (cu_count <= 0) cu_count = 256;
     auto tiles = [&](int cfg) { return ((OC + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm) * ((M + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn); };
     const int kbytes = d.ic * d.fh * d.fw;
-    if (OC <= 32) return 4;
+    if (OC <= 32) {
+        // 32 x 256 tiles waste no matrix rows, but need enough pixels to fill the chip (measured on the 4-packed
+        // 1x1 projections of MobileNetV2)
+        if (p.pin == 32 || tiles(4) >= 2 * cu_count) return 4;
+        return tiles(0) >= cu_count ? 0 : 3;
+    }
     if (p.pin == 32) {
         // 32-packed inputs: LDS-direct tiles (ids after the register-staged ones), chosen from a sweep of every
         // tile over the ResNet-50 / large-convolution shapes.  t128 = number of 128x128 tiles.
