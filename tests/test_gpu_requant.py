@@ -135,3 +135,38 @@ def test_typecvt_float32_to_int8_and_back(oracle):
     buf = torch.zeros(64, dtype=torch.float32).cuda()
     with pytest.raises(Mi355Error, match="alignment"):
         ops.typecvt_exec(buf[1:33], 1.0)
+
+
+def test_linear_form_on_every_int32():
+    """The one-instruction form against the multi-step form on ALL 2^32 inputs, on the device: an all-zero second
+    input forces the multi-step form (r + 0.0 is exact, so it computes the same function), which the sweeps above pin
+    to the CPU checker."""
+    import ctypes as C
+    from megengine_amd import lib
+    chunk = 1 << 26
+    base = torch.arange(chunk, dtype=torch.int64, device="cuda")
+    zeros = torch.zeros(chunk, dtype=torch.int8, device="cuda")
+    rng = np.random.RandomState(5)
+    drawn = []
+    for _ in range(10):   # scale pairs drawn the way the workloads draw them
+        a, b, s_dst = (float(np.float32(np.exp(rng.uniform(np.log(1e-3), np.log(5e-2))))) for _ in range(3))
+        drawn.append((float(np.float32(a) * np.float32(b)), s_dst))
+    checked = 0
+    for i, (s_src, s_dst) in enumerate([(1.3e-3, 0.0271), (0.5, 1.0), (3.1e-5, 0.011)] + drawn):
+        for nl in ("IDENTITY", "RELU"):
+            c, d = C.c_float(), C.c_float()
+            have = lib.lib().mi355_epilogue_linear_form(s_src, s_dst, NL[nl], C.byref(c), C.byref(d))
+            assert have == 1 or i >= 3, (s_src, s_dst, nl)
+            if have != 1:
+                continue   # no proved form for this drawn pair: the kernels run the multi-step form
+            checked += 1
+            say("linear form, all int32", s_src, s_dst, nl, "c", c.value, "d", d.value)
+            for k in range(-(1 << 31) // chunk, (1 << 31) // chunk):
+                x = (base + k * chunk).to(torch.int32)
+                lin = ops.requant_exec(x, s_src, s_dst, nonline=nl)
+                ref = ops.requant_exec(x, s_src, s_dst, nonline=nl, z=zeros, scale_z=0.37)
+                if not torch.equal(lin, ref):
+                    bad = torch.nonzero(lin != ref)[0].item()
+                    raise AssertionError("x=%d: linear %d, multi-step %d (scales %r %r, %s)" % (
+                        int(x[bad]), int(lin[bad]), int(ref[bad]), s_src, s_dst, nl))
+    assert checked >= 18, checked
