@@ -496,7 +496,7 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
         case 11: return launch_one<POUT, 128, 64, 2, 2, 4, 2, 2>(st, a, cu);
         case 12: return launch_one<POUT, 64, 64, 2, 2, 4, 4, 3>(st, a, cu);
         case 13: return launch_one<POUT, 64, 128, 2, 2, 4, 2, 2>(st, a, cu);
-        case 14: return launch_one<POUT, 128, 128, 2, 4, 2, 3, 2>(st, a, cu);
+        case 14: return launch_one<POUT, 128, 128, 2, 4, 2, 3, 6>(st, a, cu);  // 80 VGPRs: three 8-wave workgroups per CU
         case 15: return launch_one<POUT, 128, 64, 4, 2, 4, 3, 2>(st, a, cu);
         case 16: return launch_one<POUT, 256, 128, 4, 2, 2, 3, 4>(st, a, cu);
         case 17: return launch_one<POUT, 128, 128, 2, 4, 4, 2, 2>(st, a, cu);
