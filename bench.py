@@ -318,8 +318,9 @@ def run_extras(torch, np, util, _abi, lib, ops, workloads):
         rows = []
         for p in plan:
             p["algo"], _ = ops.conv_bias_query(p["desc"])
-            t = time_launches(torch, lambda: ops.conv_bias_exec(p["desc"], p["src"], p["flt"], p["bias"], p["z"],
-                                                                dst=p["dst"], algo=p["algo"]))
+            # pre-marshalled launches: the per-call Python work of conv_bias_exec would floor short kernels
+            call = ops.conv_bias_bind(p["desc"], p["src"], p["flt"], p["bias"], p["z"], p["dst"], p["algo"])
+            t = time_launches(torch, call, iters=50)
             l = p["layer"]
             rows.append(dict(name=l.name, algo=lib.algo_names()[p["algo"].id], us=round(t * 1e6, 2),
                              tops=round(l.ops / t / 1e12, 1), gbs=round(l.bytes / t / 1e9, 1),
