@@ -220,9 +220,10 @@ def main():
 
     out = dict(metric="ResNet-50 int8 conv-stack throughput @ bs64 (53 ConvBias layers)", value=round(img_s, 1),
                unit="img/s", n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_per_step, 4),
-               higher_is_better=True, scaling="weak", vs_baseline=None, dtype="s8*s8->s32 accumulate, f32 requant",
+               higher_is_better=True, scaling="weak", vs_baseline=None, dtype="s8",
                data="synthetic",
-               config=dict(workload="BASELINE configs[2]: ResNet-50 v1.5 int8 conv stack, batch 64, 224x224, "
+               config=dict(arithmetic="s8 x s8 products accumulated in s32 (exact), requantised to s8 through f32 as the reference does",
+                           workload="BASELINE configs[2]: ResNet-50 v1.5 int8 conv stack, batch 64, 224x224, "
                                     "NCHW4 stem + NCHW32, fused residual z + RELU, random per-tensor scales",
                            batch=batch, layers=nl, launch=launch_mode, graph=graph_note),
                eager_ms_per_step=round(eager_ms, 4),
