@@ -525,7 +525,7 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
             D128x128x64 = kNumCfgs + 0, D64x64x128 = kNumCfgs + 1, D128x128x128r2 = kNumCfgs + 7, D64x64x64r4 = kNumCfgs + 10,
             D128x64x128r2 = kNumCfgs + 11, D64x128x128r2 = kNumCfgs + 13, D128x128x64w8 = kNumCfgs + 14,
             D128x64x128w8 = kNumCfgs + 15, D256x128x64w8 = kNumCfgs + 16, D128x128x128r2w8 = kNumCfgs + 17,
-            D64x64x128r2 = kNumCfgs + 6, D64x128x128w8 = kNumCfgs + 18
+            D64x64x128r2 = kNumCfgs + 6, D64x128x128w8 = kNumCfgs + 18, D64x64x128r4 = kNumCfgs + 12
         };
         if (OC <= 64) return kbytes <= 64 ? D128x128x64w8 : kbytes <= 256 ? D64x64x128r2 : D64x128x128r2;
         const int64_t t128 = tiles(0);
@@ -536,7 +536,11 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
         // few tiles, long reductions: the deeper ring hides the cold first touch of every weight byte; the longest
         // ones (3x3 over 256 channels) run best with more pixels than channels per tile
         if (kbytes >= 2304 && tiles(6) >= cu_count) return D64x128x128w8;
-        return tiles(7) >= cu_count ? D128x64x128w8 : D64x64x128;
+        if (tiles(7) >= cu_count) return D128x64x128w8;
+        // fewer tiles than CUs: the longest reductions (3x3 over 512 channels) take the deepest ring, 2048-channel
+        // pointwise layers the 8-wave tile with more pixels than channels
+        if (kbytes >= 4608) return D64x64x128r4;
+        return kbytes >= 2048 && 4 * tiles(6) >= 3 * cu_count ? D64x128x128w8 : D64x64x128;
     }
     if (OC <= 64) return tiles(1) >= cu_count ? 1 : 3;
     // 128x128 tiles as soon as they give every CU 1.5 tiles; the deeper k stage pays once the
