@@ -512,6 +512,13 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
     if (cu_count <= 0) cu_count = 256;
     auto tiles = [&](int cfg) { return ((OC + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm) * ((M + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn); };
     const int kbytes = d.ic * d.fh * d.fw;
+    if (p.pin == 4 && p.pout == 4 && d.fh == 1 && d.fw == 1 && d.pad_h == 0 && d.pad_w == 0) {
+        // 4-packed pointwise layers (per-tile sweep of the MobileNetV2 1x1 layers): the LDS-direct tiles win wherever the
+        // register-staged loop is latency-bound -- narrow outputs, and few tiles with a long reduction
+        enum { D4_128x128x64 = kNumCfgs + 19, D4_64x64x128 = kNumCfgs + 20, D4_128x64x128 = kNumCfgs + 21 };
+        if (OC <= 32 && kbytes <= 256) return D4_128x128x64;
+        if (OC > 32 && 2 * tiles(0) < 3 * cu_count) return kbytes >= 192 ? D4_64x64x128 : D4_128x64x128;
+    }
     if (OC <= 32) {
         // 32 x 256 tiles waste no matrix rows, but need enough pixels to fill the chip (measured on the 4-packed
         // 1x1 projections of MobileNetV2)
@@ -584,8 +591,11 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
     if (cfg >= kNumCfgs) {
         const int dcfg = cfg - kNumCfgs;
         if (dcfg >= igemm_dma_num_cfgs()) return (int)hipErrorInvalidValue;
-        if (p.pin == 32) return launch_igemm_dma(st, a, p.pout, dcfg, cu_count);
-        // 4-packed inputs have no LDS-direct path: run the register-staged tile of the same shape
+        const bool c4 = igemm_dma_cfg_is_pin4(dcfg);
+        if (!c4 && p.pin == 32) return launch_igemm_dma(st, a, p.pout, dcfg, cu_count);
+        if (c4 && p.pin == 4 && p.pout == 4 && a.T == 1 && a.ph == 0 && a.pw == 0)
+            return launch_igemm_dma(st, a, 4, dcfg, cu_count);
+        // no LDS-direct kernel for this packing / filter: run the register-staged tile of the same shape
         int bm, bn, kch;
         igemm_dma_cfg_shape(dcfg, &bm, &bn, &kch);
         cfg = 0;

@@ -38,6 +38,17 @@ __device__ __forceinline__ void lds_copy64x16(uint32_t lds_addr, int voff, const
         : "memory");  // M0 is reserved by the compiler (never allocated), so it needs no clobber entry
 }
 
+// 64 x 4 bytes: lane l lands at M0 + 4 * l (4-packed activations: one pixel's channel block per lane)
+__device__ __forceinline__ void lds_copy64x4(uint32_t lds_addr, int voff, const v4i& rsrc) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dword %1, %2, 0 offen lds"
+        :
+        : "s"(lds_addr), "v"(voff), "s"(rsrc)
+        : "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N < 64, "vmcnt range");
@@ -66,7 +77,11 @@ __device__ __forceinline__ v4i uniform_rsrc(const void* p, uint32_t bytes) {
     return r;
 }
 
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, bool PW>
+// PIN = 4 (4-packed activations, pointwise only): a pixel's 4 channels are the only contiguous bytes, so the
+// activation tile travels as 64 x 4-byte copies -- lane = pixel, one channel block per copy -- and sits in LDS as
+// [block of 64 pixels][channel block][pixel] dwords; an MFMA B fragment (16 k-bytes of one pixel = 4 channel blocks)
+// is read as four dwords 256 bytes apart.  Filters are laid out and copied exactly as for 32-packed inputs.
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, bool PW, int PIN = 32>
 struct DmaKernel {
     static constexpr int NW = WM * WN;             // waves per workgroup (4 or 8)
     static constexpr int THREADS = NW * 64;
@@ -78,12 +93,19 @@ struct DmaKernel {
     static constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB;
     static constexpr int STG = A_BYTES + B_BYTES;  // one stage
     static constexpr int UA = BM / (RPL * NW);     // copies per wave per stage
-    static constexpr int UB = BN / (RPL * NW);
+    static constexpr int UB32 = BN / (RPL * NW);
+    static constexpr int NB64 = BN / 64;           // 4-packed: blocks of 64 pixels
+    static constexpr int CB = KCH * 8;             // 4-packed: channel blocks per stage
+    static constexpr int UB4 = NB64 * CB / NW;     // 4-packed: dword copies per wave per stage
+    static constexpr int CPB = CB / NW;            // ... of which per pixel block
+    static constexpr int UB = PIN == 4 ? UB4 : UB32;
+    static constexpr int NOFF = PIN == 4 ? (NB64 > 0 ? NB64 : 1) : UB32;  // per-lane activation offsets kept by the loader
     static constexpr int U = UA + UB;
+    static_assert(PIN == 32 || (PIN == 4 && PW && BN % 64 == 0 && CB % NW == 0), "4-packed inputs: pointwise tiles of whole 64-pixel blocks");
     static constexpr int BIAS_BYTES = BM * 4;  // bias of the workgroup's channel tile
     static constexpr int RING_BYTES = NS * STG + BIAS_BYTES;
     static_assert(NW == 4 || NW == 8, "4 or 8 waves");
-    static_assert(UA >= 1 && UB >= 1 && BM % (RPL * NW) == 0 && BN % (RPL * NW) == 0, "tile vs copy granularity");
+    static_assert(UA >= 1 && UB >= 1 && BM % (RPL * NW) == 0 && (PIN == 4 || BN % (RPL * NW) == 0), "tile vs copy granularity");
     static_assert(NS >= 2 && (NS - 2) * U < 64, "ring depth");
     // swz() looks at row bits 0..3; rows of copy j of wave w are (NW j + w) * RPL + lane / S, so with RPL >= 8 those
     // bits never depend on j: a lane's logical slot is the same for all of its copies
@@ -92,8 +114,8 @@ struct DmaKernel {
     struct Loader {
         int tile, stage, kc0;
         int a_off[UA];            // filter: byte offset of (row, logical slot), SENT past OC
-        int b_off[UB];            // activation: byte offset of the pixel (+ chunk / half for the pointwise path)
-        int ih0[UB], iw0[UB];     // table path: top-left input coordinate (ih0 = -0x8000 past M)
+        int b_off[NOFF];          // activation: byte offset of the pixel (+ chunk / half for the pointwise path)
+        int ih0[NOFF], iw0[NOFF]; // table path: top-left input coordinate (ih0 = -0x8000 past M)
     };
 
     __device__ static __forceinline__ void tile_coords(const IgemmArgs& a, int tile, int& oc0, int& pix0) {
@@ -114,6 +136,18 @@ struct DmaKernel {
         for (int j = 0; j < UA; ++j) {
             const int oc = oc0 + row_of(w, lane, j);
             L.a_off[j] = oc < a.OC ? oc * a.kbytes + s * 16 : SENT;
+        }
+        if (PIN == 4) {
+#pragma unroll
+            for (int b = 0; b < NB64; ++b) {
+                const int m = pix0 + b * 64 + lane;
+                const bool ok = m < a.M;
+                const uint32_t mm = ok ? m : 0;
+                const uint32_t n = fdiv(mm, a.div_ohw), rem = mm - n * a.OHW;
+                const uint32_t oh = fdiv(rem, a.div_ow), ow = rem - oh * a.OW;
+                L.b_off[b] = ok ? (int)n * a.src_sn + ((int)oh * a.sh * a.IW + (int)ow * a.sw) * 4 : SENT;
+            }
+            return;
         }
 #pragma unroll
         for (int j = 0; j < UB; ++j) {
@@ -138,7 +172,7 @@ struct DmaKernel {
 #pragma unroll
         for (int j = 0; j < UA; ++j) L.a_off[j] = SENT;
 #pragma unroll
-        for (int j = 0; j < UB; ++j) {
+        for (int j = 0; j < NOFF; ++j) {
             L.b_off[j] = SENT;
             L.ih0[j] = -0x8000;
         }
@@ -157,7 +191,19 @@ struct DmaKernel {
             // SENT plus a stage offset is still out of range
             lds_copy64x16(stage_addr + (uint32_t)((NW * j + w) * 1024), L.a_off[j] + a_k, rs_flt);
         }
-        if (PW) {
+        if (PIN == 4) {
+            // copy j of wave w: pixel block j / CPB, channel block (j % CPB) * NW + w of this stage.  A channel block
+            // past the last one (K not a whole number of stages) reads as zeros: SENT plus a pixel offset stays out
+            // of range; SENT plus SENT (a row past M as well) wraps to offset 0, whose bytes only meet discarded rows
+            const int icb = a.kbytes >> 2;
+#pragma unroll
+            for (int j = 0; j < UB4; ++j) {
+                const int cbl = (j % CPB) * NW + w;
+                const int cb = L.kc0 * 8 + cbl;
+                const int k_off = cb < icb ? cb * a.src_scb : SENT;  // wave-uniform
+                lds_copy64x4(stage_addr + (uint32_t)(A_BYTES + ((j / CPB) * CB + cbl) * 256), (int)((uint32_t)L.b_off[j / CPB] + (uint32_t)k_off), rs_src);
+            }
+        } else if (PW) {
             const int b_k = L.kc0 * a.src_scb;
 #pragma unroll
             for (int j = 0; j < UB; ++j) {
@@ -284,7 +330,9 @@ struct DmaKernel {
             advance();
         }
         v16i acc[MT][NT];
-        wait_vmcnt_for<(NS - 1) * U>(bias_reg);  // older than every copy of the prologue
+        // older than every copy of the prologue (the counter holds at most 63: with more copies than that in the
+        // prologue the oldest operations, this one first, have completed by the time the last copy was accepted)
+        wait_vmcnt_for<((NS - 1) * U < 63 ? (NS - 1) * U : 63)>(bias_reg);
         if (t < BM) sBias[t] = bias_reg;
         __syncthreads();
         init_acc_lds(acc, sBias, wm, lh);
@@ -310,8 +358,13 @@ struct DmaKernel {
 #pragma unroll
                 for (int j = 0; j < NT; ++j) {
                     const int row = wn * WTN + j * 32 + l32;
-                    const int slot = (c * 2 + lh) ^ swz<S>(row);
-                    xb[j] = *reinterpret_cast<const v4i*>(pB + row * ROWB + slot * 16);
+                    if (PIN == 4) {
+                        const int* q = reinterpret_cast<const int*>(pB) + ((row >> 6) * CB + c * 8 + lh * 4) * 64 + (row & 63);
+                        xb[j][0] = q[0]; xb[j][1] = q[64]; xb[j][2] = q[128]; xb[j][3] = q[192];
+                    } else {
+                        const int slot = (c * 2 + lh) ^ swz<S>(row);
+                        xb[j] = *reinterpret_cast<const v4i*>(pB + row * ROWB + slot * 16);
+                    }
                 }
             };
             auto mfmas = [&](int c, const v4i (&xa)[MT], const v4i (&xb)[NT]) __attribute__((always_inline)) {
@@ -398,9 +451,9 @@ struct DmaKernel {
     }
 };
 
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW>
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, int PIN = 32>
 __global__ __launch_bounds__(WM * WN * 64, MINW) void igemm_dma_kernel(IgemmArgs a) {
-    DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW>::run(a);
+    DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW, PIN>::run(a);
 }
 
 struct DmaCfg {
@@ -428,12 +481,18 @@ const DmaCfg kDma[] = {
         {"dma256x128x64w8", 256, 128, 2},
         {"dma128x128x128r2w8", 128, 128, 4},
         {"dma64x128x128w8", 64, 128, 4},
+        // 4-packed pointwise (NCHW4 in and out); other problems run the register-staged tile of the same shape
+        {"dma4_128x128x64", 128, 128, 2},
+        {"dma4_64x64x128", 64, 64, 4},
+        {"dma4_128x64x128", 128, 64, 4},
+        {"dma4_32x256x128", 32, 256, 4},
 };
+constexpr int kFirstDma4 = 19;
 constexpr int kNumDma = sizeof(kDma) / sizeof(kDma[0]);
 
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW>
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, int PIN = 32>
 int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
-    using K = DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW>;
+    using K = DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW, PIN>;
     a.tiles_m = (a.OC + BM - 1) / BM;
     a.tiles_n = (a.M + BN - 1) / BN;
     const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
@@ -442,7 +501,7 @@ int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
     a.nstages = (a.KC + KCH - 1) / KCH;
     const int tab_entries = PW ? 0 : a.nstages * KCH;
     const int lds = K::RING_BYTES + tab_entries * 8;
-    auto kern = igemm_dma_kernel<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW>;
+    auto kern = igemm_dma_kernel<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW, PIN>;
     // per-instantiation caches; atomics, because operators on different streams may launch from several threads
     static std::atomic<int> max_lds_set{0};
     if (lds > max_lds_set.load(std::memory_order_relaxed)) {
@@ -501,6 +560,10 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
         case 16: return launch_one<POUT, 256, 128, 4, 2, 2, 3, 4>(st, a, cu);
         case 17: return launch_one<POUT, 128, 128, 2, 4, 4, 2, 2>(st, a, cu);
         case 18: return launch_one<POUT, 64, 128, 2, 4, 4, 3, 2>(st, a, cu);
+        case 19: return launch_pw<4, 128, 128, 2, 2, 2, 3, 2, true, 4>(st, a, cu);
+        case 20: return launch_pw<4, 64, 64, 2, 2, 4, 4, 3, true, 4>(st, a, cu);
+        case 21: return launch_pw<4, 128, 64, 2, 2, 4, 3, 2, true, 4>(st, a, cu);
+        case 22: return launch_pw<4, 32, 256, 1, 4, 4, 3, 2, true, 4>(st, a, cu);
         default: return (int)hipErrorInvalidValue;
     }
 }
@@ -512,6 +575,8 @@ const char* igemm_dma_cfg_name(int cfg) { return cfg >= 0 && cfg < kNumDma ? kDm
 void igemm_dma_cfg_shape(int cfg, int* bm, int* bn, int* kch) {
     *bm = kDma[cfg].bm; *bn = kDma[cfg].bn; *kch = kDma[cfg].kch;
 }
+
+bool igemm_dma_cfg_is_pin4(int cfg) { return cfg >= kFirstDma4; }
 
 int launch_igemm_dma(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count) {
     return pout == 32 ? launch_fmt<32>(st, a, cfg, cu_count) : launch_fmt<4>(st, a, cfg, cu_count);

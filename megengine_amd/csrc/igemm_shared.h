@@ -182,6 +182,7 @@ __device__ __forceinline__ void igemm_run_epilogue(const IgemmArgs& a, v16i (&ac
 int igemm_dma_num_cfgs();
 const char* igemm_dma_cfg_name(int cfg);
 void igemm_dma_cfg_shape(int cfg, int* bm, int* bn, int* kch);
+bool igemm_dma_cfg_is_pin4(int cfg);  // a 4-packed pointwise tile (NCHW4 in and out, 1x1, no padding)
 int launch_igemm_dma(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count);
 
 }  // namespace mi355

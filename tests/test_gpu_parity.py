@@ -131,6 +131,9 @@ IGEMM_CASES = [
     ("NCHW4", 2, 24, 8, 8, 144, 1, 0, 1),       # MobileNetV2 expand
     ("NCHW4", 2, 144, 8, 8, 24, 1, 0, 1),       # MobileNetV2 project (oc < 32)
     ("NCHW4", 1, 12, 9, 7, 20, 3, 1, 2),        # oc % 32 != 0, K = 108
+    ("NCHW4", 3, 40, 7, 7, 40, 1, 0, 1),        # 4-packed pointwise: K = 40 and oc = 40 ragged, 147 pixels, images of 49
+    ("NCHW4", 2, 96, 9, 9, 24, 1, 0, 2),        # 4-packed pointwise, stride 2, narrow output
+    ("NCHW4", 2, 192, 6, 6, 72, 1, 0, 1),       # 4-packed pointwise, several k-stages
     ("NCHW4_NCHW32", 2, 16, 8, 8, 64, 3, 1, 1),
     ("NCHW32_NCHW4", 2, 64, 8, 8, 24, 3, 1, 1),
 ]
@@ -252,7 +255,9 @@ RAGGED = [
     ("NCHW32", 1, 64, 13, 5, 224, 5, 2, 2, "RELU", False, {}),           # 5x5 stride 2, one image
     ("NCHW32_NCHW4", 2, 64, 8, 8, 40, 3, 1, 1, "RELU", False, {}),       # 32-packed in, 4-packed out, oc % 32 != 0
     ("NCHW32", 4, 128, 6, 6, 64, 3, 1, 0, "RELU", True, {"batch_pad": 64}),  # batch-strided src / dst / z views
-    ("NCHW4", 2, 24, 9, 9, 48, 3, 1, 1, "RELU", True, {}),               # 4-packed: LDS-direct ids fall back
+    ("NCHW4", 2, 24, 9, 9, 48, 3, 1, 1, "RELU", True, {}),               # 4-packed 3x3: LDS-direct ids fall back
+    ("NCHW4", 3, 64, 6, 6, 64, 1, 1, 0, "RELU", True, {"batch_pad": 64}),  # 4-packed pointwise, batch-strided views
+    ("NCHW4", 2, 160, 7, 7, 100, 1, 1, 0, "H_SWISH", True, {}),          # 4-packed pointwise, ragged everything
 ]
 
 
