@@ -515,7 +515,9 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
     if (p.pin == 4 && p.pout == 4 && d.fh == 1 && d.fw == 1 && d.pad_h == 0 && d.pad_w == 0) {
         // 4-packed pointwise layers (per-tile sweep of the MobileNetV2 1x1 layers): the LDS-direct tiles win wherever the
         // register-staged loop is latency-bound -- narrow outputs, and few tiles with a long reduction
-        enum { D4_128x128x64 = kNumCfgs + 19, D4_64x64x128 = kNumCfgs + 20, D4_128x64x128 = kNumCfgs + 21 };
+        enum { D4_128x128x64 = kNumCfgs + 19, D4_64x64x128 = kNumCfgs + 20, D4_128x64x128 = kNumCfgs + 21, PW4_STREAM = kNumCfgs + 23 };
+        // at most 64 channels in, many out (the expansions): the streaming kernel, which has no per-tile pipeline
+        if (kbytes <= 64 && OC >= 64 && OC <= 1024) return PW4_STREAM;
         if (OC <= 32 && kbytes <= 256) return D4_128x128x64;
         if (OC > 32 && 2 * tiles(0) < 3 * cu_count) return kbytes >= 192 ? D4_64x64x128 : D4_128x64x128;
     }

@@ -486,6 +486,8 @@ const DmaCfg kDma[] = {
         {"dma4_64x64x128", 64, 64, 4},
         {"dma4_128x64x128", 128, 64, 4},
         {"dma4_32x256x128", 32, 256, 4},
+        // no tile at all: the streaming kernel of conv_pw4.hip where it applies, else dma4_128x128x64
+        {"pw4_stream", 128, 128, 2},
 };
 constexpr int kFirstDma4 = 19;
 constexpr int kNumDma = sizeof(kDma) / sizeof(kDma[0]);
@@ -564,6 +566,7 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
         case 20: return launch_pw<4, 64, 64, 2, 2, 4, 4, 3, true, 4>(st, a, cu);
         case 21: return launch_pw<4, 128, 64, 2, 2, 4, 3, 2, true, 4>(st, a, cu);
         case 22: return launch_pw<4, 32, 256, 1, 4, 4, 3, 2, true, 4>(st, a, cu);
+        case 23: return pw4s_usable(a) ? launch_pw4s(st, a, cu) : launch_pw<4, 128, 128, 2, 2, 2, 3, 2, true, 4>(st, a, cu);
         default: return (int)hipErrorInvalidValue;
     }
 }

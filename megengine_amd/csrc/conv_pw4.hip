@@ -1,0 +1,112 @@
+// Pointwise (1x1) int8 ConvBias on 4-packed activations with at most 64 input channels, NCHW4 in and out: the
+// expansion layers of the MobileNet family, whose reduction is one or two MFMA k-steps and whose cost is their output.
+//
+// A tiled implicit GEMM spends such a layer on its per-tile pipeline (stage, barrier, multiply: one k-stage per tile).
+// Here nothing is staged and nothing is shared after the first barrier:
+//   * a wave keeps the filter rows of its 64 or 96 output channels in registers for the whole launch
+//     (MFMA A fragments: lane = output channel, 16 contiguous k-bytes of its row);
+//   * it walks blocks of 32 pixels; a lane's B fragment -- 16 k-bytes of its pixel = 4 channel blocks -- is four
+//     coalesced dword loads (32 consecutive pixels x 4 bytes each), fetched for the NEXT block while this one is
+//     multiplied and requantised;
+//   * accumulators start from the bias (LDS copy), the fused epilogue and the NCHW4 stores are those of the tiled
+//     kernels (igemm_shared.h).
+// Channel blocks past the last one, and filter bytes past the end of a row, meet zero activations.
+#include "igemm_shared.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int PW4_MAX_OC = 1024;
+
+template <int MT, int KC>
+__global__ __launch_bounds__(256) void pw4s_kernel(IgemmArgs a, int n_ocg, int n_pb) {
+    __shared__ __attribute__((aligned(16))) int sBias[PW4_MAX_OC + 96];
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int l32 = lane & 31, lh = lane >> 5;
+    for (int i = t; i < PW4_MAX_OC + 96; i += 256) sBias[i] = (a.has_bias && i < a.OC) ? a.bias[i] : 0;
+    __syncthreads();
+
+    const int gw = blockIdx.x * 4 + wave, GW = gridDim.x * 4;  // GW is a multiple of n_ocg
+    const int pb0 = gw / n_ocg, ocg = gw - pb0 * n_ocg, step = GW / n_ocg;
+    const int oc_w = ocg * MT * 32;
+    const __amdgpu_buffer_rsrc_t rs_src = make_rsrc(a.src, a.src_bytes);
+    const __amdgpu_buffer_rsrc_t rs_flt = make_rsrc(a.flt, a.flt_bytes);
+
+    v4i fa[MT][KC];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int row = oc_w + i * 32 + l32;
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc)
+            fa[i][kc] = __builtin_amdgcn_raw_buffer_load_b128(rs_flt, row < a.OC ? row * a.kbytes + kc * 32 + lh * 16 : SENT, 0, 0);
+    }
+
+    const int icb = a.kbytes >> 2;
+    auto load_b = [&](int pb, v4i (&x)[KC]) __attribute__((always_inline)) {
+        const int m = pb * 32 + l32;
+        const bool ok = m < a.M;  // also false for every block past the last one
+        const uint32_t mm = ok ? m : 0;
+        const uint32_t n = fdiv(mm, a.div_ohw), rem = mm - n * a.OHW;
+        const uint32_t oh = fdiv(rem, a.div_ow), ow = rem - oh * a.OW;
+        const int pix = (int)n * a.src_sn + ((int)oh * a.sh * a.IW + (int)ow * a.sw) * 4;
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int cb = kc * 8 + lh * 4 + i;
+                x[kc][i] = __builtin_amdgcn_raw_buffer_load_b32(rs_src, (ok && cb < icb) ? pix + cb * a.src_scb : SENT, 0, 0);
+            }
+    };
+
+    v4i fb[KC], nb[KC];
+    load_b(pb0, fb);
+    for (int pb = pb0; pb < n_pb; pb += step) {
+        load_b(pb + step, nb);  // in flight during the multiply and the epilogue
+        v16i acc[MT][1];
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const v4i b = *reinterpret_cast<const v4i*>(sBias + oc_w + i * 32 + 8 * q + 4 * lh);
+                acc[i][0][4 * q + 0] = b[0]; acc[i][0][4 * q + 1] = b[1]; acc[i][0][4 * q + 2] = b[2]; acc[i][0][4 * q + 3] = b[3];
+            }
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+            for (int i = 0; i < MT; ++i) acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i][kc], fb[kc], acc[i][0], 0, 0, 0);
+        igemm_run_epilogue<4, MT, 1>(a, acc, oc_w, pb * 32, l32, lh);
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) fb[kc] = nb[kc];
+    }
+}
+
+template <int MT, int KC>
+int launch_mt(hipStream_t st, const IgemmArgs& a, int cu_count) {
+    const int ocb = (a.OC + 31) / 32;
+    const int n_ocg = (ocb + MT - 1) / MT;
+    const int n_pb = (a.M + 31) / 32;
+    if (cu_count <= 0) cu_count = 256;
+    int64_t blocks = ((int64_t)n_pb * n_ocg + 3) / 4;
+    const int64_t cap = (int64_t)cu_count * 4;  // 16 waves per CU
+    if (blocks > cap) blocks = cap;
+    blocks = (blocks + n_ocg - 1) / n_ocg * n_ocg;  // waves of one pixel block stay together; 4 * blocks % n_ocg == 0
+    hipLaunchKernelGGL((pw4s_kernel<MT, KC>), dim3((unsigned)blocks), dim3(256), 0, st, a, n_ocg, n_pb);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+bool pw4s_usable(const IgemmArgs& a) {
+    return a.T == 1 && a.ph == 0 && a.pw == 0 && a.kbytes <= 64 && a.OC <= PW4_MAX_OC;
+}
+
+int launch_pw4s(hipStream_t st, const IgemmArgs& a, int cu_count) {
+    if (a.M == 0 || a.OC == 0) return 0;
+    const int ocb = (a.OC + 31) / 32;
+    const bool three = ocb % 3 == 0 || ocb > 4;  // 96-channel waves unless the channel count splits evenly into 64s
+    if (a.kbytes <= 32) return three ? launch_mt<3, 1>(st, a, cu_count) : launch_mt<2, 1>(st, a, cu_count);
+    return three ? launch_mt<3, 2>(st, a, cu_count) : launch_mt<2, 2>(st, a, cu_count);
+}
+
+}  // namespace mi355

@@ -134,6 +134,7 @@ IGEMM_CASES = [
     ("NCHW4", 3, 40, 7, 7, 40, 1, 0, 1),        # 4-packed pointwise: K = 40 and oc = 40 ragged, 147 pixels, images of 49
     ("NCHW4", 2, 96, 9, 9, 24, 1, 0, 2),        # 4-packed pointwise, stride 2, narrow output
     ("NCHW4", 2, 192, 6, 6, 72, 1, 0, 1),       # 4-packed pointwise, several k-stages
+    ("NCHW4", 2, 64, 9, 9, 96, 1, 0, 2),        # 4-packed pointwise, 64 channels in (two k-steps), stride 2
     ("NCHW4_NCHW32", 2, 16, 8, 8, 64, 3, 1, 1),
     ("NCHW32_NCHW4", 2, 64, 8, 8, 24, 3, 1, 1),
 ]
@@ -258,6 +259,8 @@ RAGGED = [
     ("NCHW4", 2, 24, 9, 9, 48, 3, 1, 1, "RELU", True, {}),               # 4-packed 3x3: LDS-direct ids fall back
     ("NCHW4", 3, 64, 6, 6, 64, 1, 1, 0, "RELU", True, {"batch_pad": 64}),  # 4-packed pointwise, batch-strided views
     ("NCHW4", 2, 160, 7, 7, 100, 1, 1, 0, "H_SWISH", True, {}),          # 4-packed pointwise, ragged everything
+    ("NCHW4", 3, 32, 6, 6, 200, 1, 1, 0, "RELU", True, {"batch_pad": 64}),  # few channels in, 7 channel blocks out, strided views
+    ("NCHW4", 5, 20, 7, 9, 36, 1, 1, 0, "IDENTITY", False, {}),          # few channels in: K = 20, oc = 36, 315 pixels
 ]
 
 
