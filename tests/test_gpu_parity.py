@@ -135,6 +135,8 @@ IGEMM_CASES = [
     ("NCHW4", 2, 96, 9, 9, 24, 1, 0, 2),        # 4-packed pointwise, stride 2, narrow output
     ("NCHW4", 2, 192, 6, 6, 72, 1, 0, 1),       # 4-packed pointwise, several k-stages
     ("NCHW4", 2, 64, 9, 9, 96, 1, 0, 2),        # 4-packed pointwise, 64 channels in (two k-steps), stride 2
+    ("NCHW4", 2, 100, 7, 7, 128, 1, 0, 1),      # streaming kernel: four k-steps, the last one ragged
+    ("NCHW4", 1, 160, 7, 7, 640, 1, 0, 1),      # streaming kernel: five k-steps, 20 channel blocks
     ("NCHW4_NCHW32", 2, 16, 8, 8, 64, 3, 1, 1),
     ("NCHW32_NCHW4", 2, 64, 8, 8, 24, 3, 1, 1),
 ]
