@@ -1,4 +1,5 @@
-// Implicit-GEMM int8 ConvBias with LDS-direct operand staging (32-packed inputs: NCHW32, NCHW32_NCHW4).
+// Implicit-GEMM int8 ConvBias with LDS-direct operand staging (32-packed inputs: NCHW32, NCHW32_NCHW4; 4-packed
+// inputs on the pointwise path, NCHW4 in and out: see PIN = 4 at DmaKernel).
 //
 // Same tiling, MFMA layout, LDS swizzle and fused epilogue as conv_igemm.hip; what differs is how a
 // k-stage travels from global memory to LDS:

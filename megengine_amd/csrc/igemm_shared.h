@@ -178,7 +178,7 @@ __device__ __forceinline__ void igemm_run_epilogue(const IgemmArgs& a, v16i (&ac
     }
 }
 
-// LDS-direct variant (conv_igemm_dma.hip): global -> LDS copies without a register stage; 32-packed inputs only
+// LDS-direct variant (conv_igemm_dma.hip): global -> LDS copies without a register stage
 int igemm_dma_num_cfgs();
 const char* igemm_dma_cfg_name(int cfg);
 void igemm_dma_cfg_shape(int cfg, int* bm, int* bn, int* kch);
