@@ -518,6 +518,8 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
         enum { D4_128x128x64 = kNumCfgs + 19, D4_64x64x128 = kNumCfgs + 20, D4_128x64x128 = kNumCfgs + 21, PW4_STREAM = kNumCfgs + 23 };
         // at most 64 channels in, many out (the expansions): the streaming kernel, which has no per-tile pipeline
         if (kbytes <= 64 && OC >= 64 && OC <= 1024) return PW4_STREAM;
+        // one channel block out (the narrow projections): the same kernel, up to six k-steps
+        if (OC <= 32 && kbytes <= 192) return PW4_STREAM;
         if (OC <= 32 && kbytes <= 256) return D4_128x128x64;
         if (OC > 32 && 2 * tiles(0) < 3 * cu_count) return kbytes >= 192 ? D4_64x64x128 : D4_128x64x128;
     }

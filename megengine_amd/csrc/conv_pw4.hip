@@ -1,13 +1,15 @@
-// Pointwise (1x1) int8 ConvBias on 4-packed activations with at most 64 input channels, NCHW4 in and out: the
-// expansion layers of the MobileNet family, whose reduction is one or two MFMA k-steps and whose cost is their output.
+// Pointwise (1x1) int8 ConvBias on 4-packed activations, NCHW4 in and out, for the two kinds of layer that a tiled
+// kernel serves badly: at most 64 input channels and many output channels (the expansion layers of the MobileNet
+// family: one or two MFMA k-steps, the cost is the output), and at most 32 output channels with up to 192 input
+// channels (its narrow projections: a tile of 128 filter rows would be three quarters empty).
 //
 // A tiled implicit GEMM spends such a layer on its per-tile pipeline (stage, barrier, multiply: one k-stage per tile).
 // Here nothing is staged and nothing is shared after the first barrier:
-//   * a wave keeps the filter rows of its 64 or 96 output channels in registers for the whole launch
+//   * a wave keeps the filter rows of its 32, 64 or 96 output channels in registers for the whole launch
 //     (MFMA A fragments: lane = output channel, 16 contiguous k-bytes of its row);
 //   * it walks blocks of 32 pixels; a lane's B fragment -- 16 k-bytes of its pixel = 4 channel blocks -- is four
-//     coalesced dword loads (32 consecutive pixels x 4 bytes each), fetched for the NEXT block while this one is
-//     multiplied and requantised;
+//     coalesced dword loads (32 consecutive pixels x 4 bytes each), fetched for the NEXT block, together with its
+//     residual, while this one is multiplied and requantised;
 //   * accumulators start from the bias (LDS copy), the fused epilogue and the NCHW4 stores are those of the tiled
 //     kernels (igemm_shared.h).
 // Channel blocks past the last one, and filter bytes past the end of a row, meet zero activations.
@@ -18,7 +20,8 @@ namespace {
 
 constexpr int PW4_MAX_OC = 1024;
 
-template <int MT, int KC>
+// HZ: the launch has a residual (its registers exist only in that instantiation)
+template <int MT, int KC, bool HZ>
 __global__ __launch_bounds__(256) void pw4s_kernel(IgemmArgs a, int n_ocg, int n_pb) {
     __shared__ __attribute__((aligned(16))) int sBias[PW4_MAX_OC + 96];
     const int t = threadIdx.x;
@@ -60,9 +63,13 @@ __global__ __launch_bounds__(256) void pw4s_kernel(IgemmArgs a, int n_ocg, int n
     };
 
     v4i fb[KC], nb[KC];
+    ZRegs<HZ ? MT : 1, 1> zr, nz;
     load_b(pb0, fb);
+    if constexpr (HZ) igemm_load_z<4, MT, 1>(a, zr, oc_w, pb0 * 32, l32, lh);
     for (int pb = pb0; pb < n_pb; pb += step) {
-        load_b(pb + step, nb);  // in flight during the multiply and the epilogue
+        // the next block's pixels and residual are in flight during the multiply and the epilogue
+        load_b(pb + step, nb);
+        if constexpr (HZ) igemm_load_z<4, MT, 1>(a, nz, oc_w, (pb + step) * 32, l32, lh);
         v16i acc[MT][1];
 #pragma unroll
         for (int i = 0; i < MT; ++i)
@@ -75,9 +82,13 @@ __global__ __launch_bounds__(256) void pw4s_kernel(IgemmArgs a, int n_ocg, int n
         for (int kc = 0; kc < KC; ++kc)
 #pragma unroll
             for (int i = 0; i < MT; ++i) acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i][kc], fb[kc], acc[i][0], 0, 0, 0);
-        igemm_run_epilogue<4, MT, 1>(a, acc, oc_w, pb * 32, l32, lh);
+        if constexpr (HZ)
+            igemm_run_epilogue<4, MT, 1, true>(a, acc, oc_w, pb * 32, l32, lh, &zr);
+        else
+            igemm_run_epilogue<4, MT, 1>(a, acc, oc_w, pb * 32, l32, lh);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc) fb[kc] = nb[kc];
+        if constexpr (HZ) zr = nz;
     }
 }
 
@@ -91,19 +102,33 @@ int launch_mt(hipStream_t st, const IgemmArgs& a, int cu_count) {
     const int64_t cap = (int64_t)cu_count * 4;  // 16 waves per CU
     if (blocks > cap) blocks = cap;
     blocks = (blocks + n_ocg - 1) / n_ocg * n_ocg;  // waves of one pixel block stay together; 4 * blocks % n_ocg == 0
-    hipLaunchKernelGGL((pw4s_kernel<MT, KC>), dim3((unsigned)blocks), dim3(256), 0, st, a, n_ocg, n_pb);
+    if (a.epi.has_z)
+        hipLaunchKernelGGL((pw4s_kernel<MT, KC, true>), dim3((unsigned)blocks), dim3(256), 0, st, a, n_ocg, n_pb);
+    else
+        hipLaunchKernelGGL((pw4s_kernel<MT, KC, false>), dim3((unsigned)blocks), dim3(256), 0, st, a, n_ocg, n_pb);
     return (int)hipGetLastError();
 }
 
 }  // namespace
 
 bool pw4s_usable(const IgemmArgs& a) {
-    return a.T == 1 && a.ph == 0 && a.pw == 0 && a.kbytes <= 64 && a.OC <= PW4_MAX_OC;
+    if (a.T != 1 || a.ph != 0 || a.pw != 0 || a.OC > PW4_MAX_OC) return false;
+    return a.kbytes <= 64 || (a.OC <= 32 && a.kbytes <= 192);
 }
 
 int launch_pw4s(hipStream_t st, const IgemmArgs& a, int cu_count) {
     if (a.M == 0 || a.OC == 0) return 0;
     const int ocb = (a.OC + 31) / 32;
+    if (ocb == 1) {  // narrow outputs (the projections): one channel block per wave, up to six k-steps
+        switch ((a.kbytes + 31) / 32) {
+            case 1: return launch_mt<1, 1>(st, a, cu_count);
+            case 2: return launch_mt<1, 2>(st, a, cu_count);
+            case 3: return launch_mt<1, 3>(st, a, cu_count);
+            case 4: return launch_mt<1, 4>(st, a, cu_count);
+            case 5: return launch_mt<1, 5>(st, a, cu_count);
+            default: return launch_mt<1, 6>(st, a, cu_count);
+        }
+    }
     const bool three = ocb % 3 == 0 || ocb > 4;  // 96-channel waves unless the channel count splits evenly into 64s
     if (a.kbytes <= 32) return three ? launch_mt<3, 1>(st, a, cu_count) : launch_mt<2, 1>(st, a, cu_count);
     return three ? launch_mt<3, 2>(st, a, cu_count) : launch_mt<2, 2>(st, a, cu_count);

@@ -185,7 +185,7 @@ void igemm_dma_cfg_shape(int cfg, int* bm, int* bn, int* kch);
 bool igemm_dma_cfg_is_pin4(int cfg);  // a 4-packed pointwise tile (NCHW4 in and out, 1x1, no padding)
 int launch_igemm_dma(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count);
 
-// streaming kernel for 4-packed pointwise layers with at most 64 input channels (conv_pw4.hip)
+// streaming kernel for 4-packed pointwise layers with few input or few output channels (conv_pw4.hip)
 bool pw4s_usable(const IgemmArgs& a);
 int launch_pw4s(hipStream_t st, const IgemmArgs& a, int cu_count);
 

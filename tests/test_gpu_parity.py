@@ -263,6 +263,8 @@ RAGGED = [
     ("NCHW4", 2, 160, 7, 7, 100, 1, 1, 0, "H_SWISH", True, {}),          # 4-packed pointwise, ragged everything
     ("NCHW4", 3, 32, 6, 6, 200, 1, 1, 0, "RELU", True, {"batch_pad": 64}),  # few channels in, 7 channel blocks out, strided views
     ("NCHW4", 5, 20, 7, 9, 36, 1, 1, 0, "IDENTITY", False, {}),          # few channels in: K = 20, oc = 36, 315 pixels
+    ("NCHW4", 3, 192, 6, 6, 32, 1, 1, 0, "RELU", True, {"batch_pad": 64}),  # narrow projection with residual, six k-steps, strided views
+    ("NCHW4", 2, 72, 7, 7, 20, 1, 1, 0, "H_SWISH", True, {}),            # narrow projection with residual, K = 72, oc = 20
 ]
 
 
