@@ -244,6 +244,13 @@ def test_heuristic_picks(oracle):
     assert ops.conv_bias_query(d)[0].id == DW
     d = _abi.make_conv_desc("NCHW32", 1, 64, 8, 8, 64, 3, pad=1, group=2)
     assert ops.conv_bias_query(d)[0].id == DIRECT
+    # 4-packed pointwise layers at batch 64: streaming kernel for the expansions and the narrow projections, LDS-direct
+    # tiles for the long reductions on few pixels, register-staged tiles elsewhere
+    names = lib.tile_names()
+    for (ic, hw, oc), want in (((16, 112, 96), "pw4_stream"), ((96, 56, 24), "pw4_stream"), ((384, 14, 64), "dma4_64x64x128"),
+                               ((160, 7, 960), "dma4_128x64x128"), ((96, 14, 576), "128x128x64")):
+        a, _ = ops.conv_bias_query(_abi.make_conv_desc("NCHW4", 64, ic, hw, hw, oc, 1))
+        assert a.id == IGEMM and names[a.tile_cfg] == want, (ic, hw, oc, names[a.tile_cfg])
 
 
 # ---------------------------------------------------------------------------------------------
