@@ -150,6 +150,7 @@ struct Dw3Args {
     int CG, IH, IW, OH, OW, QW, OHS;  // QW = pixel quads per output row, OHS = row strips per plane
     int ph, pw;
     uint32_t items;
+    uint32_t src_bytes;  // whole source tensor if it is addressable with 31-bit offsets, else 0
     int64_t src_sn, dst_sn, z_sn;
     int has_bias;
     FastDiv div_qw, div_ohs, div_cg;
@@ -254,7 +255,29 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(Dw3Args a) {
     // window columns: L = c0, block T = c0+1 .. c0+4, then (S = 1) Rt = c0+5 or (S = 2) block U = c0+5 .. c0+8
     uint32_t L[ROWS], Rt[ROWS], pt[ROWS][4], pu[ROWS][4];
     const bool interior = c0 + 1 >= 0 && c0 + (S == 1 ? 4 : 8) < a.IW;
-    if (interior) {
+    if (interior && a.src_bytes) {
+        // bounds-checked buffer loads with 32-bit offsets: a row outside the image, or a side column outside the row,
+        // becomes the out-of-range offset and reads zeros, so there is nothing to clamp and nothing to mask afterwards
+        constexpr int OOR = (int)0x80000000;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.src), 0, a.src_bytes, 0x00020000);
+        const bool lok = c0 >= 0, rtok = c0 + 5 < a.IW;
+        const int base = (int)(n * (uint32_t)a.src_sn) + ((int)cg * a.IH * a.IW + c0) * 4;
+#pragma unroll
+        for (int ir = 0; ir < ROWS; ++ir) {
+            const int ih = oh0 * S + ir - a.ph;
+            const bool rok = (unsigned)ih < (unsigned)a.IH;
+            const int ro = base + ih * a.IW * 4;
+            L[ir] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs, (rok && lok) ? ro : OOR, 0, 0);
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, rok ? ro + 4 : OOR, 0, 0);
+            pt[ir][0] = v[0]; pt[ir][1] = v[1]; pt[ir][2] = v[2]; pt[ir][3] = v[3];
+            if (S == 1) {
+                Rt[ir] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs, (rok && rtok) ? ro + 20 : OOR, 0, 0);
+            } else {
+                const u32x4 u = __builtin_amdgcn_raw_buffer_load_b128(rs, rok ? ro + 20 : OOR, 0, 0);
+                pu[ir][0] = u[0]; pu[ir][1] = u[1]; pu[ir][2] = u[2]; pu[ir][3] = u[3];
+            }
+        }
+    } else if (interior) {
         // every vector load is in range: rows are clamped and masked afterwards, so all loads of the thread are
         // independent of any branch and go out back to back
         const bool lok = c0 >= 0, rtok = c0 + 5 < a.IW;
@@ -393,6 +416,8 @@ int launch_conv_depthwise(hipStream_t st, const ConvProblem& p, const int8_t* sr
         const int64_t items = (int64_t)d.n * b.CG * b.OHS * b.QW;
         if (items < ((int64_t)1 << 31) - 256) {
             b.items = (uint32_t)items;
+            const int64_t src_total = (int64_t)(d.n - 1) * p.src_sn + (int64_t)d.ic * d.ih * d.iw;
+            b.src_bytes = src_total < ((int64_t)1 << 31) ? (uint32_t)src_total : 0u;
             b.div_qw = make_fastdiv(b.QW); b.div_ohs = make_fastdiv(b.OHS); b.div_cg = make_fastdiv(b.CG);
             dim3 grid((unsigned)((items + 255) / 256)), block(256);
             if (d.stride_h == 1 && R == 4)
