@@ -427,3 +427,26 @@ def test_linear_epilogue_form(oracle, i):
             want = check_case(oracle, d, seed=400 + i, tag="lin " + tag, src_range=(-amp, amp), flt_range=(-amp, amp),
                               bias_range=(-b, b))
             assert len(np.unique(want)) >= (100 if nl == "RELU" else 200), len(np.unique(want))
+
+
+def test_pointwise_4packed_random_descriptors(oracle):
+    """Seeded random 4-packed pointwise problems through the chooser (streaming kernel, LDS-direct and register-staged
+    tiles): ragged channel counts and pixel counts, stride 1 or 2, every activation, with and without residual."""
+    rng = np.random.RandomState(20261125)
+    names = lib.tile_names()
+    used = set()
+    for it in range(90):
+        n = int(rng.randint(1, 5)); ic = 4 * int(rng.randint(1, 60)); oc = 4 * int(rng.randint(1, 80))
+        ih = int(rng.randint(1, 20)); iw = int(rng.randint(1, 20)); st = int(rng.choice([1, 1, 2]))
+        nl = ("IDENTITY", "RELU", "H_SWISH")[int(rng.randint(3))]
+        z = bool(rng.randint(2))
+        sb = float(np.float32(np.exp(rng.uniform(np.log(1e-5), np.log(2e-3)))))
+        sd = float(np.float32(np.exp(rng.uniform(np.log(1e-3), np.log(5e-2)))))
+        if it % 3 == 0:   # enough pixels for the many-tile branches of the chooser
+            n *= 16; ih += 20; iw += 20
+        d = _abi.make_conv_desc("NCHW4", n, ic, ih, iw, oc, 1, stride=st, nonline=nl, has_z=z, scale_bias=sb, scale_z=0.03,
+                                scale_dst=sd)
+        a, _ = ops.conv_bias_query(d)
+        used.add(names[a.tile_cfg] if a.id == IGEMM else lib.algo_names()[a.id])
+        check_case(oracle, d, seed=1000 + it, tag="pw4 random %d" % it)
+    assert {"pw4_stream", "dma4_128x64x128", "dma4_64x64x128", "128x128x64"} <= used, used
