@@ -450,3 +450,24 @@ def test_pointwise_4packed_random_descriptors(oracle):
         used.add(names[a.tile_cfg] if a.id == IGEMM else lib.algo_names()[a.id])
         check_case(oracle, d, seed=1000 + it, tag="pw4 random %d" % it)
     assert {"pw4_stream", "dma4_128x64x128", "dma4_64x64x128", "128x128x64"} <= used, used
+
+
+def test_depthwise_random_descriptors(oracle):
+    """Seeded random channel-wise 3x3 problems (stride 1 or 2, any padding up to 2, ragged widths, batch-strided views):
+    interior threads load through the buffer descriptor, edge threads through pointers, both forms of the epilogue."""
+    rng = np.random.RandomState(7)
+    for it in range(40):
+        n = int(rng.randint(1, 4)); c = 4 * int(rng.randint(1, 12))
+        ih = int(rng.randint(3, 40)); iw = int(rng.randint(3, 40)); st = int(rng.choice([1, 2])); pad = int(rng.randint(0, 3))
+        nl = ("IDENTITY", "RELU", "H_SWISH")[int(rng.randint(3))]
+        z = bool(rng.randint(2))
+        sb, sd = ((1.3e-3, 0.0271) if it % 2 else (2e-4, 0.05))   # with / without a linear epilogue form
+        kw = dict(group=c, stride=st, pad=pad, nonline=nl, has_z=z, scale_bias=sb, scale_z=0.04, scale_dst=sd)
+        d0 = _abi.make_conv_desc("NCHW4", n, c, ih, iw, c, 3, **kw)
+        if it % 4 == 0:
+            ss, fs, bs, ds = _abi.conv_shapes(d0)
+            kw.update(src_stride_n=int(np.prod(ss[1:])) + 48, dst_stride_n=int(np.prod(ds[1:])) + 16,
+                      z_stride_n=int(np.prod(ds[1:])) + 32)
+        d = _abi.make_conv_desc("NCHW4", n, c, ih, iw, c, 3, **kw)
+        assert ops.conv_bias_query(d)[0].id == DW
+        check_case(oracle, d, seed=2000 + it, tag="dw random %d" % it)
