@@ -255,12 +255,15 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(Dw3Args a) {
     // window columns: L = c0, block T = c0+1 .. c0+4, then (S = 1) Rt = c0+5 or (S = 2) block U = c0+5 .. c0+8
     uint32_t L[ROWS], Rt[ROWS], pt[ROWS][4], pu[ROWS][4];
     const bool interior = c0 + 1 >= 0 && c0 + (S == 1 ? 4 : 8) < a.IW;
-    if (interior && a.src_bytes) {
-        // bounds-checked buffer loads with 32-bit offsets: a row outside the image, or a side column outside the row,
-        // becomes the out-of-range offset and reads zeros, so there is nothing to clamp and nothing to mask afterwards
+    if (a.src_bytes && a.pw <= 1) {
+        // Bounds-checked buffer loads with 32-bit offsets, the same straight-line code for every thread.  A row outside
+        // the image, or a side column outside the row, becomes the out-of-range offset and reads zeros: nothing to
+        // clamp.  The 4-pixel blocks always start inside the row (pw <= 1); where one runs past the end of the row
+        // its surplus pixels (the next row's, or zeros past the tensor) are masked -- only in wavefronts that hold such
+        // a thread, so whole rows of interior threads carry no masks at all.
         constexpr int OOR = (int)0x80000000;
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.src), 0, a.src_bytes, 0x00020000);
-        const bool lok = c0 >= 0, rtok = c0 + 5 < a.IW;
+        const bool lok = (unsigned)c0 < (unsigned)a.IW, rtok = (unsigned)(c0 + 5) < (unsigned)a.IW;
         const int base = (int)(n * (uint32_t)a.src_sn) + ((int)cg * a.IH * a.IW + c0) * 4;
 #pragma unroll
         for (int ir = 0; ir < ROWS; ++ir) {
@@ -275,6 +278,17 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(Dw3Args a) {
             } else {
                 const u32x4 u = __builtin_amdgcn_raw_buffer_load_b128(rs, rok ? ro + 20 : OOR, 0, 0);
                 pu[ir][0] = u[0]; pu[ir][1] = u[1]; pu[ir][2] = u[2]; pu[ir][3] = u[3];
+            }
+        }
+        if (__builtin_amdgcn_ballot_w64(!interior) != 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool tok = (unsigned)(c0 + 1 + i) < (unsigned)a.IW, uok = (unsigned)(c0 + 5 + i) < (unsigned)a.IW;
+#pragma unroll
+                for (int ir = 0; ir < ROWS; ++ir) {
+                    pt[ir][i] = tok ? pt[ir][i] : 0u;
+                    if (S == 2) pu[ir][i] = uok ? pu[ir][i] : 0u;
+                }
             }
         }
     } else if (interior) {
