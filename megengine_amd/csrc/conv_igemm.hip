@@ -474,16 +474,20 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
 
 }  // namespace
 
-// tile_cfg numbering: the register-staged tiles first, then the LDS-direct ones
-int igemm_num_cfgs() { return kNumCfgs + igemm_dma_num_cfgs(); }
+// tile_cfg numbering: register-staged tiles, LDS-direct tiles, second-generation tiles
+int igemm_num_cfgs() { return kNumCfgs + igemm_dma_num_cfgs() + igemm2_num_cfgs(); }
 const char* igemm_cfg_name(int cfg) {
     if (cfg >= 0 && cfg < kNumCfgs) return kCfgs[cfg].name;
-    return igemm_dma_cfg_name(cfg - kNumCfgs);
+    if (cfg < kNumCfgs + igemm_dma_num_cfgs()) return igemm_dma_cfg_name(cfg - kNumCfgs);
+    return igemm2_cfg_name(cfg - kNumCfgs - igemm_dma_num_cfgs());
 }
+int igemm_first_v2_cfg() { return kNumCfgs + igemm_dma_num_cfgs(); }
 
 bool igemm_usable(const ConvProblem& p) {
     const mi355_conv_desc& d = p.d;
-    if (d.group != 1 || p.dw4) return false;
+    if (p.dw4) return false;
+    // group convolution: 32-packed tensors whose groups are whole channel blocks (second-generation tiles only)
+    if (d.group != 1 && !(p.pin == 32 && p.icpg % 32 == 0 && p.ocpg % 32 == 0)) return false;
     if (d.format != MI355_FMT_NCHW4 && d.format != MI355_FMT_NCHW32 && d.format != MI355_FMT_NCHW4_NCHW32 &&
         d.format != MI355_FMT_NCHW32_NCHW4)
         return false;
@@ -496,10 +500,10 @@ bool igemm_usable(const ConvProblem& p) {
     const int64_t src_b = (int64_t)(d.n - 1) * p.src_sn + (int64_t)d.ic * d.ih * d.iw;
     const int64_t dst_b = (int64_t)(d.n - 1) * p.dst_sn + (int64_t)d.oc * p.oh * p.ow;
     const int64_t z_b = d.has_z ? (int64_t)(d.n - 1) * p.z_sn + (int64_t)d.oc * p.oh * p.ow : 0;
-    const int64_t flt_b = (int64_t)d.oc * d.ic * d.fh * d.fw;
+    const int64_t flt_b = (int64_t)d.oc * p.icpg * d.fh * d.fw;
     if (src_b >= lim || dst_b >= lim || z_b >= lim || flt_b >= lim) return false;
     if ((int64_t)d.n * p.oh * p.ow >= lim) return false;
-    const int64_t entries = p.pin == 32 ? (int64_t)(d.ic / 32) * d.fh * d.fw : (int64_t)(d.ic / 4) * d.fh * d.fw;
+    const int64_t entries = p.pin == 32 ? (int64_t)(p.icpg / 32) * d.fh * d.fw : (int64_t)(p.icpg / 4) * d.fh * d.fw;
     // table capacity incl. the padding entries of the last stage (<= 8 chunks of 8 units)
     if (entries + 64 > IG_MAX_ENTRIES) return false;
     return true;
@@ -510,6 +514,8 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
     const int64_t M = (int64_t)d.n * p.oh * p.ow;
     const int OC = d.oc;
     if (cu_count <= 0) cu_count = 256;
+    // group convolution: second-generation tiles only; a channel tile never spans two groups
+    if (d.group != 1) return igemm_first_v2_cfg() + (p.ocpg <= 64 ? 3 : 0);
     auto tiles = [&](int cfg) { return ((OC + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm) * ((M + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn); };
     const int kbytes = d.ic * d.fh * d.fw;
     if (p.pin == 4 && p.pout == 4 && d.fh == 1 && d.fw == 1 && d.pad_h == 0 && d.pad_w == 0) {
@@ -573,16 +579,16 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
     a.sh = d.stride_h; a.sw = d.stride_w; a.ph = d.pad_h; a.pw = d.pad_w;
     a.OC = d.oc;
     a.M = d.n * p.oh * p.ow;
-    a.kbytes = d.ic * d.fh * d.fw;
+    a.kbytes = p.icpg * d.fh * d.fw;
     a.KC = (a.kbytes + 31) / 32;
-    a.entries = p.pin == 32 ? a.KC : (d.ic / 4) * a.T;
+    a.entries = p.pin == 32 ? a.KC : (p.icpg / 4) * a.T;
     a.src_sn = (int)p.src_sn;
     a.src_scb = d.ih * d.iw * p.pin;
     a.dst_sn = (int)p.dst_sn;
     a.dst_scb = p.oh * p.ow * p.pout;
     a.z_sn = (int)p.z_sn;
     a.src_bytes = (uint32_t)((int64_t)(d.n - 1) * p.src_sn + (int64_t)d.ic * d.ih * d.iw);
-    a.flt_bytes = (uint32_t)((int64_t)d.oc * a.kbytes);
+    a.flt_bytes = (uint32_t)((int64_t)d.oc * a.kbytes);  // (groups x ocpg) rows of icpg * fh * fw bytes
     a.dst_bytes = (uint32_t)((int64_t)(d.n - 1) * p.dst_sn + (int64_t)d.oc * a.OHW);
     a.z_bytes = d.has_z ? (uint32_t)((int64_t)(d.n - 1) * p.z_sn + (int64_t)d.oc * a.OHW) : 0;
     a.has_bias = d.bias_mode == MI355_BIAS_BROADCAST_CHANNEL;
@@ -591,7 +597,24 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
     a.div_t = make_fastdiv(a.T);
     a.div_fw = make_fastdiv(a.FW);
     a.epi = p.epi;
+    a.flt_rstride = a.kbytes;
+    a.flt_kstride = 32;
+    a.groups = d.group;
+    a.ocpg = p.ocpg;
+    a.src_sg = (p.icpg / p.pin) * a.src_scb;
     if (a.M == 0 || a.OC == 0) return 0;
+    const int first_v2 = igemm_first_v2_cfg();
+    // group convolutions exist on the second-generation tiles only
+    if (d.group != 1 && cfg < first_v2) cfg = first_v2;
+    if (cfg >= first_v2) {
+        if (p.pin == 32) return launch_igemm2(st, a, p.pout, cfg - first_v2, cu_count);
+        // 4-packed inputs: the register-staged tile of the same shape
+        int bm, bn, kch;
+        igemm2_cfg_shape(cfg - first_v2, &bm, &bn, &kch);
+        cfg = 0;
+        for (int i = 0; i < kNumCfgs; ++i)
+            if (kCfgs[i].bm == bm && kCfgs[i].bn == bn && kCfgs[i].kch == kch) cfg = i;
+    }
     if (cfg >= kNumCfgs) {
         const int dcfg = cfg - kNumCfgs;
         if (dcfg >= igemm_dma_num_cfgs()) return (int)hipErrorInvalidValue;

@@ -24,59 +24,10 @@
 #include <atomic>
 
 #include "igemm_shared.h"
+#include "lds_copy.h"
 
 namespace mi355 {
 namespace {
-
-__device__ __forceinline__ void lds_copy64x16(uint32_t lds_addr, int voff, const v4i& rsrc) {
-    // M0 needs one wait state before an LDS-direct load reads it
-    asm volatile(
-        "s_mov_b32 m0, %0\n\t"
-        "s_nop 0\n\t"
-        "buffer_load_dwordx4 %1, %2, 0 offen lds"
-        :
-        : "s"(lds_addr), "v"(voff), "s"(rsrc)
-        : "memory");  // M0 is reserved by the compiler (never allocated), so it needs no clobber entry
-}
-
-// 64 x 4 bytes: lane l lands at M0 + 4 * l (4-packed activations: one pixel's channel block per lane)
-__device__ __forceinline__ void lds_copy64x4(uint32_t lds_addr, int voff, const v4i& rsrc) {
-    asm volatile(
-        "s_mov_b32 m0, %0\n\t"
-        "s_nop 0\n\t"
-        "buffer_load_dword %1, %2, 0 offen lds"
-        :
-        : "s"(lds_addr), "v"(voff), "s"(rsrc)
-        : "memory");
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    static_assert(N >= 0 && N < 64, "vmcnt range");
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-// a dword load the compiler does not wait for: the value is valid only after wait_vmcnt_for on it
-__device__ __forceinline__ int load_dword_async(int voff, const v4i& rsrc) {
-    int v;
-    asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=v"(v) : "v"(voff), "s"(rsrc) : "memory");
-    return v;
-}
-template <int N>
-__device__ __forceinline__ void wait_vmcnt_for(int& v) {
-    static_assert(N >= 0 && N < 64, "vmcnt range");
-    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N) : "memory");
-}
-
-__device__ __forceinline__ v4i uniform_rsrc(const void* p, uint32_t bytes) {
-    const uint64_t a = (uint64_t)(uintptr_t)p;
-    v4i r;
-    r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
-    r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32));
-    r[2] = __builtin_amdgcn_readfirstlane((int)bytes);
-    r[3] = 0x00020000;
-    return r;
-}
 
 // PIN = 4 (4-packed activations, pointwise only): a pixel's 4 channels are the only contiguous bytes, so the
 // activation tile travels as 64 x 4-byte copies -- lane = pixel, one channel block per copy -- and sits in LDS as

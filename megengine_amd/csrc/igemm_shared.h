@@ -34,6 +34,13 @@ struct IgemmArgs {
     int has_bias;
     FastDiv div_ohw, div_ow, div_t, div_fw;
     EpiParams epi;
+    // filter addressing of the second-generation kernel (conv_igemm2.hip): byte offset of 16-byte half h of k-chunk kc of
+    // output channel oc = oc * flt_rstride + kc * flt_kstride + 16 h.  The reference layout has (kbytes, 32); the
+    // pre-processed layout [k-chunk][channel][32 bytes] has (32, 32 * padded channel count)
+    int flt_rstride, flt_kstride;
+    // group convolution: ocpg output channels per group, src_sg bytes between the channel blocks of two groups
+    int groups, ocpg, src_sg, tiles_m_pg;
+    int zslots;  // residual slots in LDS: 0 (no residual), 1 or 2
 };
 
 struct KEntry {
@@ -102,7 +109,7 @@ __device__ __forceinline__ void igemm_load_z(const IgemmArgs& a, ZRegs<MT, NT>& 
 // ZPRE: the residual was fetched by igemm_load_z into *zr; otherwise it is loaded here, block by block
 template <int POUT, int MT, int NT, int NL, bool HZ, bool ZPRE>
 __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], const ZRegs<MT, NT>* zr, int oc_w,
-                                               int pix_w, int l32, int lh) {
+                                               int pix_w, int l32, int lh, int oc_end) {
     const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(a.z, HZ ? a.z_bytes : 0);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
@@ -115,7 +122,7 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const int ocb = oc_w + i * 32;  // first channel of this 32-channel block
-            if (ocb >= a.OC) continue;      // wave-uniform
+            if (ocb >= oc_end) continue;    // wave-uniform
             const v16i& c = acc[i][j];
             if (POUT == 32) {
                 const int blk_off = (ocb >> 5) * a.dst_scb + lh * 16;
@@ -144,7 +151,7 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const int oc4 = ocb + 8 * q + 4 * lh;  // first of 4 channels; oc is a multiple of 4
-                    const bool ok = pok && oc4 < a.OC;
+                    const bool ok = pok && oc4 < oc_end;
                     const int off = (oc4 >> 2) * a.dst_scb;
                     uint32_t zw = 0;
                     if (HZ) zw = ZPRE ? (uint32_t)zr->v[i][j][q]
@@ -158,22 +165,25 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
 }
 
 // Fused requantisation + store of one wave tile (MT x NT blocks of 32 channels x 32 pixels).
+// oc_end: one past the last output channel this tile may write (the layer's channel count, or the end of the tile's
+// group); negative = the layer's channel count.
 template <int POUT, int MT, int NT, bool ZPRE = false>
 __device__ __forceinline__ void igemm_run_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w, int l32,
-                                                   int lh, const ZRegs<MT, NT>* zr = nullptr) {
+                                                   int lh, const ZRegs<MT, NT>* zr = nullptr, int oc_end = -1) {
+    if (oc_end < 0) oc_end = a.OC;
     if (a.epi.lin) {
-        igemm_epilogue<POUT, MT, NT, NL_LIN, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh);
+        igemm_epilogue<POUT, MT, NT, NL_LIN, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end);
     } else if (a.epi.has_z) {
         switch (a.epi.nonline) {
-            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
-            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
-            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
+            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
+            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
+            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
         }
     } else {
         switch (a.epi.nonline) {
-            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
-            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
-            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh); break;
+            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
+            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
+            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
         }
     }
 }
@@ -184,6 +194,14 @@ const char* igemm_dma_cfg_name(int cfg);
 void igemm_dma_cfg_shape(int cfg, int* bm, int* bn, int* kch);
 bool igemm_dma_cfg_is_pin4(int cfg);  // a 4-packed pointwise tile (NCHW4 in and out, 1x1, no padding)
 int launch_igemm_dma(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count);
+
+// second-generation kernel for 32-packed inputs (conv_igemm2.hip): chunk-major LDS stages, software-pipelined k-loop,
+// optional pre-processed filter, group convolution
+int igemm2_num_cfgs();
+const char* igemm2_cfg_name(int cfg);
+void igemm2_cfg_shape(int cfg, int* bm, int* bn, int* kch);
+int launch_igemm2(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count);
+int igemm_first_v2_cfg();  // tile_cfg of the first second-generation tile
 
 // streaming kernel for 4-packed pointwise layers with few input or few output channels (conv_pw4.hip)
 bool pw4s_usable(const IgemmArgs& a);

@@ -242,7 +242,12 @@ def test_heuristic_picks(oracle):
     assert ops.conv_bias_query(d)[0].id == DIRECT
     d = _abi.make_conv_desc("NCHW4", 1, 32, 8, 8, 32, 3, pad=1, group=32)
     assert ops.conv_bias_query(d)[0].id == DW
+    # group convolution over whole 32-channel blocks runs on the MFMA kernel (second-generation tiles); groups that
+    # split a channel block stay on the generic kernel
     d = _abi.make_conv_desc("NCHW32", 1, 64, 8, 8, 64, 3, pad=1, group=2)
+    a = ops.conv_bias_query(d)[0]
+    assert a.id == IGEMM and lib.tile_names()[a.tile_cfg].startswith("v2_")
+    d = _abi.make_conv_desc("NCHW4", 1, 32, 8, 8, 32, 3, pad=1, group=4)
     assert ops.conv_bias_query(d)[0].id == DIRECT
     # 4-packed pointwise layers at batch 64: streaming kernel for the expansions and the narrow projections, LDS-direct
     # tiles for the long reductions on few pixels, register-staged tiles elsewhere
