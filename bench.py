@@ -31,53 +31,6 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def build_stack(layers, seed, torch, np, util, _abi):
-    """Allocates every tensor of a layer list on the GPU and returns launch closures."""
-    rng = np.random.RandomState(seed)
-
-    def scale():
-        return float(np.float32(np.exp(rng.uniform(np.log(1e-3), np.log(5e-2)))))
-
-    def rand_i8(shape, lo=-128, hi=127):
-        return torch.randint(lo, hi + 1, shape, dtype=torch.int8, device="cuda")
-
-    outs, out_scale, inputs = {}, {}, {}
-    plan = []
-    prev = None
-    for i, L in enumerate(layers):
-        d0 = L.desc(1.0, 1.0, 1.0)
-        src_s, flt_s, bias_s, dst_s = _abi.conv_shapes(d0)
-        # source tensor
-        sname = L.src if L.src is not None else prev
-        if sname is None or sname.startswith("input:") or sname not in outs or tuple(outs[sname].shape) != tuple(src_s):
-            key = "in:%s:%s" % (sname, src_s)
-            if key not in inputs:
-                inputs[key] = (rand_i8(src_s), scale())
-            src, s_src = inputs[key]
-        else:
-            src, s_src = outs[sname], out_scale[sname]
-        s_flt = scale()
-        s_bias = float(np.float32(s_src) * np.float32(s_flt))
-        s_dst = scale()
-        flt = rand_i8(flt_s, -127, 127)
-        bias = torch.randint(-1000, 1001, bias_s, dtype=torch.int32, device="cuda")
-        z, s_z = None, 1.0
-        if L.z is not None:
-            if L.z in outs and tuple(outs[L.z].shape) == tuple(dst_s):
-                z, s_z = outs[L.z], out_scale[L.z]
-            else:
-                key = "z:%s:%s" % (L.z, dst_s)
-                if key not in inputs:
-                    inputs[key] = (rand_i8(dst_s), scale())
-                z, s_z = inputs[key]
-        dst = torch.empty(dst_s, dtype=torch.int8, device="cuda")
-        desc = L.desc(s_bias, s_z, s_dst)
-        outs[L.name], out_scale[L.name] = dst, s_dst
-        prev = L.name
-        plan.append(dict(layer=L, desc=desc, src=src, flt=flt, bias=bias, z=z, dst=dst))
-    return plan
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -99,7 +52,6 @@ def main():
     import torch
 
     from megengine_amd import _abi, lib, ops, workloads
-    from tests import util
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -111,7 +63,7 @@ def main():
     torch.manual_seed(1234)
     batch = 64
     layers = workloads.resnet50(batch)
-    plan = build_stack(layers, 7, torch, np, util, _abi)
+    plan = workloads.build_stack(layers, 7)
     for p in plan:
         p["algo"], _ = ops.conv_bias_query(p["desc"])
     side = torch.cuda.Stream()          # default priority; every launch of the bench goes here
@@ -242,13 +194,13 @@ def main():
     extras = {}
     if not args.no_extras:
         try:
-            extras = run_extras(torch, np, util, _abi, lib, ops, workloads)
+            extras = run_extras(torch, np, _abi, lib, ops, workloads)
         except Exception as e:  # side measurements must not lose the headline
             extras = dict(error=repr(e))
         out["other_configs"] = extras
 
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(np, util, _abi, workloads)
+        out["cpu_baseline"] = cpu_baseline(np, plan)
 
     if args.layers_out:
         with open(args.layers_out, "w") as f:
@@ -310,12 +262,12 @@ def time_launches(torch, fn, iters=20, warm=3):
     return e0.elapsed_time(e1) / iters * 1e-3
 
 
-def run_extras(torch, np, util, _abi, lib, ops, workloads):
+def run_extras(torch, np, _abi, lib, ops, workloads):
     """Side measurements for the other workload configurations (not the headline value)."""
     res = {}
 
     def measure(layers, seed):
-        plan = build_stack(layers, seed, torch, np, util, _abi)
+        plan = workloads.build_stack(layers, seed)
         rows = []
         for p in plan:
             p["algo"], _ = ops.conv_bias_query(p["desc"])
@@ -375,39 +327,47 @@ def run_extras(torch, np, util, _abi, lib, ops, workloads):
     return res
 
 
-def cpu_baseline(np, util, _abi, workloads):
-    """The CPU parity checker (a port of the reference's naive ConvBias, OpenMP over output rows)
-    on a bounded sample of the same workload: the same 53 layers at a batch chosen so that the
-    whole leg is 10-30 s of CPU work on this host, scaled to images per second."""
+def cpu_baseline(np, plan):
+    """The CPU parity checker (a port of the reference's naive ConvBias, OpenMP over output rows) on a bounded sample
+    of the SAME workload: the first b images of the very tensors the GPU plan ran on (same weights, biases, residuals
+    and scales, layer by layer), b chosen so that the whole leg is 10-30 s of CPU work on this host; scaled to images
+    per second.  Its outputs are compared with the first b images of the GPU's outputs."""
+    import copy
+
     from oracle import oracle
     oracle.lib()
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     os.environ["OMP_NUM_THREADS"] = str(cores)
+    total_macs = sum(p["layer"].ops // 2 for p in plan) / plan[0]["layer"].n  # per image
 
     def run(batch, budget):
-        t_tot, macs, done = 0.0, 0, 0
-        layers = workloads.resnet50(batch)
-        for i, l in enumerate(layers):
-            d = l.desc(2e-4, 0.05, 0.05)
-            src, flt, bias, z = util.make_tensors(d, seed=i + 1, flt_range=(-127, 127))
+        t_tot, macs, done, bad = 0.0, 0, 0, 0
+        for p in plan:
+            d = copy.copy(p["desc"])
+            d.n = batch
+            host = [None if t is None else t[:batch].cpu().numpy() for t in (p["src"], p["z"])]
+            flt, bias = p["flt"].cpu().numpy(), p["bias"].cpu().numpy()
             t0 = time.perf_counter()
-            oracle.conv_bias(d, src, flt, bias, z)
+            out = oracle.conv_bias(d, host[0], flt, bias, host[1])
             t_tot += time.perf_counter() - t0
-            macs += l.ops // 2
+            bad += int((out != p["dst"][:batch].cpu().numpy()).sum())
+            macs += p["layer"].ops // 2 // p["layer"].n * batch
             done += 1
             if t_tot > budget:
                 break
-        return t_tot, macs, done, sum(l.ops // 2 for l in layers)
+        return t_tot, macs, done, bad
 
-    t1, m1, _, tm1 = run(1, 10.0)                 # probe: one image
-    est = t1 * tm1 / max(m1, 1)
-    batch = int(max(1, min(64, round(15.0 / max(est, 1e-3)))))
-    t_tot, macs, done, total_macs = run(batch, 30.0)
-    img_s = batch * (macs / total_macs) / t_tot if t_tot > 0 else 0.0
+    t1, m1, _, _ = run(1, 10.0)                 # probe: one image
+    est = t1 * total_macs / max(m1, 1)
+    batch = int(max(1, min(plan[0]["layer"].n, round(15.0 / max(est, 1e-3)))))
+    t_tot, macs, done, bad = run(batch, 30.0)
+    img_s = (macs / total_macs) / t_tot if t_tot > 0 else 0.0
     return dict(value=round(img_s, 3), unit="img/s", cores=cores, kind="port",
-                sample="batch %d through the first %d of 53 layers (%.1f of %.1f GMAC) in %.1f s on %d threads, "
-                       "scaled by MACs" % (batch, done, macs / 1e9, total_macs / 1e9, t_tot, cores))
+                sample="the first %d images of the GPU plan's own tensors and scales through the first %d of %d layers "
+                       "(%.1f GMAC of %.1f per image x %d) in %.1f s on %d threads, scaled by MACs" % (
+                           batch, done, len(plan), macs / 1e9, total_macs / 1e9, batch, t_tot, cores),
+                outputs_differing_from_gpu=bad)
 
 
 if __name__ == "__main__":

@@ -132,6 +132,10 @@ typedef struct mi355_algo {
 } mi355_algo;
 
 #define MI355_ALGO_HEURISTIC (-1)
+/* bit of mi355_algo.reserved, set by query() when the heuristic chose the algorithm: exec() may then replace it by
+ * the generic kernel when a tensor is not aligned for the tiled kernels (the reference accepts any pointer); an
+ * algorithm requested by id is never replaced, exec() reports MI355_ERR_ALGO instead. */
+#define MI355_ALGO_FLAG_HEURISTIC 1ull
 
 /* ---- library / device ---- */
 int mi355_abi_version(void);

@@ -216,10 +216,14 @@ int canonize(const mi355_conv_desc* d, ConvProblem* p) {
         return fail(MI355_ERR_UNSUPPORTED, "a Float32 dst needs format NCHW4_NCHW");
     if (d->has_z && (d->format == MI355_FMT_NCHW4_NCHW32 || d->format == MI355_FMT_NCHW32_NCHW4))
         return fail(MI355_ERR_SHAPE, "z is not allowed for NCHW4_NCHW32 / NCHW32_NCHW4");
-    const uint32_t dfh = (d->fh - 1) * d->dilate_h + 1, dfw = (d->fw - 1) * d->dilate_w + 1;
-    if (d->ih + 2 * d->pad_h < dfh || d->iw + 2 * d->pad_w < dfw)
-        return fail(MI355_ERR_SHAPE, "filter %ux%u larger than padded input %ux%u", dfh, dfw, d->ih + 2 * d->pad_h,
-                    d->iw + 2 * d->pad_w);
+    // 64-bit: huge paddings or dilations must not wrap past the test
+    const uint64_t dfh = (uint64_t)(d->fh - 1) * d->dilate_h + 1, dfw = (uint64_t)(d->fw - 1) * d->dilate_w + 1;
+    const uint64_t pih = (uint64_t)d->ih + 2ull * d->pad_h, piw = (uint64_t)d->iw + 2ull * d->pad_w;
+    if (pih < dfh || piw < dfw)
+        return fail(MI355_ERR_SHAPE, "filter %llux%llu larger than padded input %llux%llu", (unsigned long long)dfh,
+                    (unsigned long long)dfw, (unsigned long long)pih, (unsigned long long)piw);
+    if (dfh > 0x7fffffffull || dfw > 0x7fffffffull || pih > 0x7fffffffull || piw > 0x7fffffffull)
+        return fail(MI355_ERR_SHAPE, "convolution geometry out of range");
     p->oh = conv_out_size(d->ih, d->fh, d->dilate_h, d->stride_h, d->pad_h);
     p->ow = conv_out_size(d->iw, d->fw, d->dilate_w, d->stride_w, d->pad_w);
     const int64_t src_img = (int64_t)d->ic * d->ih * d->iw, dst_img = (int64_t)d->oc * p->oh * p->ow;
@@ -359,7 +363,9 @@ int mi355_convbias_s8_query(const mi355_conv_desc* d, int algo_request, mi355_al
     if (algo_out) {
         algo_out->id = id;
         algo_out->tile_cfg = id == ALGO_IGEMM_MFMA ? igemm_pick_cfg(p, cu_count()) : 0;
-        algo_out->reserved = 0;
+        // an algorithm the heuristic chose may be replaced by the generic kernel at exec time (misaligned tensors);
+        // one the caller asked for by id may not
+        algo_out->reserved = algo_request == MI355_ALGO_HEURISTIC ? MI355_ALGO_FLAG_HEURISTIC : 0;
     }
     // every kernel reads the reference layouts in place: no filter repack, no float staging
     if (workspace_bytes) *workspace_bytes = 0;
@@ -392,7 +398,7 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
         bool al = aligned16(src) && aligned16(filter) && aligned16(dst) && (!bias || aligned16(bias)) &&
                   (!z || aligned16(z)) && p.src_sn % sa == 0 && p.dst_sn % da == 0 && p.z_sn % da == 0;
         if (!al) {
-            if (algo && algo->id != MI355_ALGO_HEURISTIC)
+            if (algo && algo->id != MI355_ALGO_HEURISTIC && !(algo->reserved & MI355_ALGO_FLAG_HEURISTIC))
                 return fail(MI355_ERR_ALGO, "%s needs 16-byte aligned tensors", kAlgoNames[id]);
             id = ALGO_DIRECT;
         }

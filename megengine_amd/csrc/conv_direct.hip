@@ -118,8 +118,15 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(DirectArgs a) {
         acc += a.bias[idx];
     const bool hz = a.epi.has_z != 0;
     if (a.dst_s32) {
-        int zv = hz ? reinterpret_cast<const int*>(a.z)[(int64_t)n * a.z_sn + r] : 0;
-        reinterpret_cast<int*>(a.dst)[(int64_t)n * a.dst_sn + r] = requant_s32_exact(acc, hz, zv, a.epi);
+        // The reference accumulates a QuantizedS32 result in dst itself (naive/conv_bias/opr_impl.cpp:223-228): IDENTITY
+        // without z leaves the raw sum there (:52,:89-93), every other case dequantises it with the scale of dst
+        // (a.epi.s_b holds that scale here, see launch_conv_direct)
+        int out = acc;
+        if (hz || a.epi.nonline != NL_IDENTITY) {
+            int zv = hz ? reinterpret_cast<const int*>(a.z)[(int64_t)n * a.z_sn + r] : 0;
+            out = requant_s32_exact(acc, hz, zv, a.epi);
+        }
+        reinterpret_cast<int*>(a.dst)[(int64_t)n * a.dst_sn + r] = out;
     } else {
         int zv = hz ? (int)reinterpret_cast<const int8_t*>(a.z)[(int64_t)n * a.z_sn + r] : 0;
         int out;
@@ -166,6 +173,7 @@ int launch_conv_direct(hipStream_t st, const ConvProblem& p, const int8_t* src, 
     a.dst_f32 = d.dst_dtype == MI355_DT_F32;
     a.src_sn = p.src_sn; a.dst_sn = p.dst_sn; a.z_sn = p.z_sn;
     a.epi = p.epi;
+    if (a.dst_s32) a.epi.s_b = a.epi.s_d;  // the sum lives in dst and is dequantised with the dtype of dst
     const int64_t total = (int64_t)d.n * d.oc * p.oh * p.ow;
     if (total == 0) return 0;
     const int64_t blocks = (total + 255) / 256;

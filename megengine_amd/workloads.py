@@ -102,3 +102,55 @@ def large_hswish(batch=128):
 
 def config0():
     return Layer("cfg0", "NCHW4", 16, 64, 56, 56, 64, 3, pad=1, nonline="RELU")
+
+
+def build_stack(layers, seed):
+    """Allocates every tensor of a layer list on the GPU (seeded random weights and inputs, per-tensor scales drawn
+    log-uniform in [1e-3, 5e-2], bias scale = source scale x filter scale, residuals and sources wired to the real
+    producer outputs) and returns one dict per layer: layer, desc, src, flt, bias, z, dst."""
+    import numpy as np
+    import torch
+
+    rng = np.random.RandomState(seed)
+
+    def scale():
+        return float(np.float32(np.exp(rng.uniform(np.log(1e-3), np.log(5e-2)))))
+
+    def rand_i8(shape, lo=-128, hi=127):
+        return torch.randint(lo, hi + 1, shape, dtype=torch.int8, device="cuda")
+
+    outs, out_scale, inputs = {}, {}, {}
+    plan = []
+    prev = None
+    for i, L in enumerate(layers):
+        d0 = L.desc(1.0, 1.0, 1.0)
+        src_s, flt_s, bias_s, dst_s = _abi.conv_shapes(d0)
+        # source tensor
+        sname = L.src if L.src is not None else prev
+        if sname is None or sname.startswith("input:") or sname not in outs or tuple(outs[sname].shape) != tuple(src_s):
+            key = "in:%s:%s" % (sname, src_s)
+            if key not in inputs:
+                inputs[key] = (rand_i8(src_s), scale())
+            src, s_src = inputs[key]
+        else:
+            src, s_src = outs[sname], out_scale[sname]
+        s_flt = scale()
+        s_bias = float(np.float32(s_src) * np.float32(s_flt))
+        s_dst = scale()
+        flt = rand_i8(flt_s, -127, 127)
+        bias = torch.randint(-1000, 1001, bias_s, dtype=torch.int32, device="cuda")
+        z, s_z = None, 1.0
+        if L.z is not None:
+            if L.z in outs and tuple(outs[L.z].shape) == tuple(dst_s):
+                z, s_z = outs[L.z], out_scale[L.z]
+            else:
+                key = "z:%s:%s" % (L.z, dst_s)
+                if key not in inputs:
+                    inputs[key] = (rand_i8(dst_s), scale())
+                z, s_z = inputs[key]
+        dst = torch.empty(dst_s, dtype=torch.int8, device="cuda")
+        desc = L.desc(s_bias, s_z, s_dst)
+        outs[L.name], out_scale[L.name] = dst, s_dst
+        prev = L.name
+        plan.append(dict(layer=L, desc=desc, src=src, flt=flt, bias=bias, z=z, dst=dst))
+    return plan

@@ -466,9 +466,19 @@ int oracle_convbias_s8(const mi355_conv_desc* d, const int8_t* src, const int8_t
                 ((int8_t*)dst)[n * dsn + i] =
                         oracle_epilogue_s8(v, d->scale_bias, d->has_z, zv, d->scale_z, d->nonline, d->scale_dst);
             } else {
-                int32_t zv = d->has_z ? ((const int32_t*)z)[n * zsn + i] : 0;
-                ((int32_t*)dst)[n * dsn + i] =
-                        oracle_epilogue_s32(v, d->scale_bias, d->has_z, zv, d->scale_z, d->nonline, d->scale_dst);
+                /* QuantizedS32 dst: bias and dst have the same dtype enum, so the reference accumulates straight into
+                 * dst (sfb = dst, naive/conv_bias/opr_impl.cpp:223-228).  IDENTITY without z then leaves the raw sum
+                 * where it is (res.raw_ptr() == dst.raw_ptr(), :52,:89-93): no float round trip, the scales are not
+                 * used.  Every other case dequantises that tensor with ITS dtype, i.e. with the scale of dst (:44-46 TypeCvt
+                 * of conv_bias_tensor = dst; :69-73 ElemwiseMultiType reads param0 from the dtype of res = dst,
+                 * naive/elemwise_multi_type/opr_impl.h:54-60), never with the scale of the bias tensor. */
+                if (d->nonline == MI355_NL_IDENTITY && !d->has_z) {
+                    ((int32_t*)dst)[n * dsn + i] = v;
+                } else {
+                    int32_t zv = d->has_z ? ((const int32_t*)z)[n * zsn + i] : 0;
+                    ((int32_t*)dst)[n * dsn + i] =
+                            oracle_epilogue_s32(v, d->scale_dst, d->has_z, zv, d->scale_z, d->nonline, d->scale_dst);
+                }
             }
         }
     free(sfb);

@@ -103,6 +103,58 @@ def test_direct_s32_dst_and_full_bias(oracle, kats):
                                            scale_bias=2e-4, scale_dst=2e-4), algo=DIRECT)
 
 
+def test_s32_dst_in_place_semantics(oracle):
+    """QuantizedS32 dst: raw sums for IDENTITY without z (also beyond 2^24, also with a dst scale that differs from
+    the bias scale), the scale of dst everywhere else."""
+    src = np.array([1, 2, 3, 5], np.int8).reshape(1, 1, 2, 2)
+    flt = np.ones((1, 1, 1, 1), np.int8)
+    bias = np.array([3 << 24], np.int32).reshape(1, 1, 1, 1)
+    for s_b, s_d in ((2e-4, 2e-4), (2e-4, 2.0000001e-4), (1.0, 0.37)):
+        d = _abi.make_conv_desc("NCHW", 1, 1, 2, 2, 1, 1, dst_dtype=_abi.DT_QS32, scale_bias=s_b, scale_dst=s_d)
+        say("case s32 raw", s_b, s_d)
+        got = run_gpu(d, src, flt, bias, None, algo=DIRECT)
+        assert got.reshape(-1).tolist() == [50331649, 50331650, 50331651, 50331653]
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        for z in (False, True):
+            d = _abi.make_conv_desc("NCHW32", 2, 64, 6, 6, 32, 3, pad=1, nonline=nl, has_z=z, dst_dtype=_abi.DT_QS32,
+                                    scale_bias=2e-4, scale_z=3e-4, scale_dst=2.0000001e-4)
+            check_case(oracle, d, seed=91, tag="s32 " + nl, bias_range=(-(1 << 26), 1 << 26), z_range=(-100000, 100000))
+
+
+def test_misaligned_tensors_take_the_generic_kernel(oracle):
+    """Views at a 4-byte offset and a batch stride that is no multiple of 16: the heuristic's choice is replaced by the
+    generic kernel (the reference accepts any pointer); an algorithm asked for by id reports an error instead."""
+    d = _abi.make_conv_desc("NCHW32", 2, 64, 7, 7, 64, 3, pad=1, nonline="RELU", has_z=True, **S)
+    src, flt, bias, z = util.make_tensors(d, seed=5)
+    want = oracle.conv_bias(d, src, flt, bias, z)
+
+    def shifted(x, extra=0):
+        flat = torch.zeros(x.size + 64 + extra, dtype=torch.int8, device="cuda")
+        flat[4:4 + x.size] = torch.from_numpy(x.reshape(-1)).cuda()
+        return flat, flat[4:4 + x.size].view(*x.shape)
+
+    algo, _ = ops.conv_bias_query(d)
+    assert algo.id == IGEMM
+    for which in ("src", "z", "dst"):
+        say("case misaligned", which)
+        t = dict(src=to_dev(src), z=to_dev(z), dst=torch.empty(want.shape, dtype=torch.int8, device="cuda"))
+        keep, t[which] = shifted(dict(src=src, z=z, dst=want)[which])
+        assert t[which].data_ptr() % 16 == 4
+        rc = lib.lib().mi355_convbias_s8_exec(ops._stream(), d, algo, ops._ptr(t["src"]), ops._ptr(to_dev(flt)),
+                                             ops._ptr(to_dev(bias)), ops._ptr(t["z"]), ops._ptr(t["dst"]), None, 0)
+        assert rc == 0, lib.lib().mi355_last_error()
+        torch.cuda.synchronize()
+        assert np.array_equal(t["dst"].cpu().numpy(), want)
+        forced, _ = ops.conv_bias_query(d, IGEMM)
+        rc = lib.lib().mi355_convbias_s8_exec(ops._stream(), d, forced, ops._ptr(t["src"]), ops._ptr(to_dev(flt)),
+                                             ops._ptr(to_dev(bias)), ops._ptr(t["z"]), ops._ptr(t["dst"]), None, 0)
+        assert rc == _abi.ERR_ALGO
+    # a batch stride that is not a multiple of 16 bytes
+    per = src[0].size
+    d2 = _abi.make_conv_desc("NCHW32", 2, 64, 7, 7, 64, 3, pad=1, nonline="RELU", has_z=True, src_stride_n=per + 4, **S)
+    check_case(oracle, d2, seed=5, tag="odd batch stride")
+
+
 def test_direct_exact_epilogue_for_odd_scales(oracle):
     """Scales outside the fast form's envelope take the literal IEEE-divide epilogue."""
     for sd in (1e-20, 3e15):

@@ -16,6 +16,38 @@ from tests import util
 # reference known-answer vectors
 # ----------------------------------------------------------------------------------------
 
+def test_qs32_dst_accumulates_in_place(oracle):
+    """QuantizedS32 dst: the reference accumulates into dst itself (naive/conv_bias/opr_impl.cpp:223-228), so IDENTITY
+    without z stores the raw int32 sum (no float round trip: sums beyond 2^24 stay exact, the scales are not used),
+    and every other case dequantises with the scale of dst.  Expected values are written out by hand / with numpy
+    float32 scalars, not with the checker."""
+    src = np.array([1, 2, 3, 5], np.int8).reshape(1, 1, 2, 2)
+    flt = np.ones((1, 1, 1, 1), np.int8)
+    bias = np.array([3 << 24], np.int32).reshape(1, 1, 1, 1)
+    for s_b, s_d in ((2e-4, 2e-4), (2e-4, 2.0000001e-4), (1.0, 0.37)):
+        d = _abi.make_conv_desc("NCHW", 1, 1, 2, 2, 1, 1, dst_dtype=_abi.DT_QS32, scale_bias=s_b, scale_dst=s_d)
+        out = oracle.conv_bias(d, src, flt, bias, None)
+        assert out.reshape(-1).tolist() == [50331649, 50331650, 50331651, 50331653]
+    # RELU: quantize_s32(relu(float(sum) * s_dst), s_dst) with the scale of dst on both sides (bias scale unused)
+    s_b, s_d = np.float32(2e-4), np.float32(2.0000001e-4)
+    assert s_b != s_d
+    bias = np.array([-7], np.int32).reshape(1, 1, 1, 1)
+    src = np.array([1, 100, -100, 9], np.int8).reshape(1, 1, 2, 2)
+    flt = np.full((1, 1, 1, 1), 3, np.int8)
+    d = _abi.make_conv_desc("NCHW", 1, 1, 2, 2, 1, 1, nonline="RELU", dst_dtype=_abi.DT_QS32, scale_bias=float(s_b),
+                            scale_dst=float(s_d))
+    out = oracle.conv_bias(d, src, flt, bias, None).reshape(-1)
+    libm = C.CDLL("libm.so.6")
+    libm.roundf.restype = C.c_float
+    libm.roundf.argtypes = [C.c_float]
+    want = []
+    for x in (3 * 1 - 7, 3 * 100 - 7, -3 * 100 - 7, 3 * 9 - 7):
+        r = np.float32(x) * s_d
+        r = np.float32(0) if r <= 0 else r
+        want.append(int(libm.roundf(float(np.float32(r / s_d)))))
+    assert out.tolist() == want == [0, 293, 0, 20]
+
+
 def test_kat_conv_bias_quantized8x8x32(oracle, kats):
     k = kats["conv_bias_quantized8x8x32"]
     s_src, s_flt = np.float32(0.1), np.float32(0.2)
