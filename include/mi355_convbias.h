@@ -132,6 +132,9 @@ typedef struct mi355_algo {
 } mi355_algo;
 
 #define MI355_ALGO_HEURISTIC (-1)
+/* the heuristic for a caller that will pre-process the filter for the algorithm it is given (the reference's
+ * weight_preprocess graph option): it may prefer an algorithm that is fastest only with its pre-processed filter */
+#define MI355_ALGO_HEURISTIC_PREPROCESS (-2)
 /* bit of mi355_algo.reserved, set by query() when the heuristic chose the algorithm: exec() may then replace it by
  * the generic kernel when a tensor is not aligned for the tiled kernels (the reference accepts any pointer); an
  * algorithm requested by id is never replaced, exec() reports MI355_ERR_ALGO instead. */
@@ -164,8 +167,8 @@ const char* mi355_convbias_algo_name(int id);
 /* MI355_OK if algorithm `id` can run descriptor `d` */
 int mi355_convbias_algo_usable(const mi355_conv_desc* d, int id);
 
-/* Validate d, pick an algorithm (algo_request = MI355_ALGO_HEURISTIC or a table id) and
- * report the workspace it needs. */
+/* Validate d, pick an algorithm (algo_request = MI355_ALGO_HEURISTIC, MI355_ALGO_HEURISTIC_PREPROCESS or a table
+ * id) and report the workspace it needs. */
 int mi355_convbias_s8_query(const mi355_conv_desc* d, int algo_request, mi355_algo* algo_out,
                             size_t* workspace_bytes);
 
@@ -173,6 +176,24 @@ int mi355_convbias_s8_query(const mi355_conv_desc* d, int algo_request, mi355_al
 int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_algo* algo,
                            const int8_t* src, const int8_t* filter, const int32_t* bias,
                            const int8_t* z, void* dst, void* workspace, size_t workspace_bytes);
+
+/* Weight pre-processing: ConvBiasForward::deduce_preprocessed_filter_layout / get_preprocess_workspace_in_bytes /
+ * exec_preprocess and the PreprocessedFilter argument of exec (dnn/include/megdnn/oprs/nn.h:381-385,400-447; CUDA
+ * precedent dnn/src/cuda/conv_bias/implicit_gemm_int8_nchw32_imma.cpp:164-198: the filter re-ordered once for the
+ * kernel, outside exec).  The artefact belongs to ONE algorithm (pass the mi355_algo of query(), tile included):
+ *   _preprocess_size   bytes of its one pre-processed tensor; 0 when the algorithm reads the reference layout only
+ *                      (then _preprocess does nothing, like the reference's naive backend, and exec takes the filter);
+ *   _preprocess        writes it from the filter in the reference layout (asynchronous on `stream`, no workspace);
+ *   _exec_preprocessed exec with that tensor in place of the filter.
+ * Today the second-generation MFMA tiles ("v2_*") on 32-packed inputs have one: the filter as
+ * [32-byte k-chunk][output channel, padded to a multiple of 32][32 bytes], so that every global -> LDS copy of the
+ * kernel moves one contiguous kilobyte. */
+int mi355_convbias_s8_preprocess_size(const mi355_conv_desc* d, const mi355_algo* algo, size_t* bytes);
+int mi355_convbias_s8_preprocess(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* filter,
+                                 void* preprocessed, size_t preprocessed_bytes);
+int mi355_convbias_s8_exec_preprocessed(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src,
+                                        const void* preprocessed, size_t preprocessed_bytes, const int32_t* bias,
+                                        const int8_t* z, void* dst, void* workspace, size_t workspace_bytes);
 
 /* Profiling primitive of a fast-run chooser (the role of rdnn::AlgoChooser's timed trial runs over
  * get_all_algorithms_info_safe, src/rdnn/impl/algo_chooser.cpp; dnn/include/megdnn/oprs/base.h:545-615): `warmup`

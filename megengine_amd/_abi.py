@@ -25,6 +25,7 @@ BIAS_NONE, BIAS_BROADCAST_CHANNEL, BIAS_FULL = 0, 1, 2
 DT_QS8, DT_QS32, DT_F32 = 0, 1, 2
 
 ALGO_HEURISTIC = -1
+ALGO_HEURISTIC_PREPROCESS = -2
 
 # param::RelayoutFormat::Mode (+ extension modes 32..35)
 RL_NCHW_NCHW4_IC_SMALL = 22

@@ -353,7 +353,8 @@ int mi355_convbias_s8_query(const mi355_conv_desc* d, int algo_request, mi355_al
     int st = canonize(d, &p);
     if (st) return st;
     int id = algo_request;
-    if (id == MI355_ALGO_HEURISTIC) {
+    const bool pre = algo_request == MI355_ALGO_HEURISTIC_PREPROCESS;
+    if (id == MI355_ALGO_HEURISTIC || pre) {
         id = pick_algo(p);
     } else if (id < 0 || id >= ALGO_COUNT) {
         return fail(MI355_ERR_ALGO, "unknown algorithm id %d", id);
@@ -362,21 +363,19 @@ int mi355_convbias_s8_query(const mi355_conv_desc* d, int algo_request, mi355_al
     }
     if (algo_out) {
         algo_out->id = id;
-        algo_out->tile_cfg = id == ALGO_IGEMM_MFMA ? igemm_pick_cfg(p, cu_count()) : 0;
+        algo_out->tile_cfg = id == ALGO_IGEMM_MFMA ? igemm_pick_cfg(p, cu_count(), pre) : 0;
         // an algorithm the heuristic chose may be replaced by the generic kernel at exec time (misaligned tensors);
         // one the caller asked for by id may not
-        algo_out->reserved = algo_request == MI355_ALGO_HEURISTIC ? MI355_ALGO_FLAG_HEURISTIC : 0;
+        algo_out->reserved = algo_request == MI355_ALGO_HEURISTIC || pre ? MI355_ALGO_FLAG_HEURISTIC : 0;
     }
     // every kernel reads the reference layouts in place: no filter repack, no float staging
     if (workspace_bytes) *workspace_bytes = 0;
     return MI355_OK;
 }
 
-int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src,
-                           const int8_t* filter, const int32_t* bias, const int8_t* z, void* dst, void* workspace,
-                           size_t workspace_bytes) {
-    (void)workspace;
-    (void)workspace_bytes;
+// filter: the reference layout, or (preprocessed) the artefact of mi355_convbias_s8_preprocess for this algorithm
+static int exec_impl(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src, const int8_t* filter,
+                     bool preprocessed, const int32_t* bias, const int8_t* z, void* dst) {
     ConvProblem p;
     int st = canonize(d, &p);
     if (st) return st;
@@ -391,6 +390,9 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
     }
     if (id < 0 || id >= ALGO_COUNT) return fail(MI355_ERR_ALGO, "unknown algorithm id %d", id);
     if (!algo_usable(p, id)) return fail(MI355_ERR_ALGO, "%s cannot run this problem", kAlgoNames[id]);
+    if (id == ALGO_IGEMM_MFMA && (cfg < 0 || cfg >= igemm_num_cfgs())) cfg = igemm_pick_cfg(p, cu_count());
+    if (preprocessed && (id != ALGO_IGEMM_MFMA || igemm_preprocessed_bytes(p, cfg) == 0))
+        return fail(MI355_ERR_ALGO, "this algorithm has no pre-processed filter form");
     // the tiled kernels use 16-byte vector accesses; misaligned tensors take the generic kernel
     if (id != ALGO_DIRECT) {
         // (pack-32 tensors move as 16-byte vectors, pack-4 tensors as dwords)
@@ -398,7 +400,8 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
         bool al = aligned16(src) && aligned16(filter) && aligned16(dst) && (!bias || aligned16(bias)) &&
                   (!z || aligned16(z)) && p.src_sn % sa == 0 && p.dst_sn % da == 0 && p.z_sn % da == 0;
         if (!al) {
-            if (algo && algo->id != MI355_ALGO_HEURISTIC && !(algo->reserved & MI355_ALGO_FLAG_HEURISTIC))
+            // the generic kernel reads the reference filter layout only
+            if (preprocessed || (algo && algo->id != MI355_ALGO_HEURISTIC && !(algo->reserved & MI355_ALGO_FLAG_HEURISTIC)))
                 return fail(MI355_ERR_ALGO, "%s needs 16-byte aligned tensors", kAlgoNames[id]);
             id = ALGO_DIRECT;
         }
@@ -410,8 +413,7 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
             rc = launch_conv_direct(hs, p, src, filter, bias, z, dst);
             break;
         case ALGO_IGEMM_MFMA:
-            if (cfg < 0 || cfg >= igemm_num_cfgs()) cfg = igemm_pick_cfg(p, cu_count());
-            rc = launch_conv_igemm(hs, p, cfg, cu_count(), src, filter, bias, z, reinterpret_cast<int8_t*>(dst));
+            rc = launch_conv_igemm(hs, p, cfg, cu_count(), src, filter, bias, z, reinterpret_cast<int8_t*>(dst), preprocessed);
             break;
         case ALGO_DEPTHWISE:
             rc = launch_conv_depthwise(hs, p, src, filter, bias, z, reinterpret_cast<int8_t*>(dst));
@@ -422,6 +424,65 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
     }
     if (rc) return fail(MI355_ERR_LAUNCH, "%s: %s", kAlgoNames[id], hipGetErrorString((hipError_t)rc));
     return MI355_OK;
+}
+
+int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src,
+                           const int8_t* filter, const int32_t* bias, const int8_t* z, void* dst, void* workspace,
+                           size_t workspace_bytes) {
+    (void)workspace;
+    (void)workspace_bytes;
+    return exec_impl(stream, d, algo, src, filter, false, bias, z, dst);
+}
+
+// ---- weight pre-processing ----
+static int preprocess_problem(const mi355_conv_desc* d, const mi355_algo* algo, ConvProblem* p, size_t* bytes) {
+    int st = canonize(d, p);
+    if (st) return st;
+    if (!algo) return fail(MI355_ERR_BAD_ARG, "pre-processing belongs to one algorithm: pass the result of query()");
+    *bytes = 0;
+    if (algo->id == ALGO_IGEMM_MFMA && igemm_usable(*p)) {
+        int cfg = algo->tile_cfg;
+        if (cfg < 0 || cfg >= igemm_num_cfgs()) cfg = igemm_pick_cfg(*p, cu_count());
+        *bytes = igemm_preprocessed_bytes(*p, cfg);
+    }
+    return MI355_OK;
+}
+
+int mi355_convbias_s8_preprocess_size(const mi355_conv_desc* d, const mi355_algo* algo, size_t* bytes) {
+    if (!bytes) return fail(MI355_ERR_BAD_ARG, "null argument");
+    ConvProblem p;
+    return preprocess_problem(d, algo, &p, bytes);
+}
+
+int mi355_convbias_s8_preprocess(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* filter,
+                                 void* preprocessed, size_t preprocessed_bytes) {
+    ConvProblem p;
+    size_t need = 0;
+    int st = preprocess_problem(d, algo, &p, &need);
+    if (st) return st;
+    if (need == 0) return MI355_OK;  // nothing to hoist for this algorithm (the reference's naive form)
+    if (!filter || !preprocessed) return fail(MI355_ERR_BAD_ARG, "null tensor pointer");
+    if (preprocessed_bytes < need)
+        return fail(MI355_ERR_WORKSPACE, "pre-processed filter of %zu bytes, %zu needed", preprocessed_bytes, need);
+    if (!aligned16(filter) || !aligned16(preprocessed)) return fail(MI355_ERR_BAD_ARG, "filter tensors need 16-byte alignment");
+    int rc = launch_igemm_preprocess(reinterpret_cast<hipStream_t>(stream), p, filter, reinterpret_cast<int8_t*>(preprocessed));
+    if (rc) return fail(MI355_ERR_LAUNCH, "preprocess: %s", hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
+}
+
+int mi355_convbias_s8_exec_preprocessed(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src,
+                                        const void* preprocessed, size_t preprocessed_bytes, const int32_t* bias,
+                                        const int8_t* z, void* dst, void* workspace, size_t workspace_bytes) {
+    (void)workspace;
+    (void)workspace_bytes;
+    ConvProblem p;
+    size_t need = 0;
+    int st = preprocess_problem(d, algo, &p, &need);
+    if (st) return st;
+    if (need == 0) return fail(MI355_ERR_ALGO, "this algorithm has no pre-processed filter form");
+    if (preprocessed_bytes < need)
+        return fail(MI355_ERR_WORKSPACE, "pre-processed filter of %zu bytes, %zu needed", preprocessed_bytes, need);
+    return exec_impl(stream, d, algo, src, reinterpret_cast<const int8_t*>(preprocessed), true, bias, z, dst);
 }
 
 int mi355_convbias_s8_profile(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src,

@@ -37,9 +37,15 @@ int launch_conv_direct(hipStream_t st, const ConvProblem& p, const int8_t* src, 
 int igemm_num_cfgs();
 const char* igemm_cfg_name(int cfg);
 bool igemm_usable(const ConvProblem& p);
-int igemm_pick_cfg(const ConvProblem& p, int cu_count);
+// will_preprocess: the caller will hand exec the filter pre-processed for the chosen tile
+int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess = false);
+// flt_preprocessed: flt points to the artefact of launch_igemm_preprocess (only tiles with igemm_preprocessed_bytes > 0)
 int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int tile_cfg, int cu_count, const int8_t* src,
-                      const int8_t* flt, const int32_t* bias, const int8_t* z, int8_t* dst);
+                      const int8_t* flt, const int32_t* bias, const int8_t* z, int8_t* dst, bool flt_preprocessed = false);
+// weight pre-processing: bytes of the re-tiled filter for this problem and tile (0: the tile reads the reference
+// layout only), and the pass that writes it
+size_t igemm_preprocessed_bytes(const ConvProblem& p, int tile_cfg);
+int launch_igemm_preprocess(hipStream_t st, const ConvProblem& p, const int8_t* flt, int8_t* out);
 
 bool depthwise_usable(const ConvProblem& p);
 int launch_conv_depthwise(hipStream_t st, const ConvProblem& p, const int8_t* src, const int8_t* flt,

@@ -509,8 +509,25 @@ bool igemm_usable(const ConvProblem& p) {
     return true;
 }
 
-int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
+int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess) {
     const mi355_conv_desc& d = p.d;
+    if (will_preprocess && p.pin == 32 && p.pout == 32 && d.group == 1 && !d.has_z) {
+        // The caller re-tiles the filter for the chosen algorithm (weight pre-processing): the second-generation tiles
+        // then copy whole kilobytes for both operands and win on the layers without a residual (in-stack sweep of
+        // every tile over the ResNet-50 shapes, plain and pre-processed filters).  Residual layers stay below.
+        enum { V128x128x64r4 = 0, V64x128x128r3 = 3, V64x128x64r4 = 4, V64x64x128r4 = 8 };
+        const int v2 = igemm_first_v2_cfg();
+        const int cu = cu_count > 0 ? cu_count : 256;
+        const int64_t M = (int64_t)d.n * p.oh * p.ow;
+        const int64_t t128 = ((d.oc + 127) / 128) * ((M + 127) / 128);
+        const int kb = (int)(p.icpg * d.fh * d.fw);
+        const bool pw = d.fh == 1 && d.fw == 1 && d.pad_h == 0 && d.pad_w == 0;
+        if (d.oc <= 64) return v2 + (pw && kb >= 256 ? V64x128x128r3 : V64x128x64r4);
+        if (t128 >= cu) return v2 + V128x128x64r4;
+        if (pw) return v2 + V64x128x128r3;
+        if (d.stride_h == 1 && d.stride_w == 1) return v2 + (kb >= 4608 ? V64x64x128r4 : V64x128x128r3);
+        // few tiles, strided 3x3: the first-generation tiles below
+    }
     const int64_t M = (int64_t)d.n * p.oh * p.ow;
     const int OC = d.oc;
     if (cu_count <= 0) cu_count = 256;
@@ -569,8 +586,17 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count) {
     return 3;
 }
 
+size_t igemm_preprocessed_bytes(const ConvProblem& p, int cfg) {
+    if (p.pin != 32 || cfg < igemm_first_v2_cfg() || cfg >= igemm_num_cfgs()) return 0;
+    return igemm2_preprocessed_bytes((int)p.d.oc, (int)(p.icpg * p.d.fh * p.d.fw));
+}
+
+int launch_igemm_preprocess(hipStream_t st, const ConvProblem& p, const int8_t* flt, int8_t* out) {
+    return launch_igemm2_preprocess(st, flt, out, (int)p.d.oc, (int)(p.icpg * p.d.fh * p.d.fw));
+}
+
 int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_count, const int8_t* src,
-                      const int8_t* flt, const int32_t* bias, const int8_t* z, int8_t* dst) {
+                      const int8_t* flt, const int32_t* bias, const int8_t* z, int8_t* dst, bool flt_preprocessed) {
     const mi355_conv_desc& d = p.d;
     IgemmArgs a;
     a.src = src; a.flt = flt; a.bias = bias; a.z = z; a.dst = dst;
@@ -599,6 +625,13 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
     a.epi = p.epi;
     a.flt_rstride = a.kbytes;
     a.flt_kstride = 32;
+    if (flt_preprocessed) {
+        if (igemm_preprocessed_bytes(p, cfg) == 0) return (int)hipErrorInvalidValue;
+        const int ocp = (a.OC + 31) / 32 * 32;
+        a.flt_rstride = 32;
+        a.flt_kstride = ocp * 32;
+        a.flt_bytes = (uint32_t)igemm_preprocessed_bytes(p, cfg);
+    }
     a.groups = d.group;
     a.ocpg = p.ocpg;
     a.src_sg = (p.icpg / p.pin) * a.src_scb;

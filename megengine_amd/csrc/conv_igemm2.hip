@@ -722,6 +722,36 @@ void igemm2_cfg_shape(int cfg, int* bm, int* bn, int* kch) {
     *bm = kCfg2[cfg].bm; *bn = kCfg2[cfg].bn; *kch = kCfg2[cfg].kch;
 }
 
+namespace {
+// [k-chunk][channel, padded to 32][32 bytes]: the 32-byte k-chunk of 32 consecutive filter rows is one contiguous
+// kilobyte -- what one LDS-direct wave copy of the kernel above fetches.  One thread moves 16 bytes.
+__global__ __launch_bounds__(256) void igemm2_preprocess_kernel(const int8_t* flt, int8_t* out, int oc, int ocp, int kbytes,
+                                                                int64_t units) {
+    const int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (u >= units) return;
+    const int64_t kc = u / (ocp * 2);
+    const int r = (int)(u - kc * (ocp * 2));
+    const int row = r >> 1, half = r & 1;
+    v4i v = {0, 0, 0, 0};
+    if (row < oc) v = *reinterpret_cast<const v4i*>(flt + (int64_t)row * kbytes + kc * 32 + half * 16);
+    *reinterpret_cast<v4i*>(out + u * 16) = v;
+}
+}  // namespace
+
+size_t igemm2_preprocessed_bytes(int oc, int kbytes) {
+    const int64_t ocp = (oc + 31) / 32 * 32, kc = (kbytes + 31) / 32;
+    return (size_t)(kc * ocp * 32);
+}
+
+int launch_igemm2_preprocess(hipStream_t st, const int8_t* flt, int8_t* out, int oc, int kbytes) {
+    const int ocp = (oc + 31) / 32 * 32, kc = (kbytes + 31) / 32;
+    const int64_t units = (int64_t)kc * ocp * 2;
+    if (units == 0) return 0;
+    hipLaunchKernelGGL(igemm2_preprocess_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, st, flt, out, oc, ocp,
+                       kbytes, units);
+    return (int)hipGetLastError();
+}
+
 int launch_igemm2(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count) {
     int rc = pout == 32 ? launch_fmt<32>(st, a, cfg, cu_count) : launch_fmt<4>(st, a, cfg, cu_count);
     // the large tiles with a residual need more LDS than a CU has: 128 x 128 x 64 with a ring of three always fits

@@ -202,6 +202,9 @@ const char* igemm2_cfg_name(int cfg);
 void igemm2_cfg_shape(int cfg, int* bm, int* bn, int* kch);
 int launch_igemm2(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count);
 int igemm_first_v2_cfg();  // tile_cfg of the first second-generation tile
+// pre-processed filter of the second-generation kernel: [k-chunk][channel padded to 32][32 bytes]
+size_t igemm2_preprocessed_bytes(int oc, int kbytes);
+int launch_igemm2_preprocess(hipStream_t st, const int8_t* flt, int8_t* out, int oc, int kbytes);
 
 // streaming kernel for 4-packed pointwise layers with few input or few output channels (conv_pw4.hip)
 bool pw4s_usable(const IgemmArgs& a);

@@ -387,7 +387,8 @@ static mi355_algo resolve_algo(const mi355_conv_desc& d, const ExecutionPolicy& 
         return a;
     }
     mi355_algo a;
-    check_abi(mi355_convbias_s8_query(&d, pol.valid() ? pol.algo.id : MI355_ALGO_HEURISTIC, &a, ws));
+    const int heur = pol.weight_preprocess ? MI355_ALGO_HEURISTIC_PREPROCESS : MI355_ALGO_HEURISTIC;
+    check_abi(mi355_convbias_s8_query(&d, pol.valid() ? pol.algo.id : heur, &a, ws));
     if (pol.valid() && pol.algo.tile_cfg >= 0) {
         if (pol.algo.tile_cfg >= mi355_igemm_tile_count()) fail(MI355_ERR_ALGO, "unknown tile configuration");
         a.tile_cfg = pol.algo.tile_cfg;
@@ -405,8 +406,60 @@ size_t ConvBiasForward::get_workspace_in_bytes(const TensorLayout& src, const Te
     return ws;
 }
 
+std::vector<TensorLayout> ConvBiasForward::deduce_preprocessed_filter_layout(const TensorLayout& src,
+                                                                             const TensorLayout& filter,
+                                                                             const TensorLayout& bias, const TensorLayout& z,
+                                                                             const TensorLayout& dst) const {
+    Canon c;
+    canonize(src, filter, bias, z, dst, c, true);
+    size_t ws = 0, bytes = 0;
+    mi355_algo a = resolve_algo(c.d, m_policy, &ws);
+    check_abi(mi355_convbias_s8_preprocess_size(&c.d, &a, &bytes));
+    if (bytes == 0) return {};
+    return {TensorLayout(TensorShape{bytes}, dtype::Int8())};
+}
+
+void ConvBiasForward::exec_preprocess(const TensorLayout& src_layout, const TensorND& filter, const TensorND& bias,
+                                      const TensorLayout& z_layout, const TensorLayout& dst_layout,
+                                      PreprocessedFilter* pf, const Workspace&) {
+    HOST_ASSERT(pf != nullptr, MI355_ERR_BAD_ARG, "null PreprocessedFilter");
+    Canon c;
+    canonize(src_layout, filter.layout, bias.layout, z_layout, dst_layout, c, true);
+    size_t ws = 0, bytes = 0;
+    mi355_algo a = resolve_algo(c.d, m_policy, &ws);
+    pf->algorithm = AlgorithmDesc{a.id, a.tile_cfg};
+    check_abi(mi355_convbias_s8_preprocess_size(&c.d, &a, &bytes));
+    if (bytes == 0) {
+        HOST_ASSERT(pf->tensors.empty(), MI355_ERR_BAD_ARG, "this algorithm has no pre-processed tensors");
+        return;
+    }
+    HOST_ASSERT(pf->tensors.size() == 1 && pf->tensors[0].raw_ptr && pf->tensors[0].layout.total_nr_elems() >= bytes,
+                MI355_ERR_BAD_ARG, "PreprocessedFilter needs the one tensor of deduce_preprocessed_filter_layout (%zu bytes)",
+                bytes);
+    HOST_ASSERT(filter.raw_ptr, MI355_ERR_BAD_ARG, "null filter");
+    check_abi(mi355_convbias_s8_preprocess(m_handle->stream(), &c.d, &a, (const int8_t*)filter.raw_ptr,
+                                           pf->tensors[0].raw_ptr, pf->tensors[0].layout.total_nr_elems()));
+}
+
 void ConvBiasForward::exec(const TensorND& src, const TensorND& filter, const TensorND& bias, const TensorND& z,
-                           const TensorND& dst, const PreprocessedFilter*, const Workspace& workspace) {
+                           const TensorND& dst, const PreprocessedFilter* pf, const Workspace& workspace) {
+    if (pf && !pf->tensors.empty()) {
+        // the artefact was made for pf->algorithm: run exactly that one
+        Canon c;
+        canonize(src.layout, filter.layout, bias.layout, z.layout, dst.layout, c, true);
+        HOST_ASSERT(src.raw_ptr && dst.raw_ptr && pf->tensors[0].raw_ptr, MI355_ERR_BAD_ARG, "null tensor pointer");
+        size_t ws = 0;
+        mi355_algo a;
+        check_abi(mi355_convbias_s8_query(&c.d, pf->algorithm.id, &a, &ws));
+        if (pf->algorithm.tile_cfg >= 0) a.tile_cfg = pf->algorithm.tile_cfg;
+        HOST_ASSERT(workspace.size >= ws, MI355_ERR_WORKSPACE, "workspace of %zu bytes, %zu needed", workspace.size, ws);
+        check_abi(mi355_convbias_s8_exec_preprocessed(m_handle->stream(), &c.d, &a, (const int8_t*)src.raw_ptr,
+                                                      pf->tensors[0].raw_ptr, pf->tensors[0].layout.total_nr_elems(),
+                                                      bias.layout.ndim ? (const int32_t*)bias.raw_ptr : nullptr,
+                                                      z.layout.ndim ? (const int8_t*)z.raw_ptr : nullptr, dst.raw_ptr,
+                                                      workspace.raw_ptr, workspace.size));
+        return;
+    }
     Canon c;
     canonize(src.layout, filter.layout, bias.layout, z.layout, dst.layout, c, true);
     HOST_ASSERT(src.raw_ptr && filter.raw_ptr && dst.raw_ptr, MI355_ERR_BAD_ARG, "null tensor pointer");

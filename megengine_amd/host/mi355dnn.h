@@ -153,6 +153,9 @@ struct ExecutionPolicy {
     enum class Strategy : uint32_t { HEURISTIC = 0, PROFILE = 1 };
     AlgorithmDesc algo;  // id >= 0: use exactly this one, whatever the strategy
     Strategy strategy = Strategy::HEURISTIC;
+    // the caller runs exec_preprocess once and hands exec the PreprocessedFilter (the reference's weight_preprocess
+    // graph option): the heuristic may then choose an algorithm that is fastest only with its pre-processed filter
+    bool weight_preprocess = false;
     bool valid() const { return algo.id >= 0; }
 };
 
@@ -198,7 +201,10 @@ class ConvBiasForward : public OperatorBase {
 public:
     using Param = param::ConvBias;
     enum class BiasMode : uint32_t { NO_BIAS = 0, BROADCAST_CHANNEL_BIAS, BIAS };
+    // the tensors that exec_preprocess filled for `algorithm` (megdnn::detail::PreprocessedFilter,
+    // dnn/include/megdnn/oprs/nn.h:47-52); exec uses them instead of the filter
     struct PreprocessedFilter {
+        AlgorithmDesc algorithm;
         std::vector<TensorND> tensors;
     };
 
@@ -220,14 +226,18 @@ public:
     void exec(const TensorND& src, const TensorND& filter, const TensorND& bias, const TensorND& z,
               const TensorND& dst, const PreprocessedFilter* preprocessed_filter, const Workspace& workspace);
 
-    // weight preprocessing: the kernels read the reference filter layout directly
+    // Weight pre-processing (dnn/include/megdnn/oprs/nn.h:400-447).  The artefact belongs to the algorithm the
+    // execution policy resolves to for these layouts: one Int8 tensor (the filter re-tiled for that kernel's copies),
+    // or no tensor at all when the algorithm reads the reference layout only -- then exec_preprocess does nothing
+    // and exec ignores an empty PreprocessedFilter, as the reference's naive backend does.  No workspace is needed.
     size_t get_preprocess_workspace_in_bytes(const TensorLayout&, const TensorLayout&, const TensorLayout&,
                                              const TensorLayout&, const TensorLayout&) const { return 0; }
-    std::vector<TensorLayout> deduce_preprocessed_filter_layout(const TensorLayout&, const TensorLayout&,
-                                                                const TensorLayout&, const TensorLayout&,
-                                                                const TensorLayout&) const { return {}; }
-    void exec_preprocess(const TensorLayout&, const TensorND&, const TensorND&, const TensorLayout&,
-                         const TensorLayout&, PreprocessedFilter*, const Workspace&) {}
+    std::vector<TensorLayout> deduce_preprocessed_filter_layout(const TensorLayout& src, const TensorLayout& filter,
+                                                                const TensorLayout& bias, const TensorLayout& z,
+                                                                const TensorLayout& dst) const;
+    void exec_preprocess(const TensorLayout& src_layout, const TensorND& filter, const TensorND& bias,
+                         const TensorLayout& z_layout, const TensorLayout& dst_layout,
+                         PreprocessedFilter* preprocessed_filter, const Workspace& workspace);
 
     // algorithm surface
     std::vector<AlgorithmInfo> get_all_algorithms_info(const TensorLayout& src, const TensorLayout& filter,

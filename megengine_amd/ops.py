@@ -73,6 +73,26 @@ def conv_bias_exec(desc, src, flt, bias=None, z=None, dst=None, algo=None, works
     return dst
 
 
+def conv_bias_preprocess(desc, flt, algo):
+    """exec_preprocess: the filter re-tiled for `algo` (a torch uint8 tensor), or None when the algorithm reads the
+    reference layout only (deduce_preprocessed_filter_layout returns nothing for it)."""
+    n = C.c_size_t()
+    check(lib().mi355_convbias_s8_preprocess_size(C.byref(desc), C.byref(algo), C.byref(n)))
+    if n.value == 0:
+        return None
+    out = torch.empty(n.value, dtype=torch.uint8, device=flt.device)
+    check(lib().mi355_convbias_s8_preprocess(_stream(), C.byref(desc), C.byref(algo), _ptr(flt), _ptr(out), n.value))
+    return out
+
+
+def conv_bias_exec_preprocessed(desc, src, pre, bias=None, z=None, dst=None, algo=None):
+    if dst is None:
+        dst = torch.empty(_abi.conv_shapes(desc)[3], dtype=torch.int8, device=src.device)
+    check(lib().mi355_convbias_s8_exec_preprocessed(_stream(), C.byref(desc), C.byref(algo), _ptr(src), _ptr(pre),
+                                                   pre.numel(), _ptr(bias), _ptr(z), _ptr(dst), None, 0))
+    return dst
+
+
 def conv_bias_profile(desc, src, flt, bias, z, dst, algo, warmup=2, iters=10, workspace=None):
     """Average time in microseconds of one launch of `algo` (synchronises the current stream, overwrites dst)."""
     us = C.c_float()
@@ -82,14 +102,20 @@ def conv_bias_profile(desc, src, flt, bias, z, dst, algo, warmup=2, iters=10, wo
     return us.value
 
 
-def conv_bias_bind(desc, src, flt, bias, z, dst, algo, workspace=None, stream=None):
+def conv_bias_bind(desc, src, flt, bias, z, dst, algo, workspace=None, stream=None, preprocessed=None):
     """Pre-marshals one exec call; the returned callable launches it on the CURRENT torch stream
     when `stream` is None, else on that raw stream handle, and raises on a non-zero status.
-    Keeps the tensors alive.  For callers that replay the same launch many times."""
-    fn = lib().mi355_convbias_s8_exec
+    Keeps the tensors alive.  For callers that replay the same launch many times.  With `preprocessed` (the result of
+    conv_bias_preprocess for the same algo) the call is exec with a PreprocessedFilter."""
     wsn = workspace.numel() if workspace is not None else 0
-    tail = (C.byref(desc), C.byref(algo), _ptr(src), _ptr(flt), _ptr(bias), _ptr(z), _ptr(dst), _ptr(workspace), wsn)
-    keep = (desc, algo, src, flt, bias, z, dst, workspace)
+    if preprocessed is not None:
+        fn = lib().mi355_convbias_s8_exec_preprocessed
+        tail = (C.byref(desc), C.byref(algo), _ptr(src), _ptr(preprocessed), preprocessed.numel(), _ptr(bias), _ptr(z),
+                _ptr(dst), _ptr(workspace), wsn)
+    else:
+        fn = lib().mi355_convbias_s8_exec
+        tail = (C.byref(desc), C.byref(algo), _ptr(src), _ptr(flt), _ptr(bias), _ptr(z), _ptr(dst), _ptr(workspace), wsn)
+    keep = (desc, algo, src, flt, bias, z, dst, workspace, preprocessed)
     fixed = None if stream is None else C.c_void_p(stream)
 
     def call(_keep=keep):

@@ -154,3 +154,22 @@ def build_stack(layers, seed):
         prev = L.name
         plan.append(dict(layer=L, desc=desc, src=src, flt=flt, bias=bias, z=z, dst=dst))
     return plan
+
+
+def choose_algorithms(plan, weight_preprocess=True):
+    """Algorithm choice for every layer of a plan, as an inference graph does it once at load time: the heuristic
+    (for a caller that pre-processes weights when `weight_preprocess`), then exec_preprocess of the filter where the
+    chosen algorithm has a pre-processed form.  Fills p["algo"] and p["pre"] (None: exec takes the filter)."""
+    from . import ops
+    for p in plan:
+        req = _abi.ALGO_HEURISTIC_PREPROCESS if weight_preprocess else _abi.ALGO_HEURISTIC
+        p["algo"], _ = ops.conv_bias_query(p["desc"], req)
+        p["pre"] = ops.conv_bias_preprocess(p["desc"], p["flt"], p["algo"]) if weight_preprocess else None
+    return plan
+
+
+def bind_plan(plan, stream=None):
+    """One pre-marshalled launch per layer (exec, or exec with the PreprocessedFilter)."""
+    from . import ops
+    return [ops.conv_bias_bind(p["desc"], p["src"], p["flt"], p["bias"], p["z"], p["dst"], p["algo"], stream=stream,
+                               preprocessed=p.get("pre")) for p in plan]

@@ -561,6 +561,79 @@ static void run_fast_run_gpu(Handle* h) {
     AlgorithmCache::instance().clear();
 }
 
+// weight pre-processing: deduce_preprocessed_filter_layout -> exec_preprocess -> exec with the PreprocessedFilter, the way the
+// reference's OprProxy drives it (dnn/test/common/opr_proxy.h, "weight preprocess" proxies)
+static void run_preprocess_gpu(Handle* h) {
+    printf("case: weight pre-processing\n");
+    fflush(stdout);
+    const float s_src = 0.02f, s_flt = 0.01f, s_dst = 0.05f;
+    for (int variant = 0; variant < 3; ++variant) {
+        auto opr = h->create_operator<ConvBiasForward>();
+        opr->param().format = CB::Format::NCHW32;
+        opr->param().nonlineMode = variant == 1 ? CB::NonlineMode::H_SWISH : CB::NonlineMode::RELU;
+        const bool pw = variant == 2;
+        opr->param().pad_h = opr->param().pad_w = pw ? 0 : 1;
+        opr->execution_policy().weight_preprocess = true;
+        TensorLayout src({3, 4, 14, 14, 32}, dtype::QuantizedS8(s_src));
+        TensorLayout flt(pw ? TensorShape{160, 4, 1, 1, 32} : TensorShape{160, 4, 3, 3, 32}, dtype::QuantizedS8(s_flt));
+        TensorLayout bias({1, 5, 1, 1, 32}, dtype::QuantizedS32(s_src * s_flt)), z, dst;
+        dst.dtype = dtype::QuantizedS8(s_dst);
+        opr->deduce_layout(src, flt, bias, z, dst);
+        std::vector<int8_t> hsrc(src.total_nr_elems()), hflt(flt.total_nr_elems());
+        std::vector<int32_t> hbias(bias.total_nr_elems());
+        fill_s8(hsrc, 31 + variant, -128, 127);
+        fill_s8(hflt, 32 + variant, -127, 127);
+        fill_s32(hbias, 33 + variant, -1000, 1000);
+        mi355_conv_desc d = mi355_conv_desc();
+        d.format = MI355_FMT_NCHW32; d.nonline = (uint32_t)opr->param().nonlineMode; d.n = 3; d.ic = 128; d.ih = d.iw = 14;
+        d.oc = 160; d.fh = d.fw = pw ? 1 : 3; d.group = 1; d.pad_h = d.pad_w = pw ? 0 : 1; d.stride_h = d.stride_w = 1;
+        d.dilate_h = d.dilate_w = 1; d.bias_mode = MI355_BIAS_BROADCAST_CHANNEL; d.scale_bias = s_src * s_flt; d.scale_z = 1.f;
+        d.scale_dst = s_dst;
+        std::vector<int8_t> expect(dst.total_nr_elems()), got(dst.total_nr_elems());
+        EXPECT(oracle_convbias_s8(&d, hsrc.data(), hflt.data(), hbias.data(), nullptr, expect.data()) == 0, "CPU checker");
+        DevBuf dsrc(hsrc.size()), dflt(hflt.size()), dbias(hbias.size() * 4), ddst(got.size()), dws(16);
+        HIP_OK(hipMemcpy(dsrc.p, hsrc.data(), hsrc.size(), hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dflt.p, hflt.data(), hflt.size(), hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dbias.p, hbias.data(), hbias.size() * 4, hipMemcpyHostToDevice));
+
+        EXPECT(opr->get_preprocess_workspace_in_bytes(src, flt, bias, z, dst) == 0, "no pre-processing workspace");
+        auto layouts = opr->deduce_preprocessed_filter_layout(src, flt, bias, z, dst);
+        EXPECT(layouts.size() == 1, "the heuristic for pre-processing callers must pick an algorithm with a pre-processed filter");
+        if (layouts.size() != 1) return;
+        EXPECT(layouts[0].total_nr_elems() >= flt.total_nr_elems(), "the re-tiled filter holds every filter byte");
+        DevBuf dpre(layouts[0].total_nr_elems());
+        HIP_OK(hipMemset(dpre.p, 0x77, layouts[0].total_nr_elems()));
+        ConvBiasForward::PreprocessedFilter pf;
+        pf.tensors.push_back(TensorND(dpre.p, layouts[0]));
+        opr->exec_preprocess(src, TensorND(dflt.p, flt), TensorND(dbias.p, bias), z, dst, &pf, Workspace(dws.p, 0));
+        // exec must not touch the filter any more: poison it
+        HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
+        HIP_OK(hipMemset(dflt.p, 0x33, hflt.size()));
+        HIP_OK(hipMemset(ddst.p, 0x5a, got.size()));
+        opr->exec(TensorND(dsrc.p, src), TensorND(dflt.p, flt), TensorND(dbias.p, bias), TensorND(nullptr, z), TensorND(ddst.p, dst),
+                  &pf, Workspace(dws.p, 0));
+        HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
+        HIP_OK(hipMemcpy(got.data(), ddst.p, got.size(), hipMemcpyDeviceToHost));
+        size_t bad = 0;
+        for (size_t i = 0; i < got.size(); ++i) bad += got[i] != expect[i];
+        EXPECT(bad == 0, "exec with a PreprocessedFilter (variant %d): %zu bytes differ from the CPU checker", variant, bad);
+        // a PreprocessedFilter with the wrong tensor count is refused
+        ConvBiasForward::PreprocessedFilter empty;
+        EXPECT(throws([&] { opr->exec_preprocess(src, TensorND(dflt.p, flt), TensorND(dbias.p, bias), z, dst, &empty,
+                                                 Workspace(dws.p, 0)); }, MI355_ERR_BAD_ARG),
+               "exec_preprocess must refuse a PreprocessedFilter without the deduced tensor");
+    }
+    // an algorithm that reads the reference layout only: nothing to hoist (the naive backend's answer)
+    auto opr = h->create_operator<ConvBiasForward>();
+    opr->param().format = CB::Format::NCHW4;
+    opr->param().pad_h = opr->param().pad_w = 1;
+    TensorLayout src({1, 4, 8, 8, 4}, dtype::QuantizedS8(s_src)), flt({16, 4, 3, 3, 4}, dtype::QuantizedS8(s_flt));
+    TensorLayout bias({1, 4, 1, 1, 4}, dtype::QuantizedS32(s_src * s_flt)), z, dst;
+    dst.dtype = dtype::QuantizedS8(s_dst);
+    opr->deduce_layout(src, flt, bias, z, dst);
+    EXPECT(opr->deduce_preprocessed_filter_layout(src, flt, bias, z, dst).empty(), "4-packed inputs have no pre-processed form");
+}
+
 int main(int argc, char** argv) {
     bool gpu = argc > 1 && !strcmp(argv[1], "--gpu");
     bool cpu = argc > 1 && !strcmp(argv[1], "--cpu");
@@ -583,6 +656,7 @@ int main(int argc, char** argv) {
         if (gpu) run_elemwise_gpu(handle.get());
         if (gpu) run_pooling_gpu(handle.get());
         if (gpu) run_fast_run_gpu(handle.get());
+        if (gpu) run_preprocess_gpu(handle.get());
     } catch (const Error& e) {
         printf("unexpected mi355dnn::Error %d: %s\n", e.status(), e.what());
         return 1;

@@ -310,6 +310,48 @@ def test_heuristic_picks(oracle):
         assert a.id == IGEMM and names[a.tile_cfg] == want, (ic, hw, oc, names[a.tile_cfg])
 
 
+def test_preprocessed_filter_equals_plain_filter(oracle):
+    """exec with a PreprocessedFilter == exec with the filter, bit for bit, for every tile that has a pre-processed form;
+    tiles without one report size 0 (nothing to hoist) and refuse exec_preprocessed."""
+    names = lib.tile_names()
+    n_pre = 0
+    for ci, (fmt, n, ic, ih, iw, oc, f, pad, stride) in enumerate(IGEMM_CASES):
+        for nl, z in (("RELU", True), ("IDENTITY", False)):
+            if z and fmt in ("NCHW4_NCHW32", "NCHW32_NCHW4"):
+                continue
+            d = _abi.make_conv_desc(fmt, n, ic, ih, iw, oc, f, pad=pad, stride=stride, nonline=nl, has_z=z, **S)
+            src, flt, bias, zz = util.make_tensors(d, seed=700 + ci)
+            dev = [to_dev(x) for x in (src, flt, bias, zz)]
+            for tile in range(len(names)):
+                a, _ = ops.conv_bias_query(d, IGEMM)
+                a.tile_cfg = tile
+                pre = ops.conv_bias_preprocess(d, dev[1], a)
+                if pre is None:
+                    assert not (names[tile].startswith("v2_") and fmt in ("NCHW32", "NCHW32_NCHW4"))
+                    continue
+                assert names[tile].startswith("v2_")
+                say("case preprocessed", fmt, n, ic, ih, iw, oc, f, pad, stride, nl, z, names[tile])
+                plain = ops.conv_bias_exec(d, dev[0], dev[1], dev[2], dev[3], algo=a)
+                got = ops.conv_bias_exec_preprocessed(d, dev[0], pre, dev[2], dev[3], algo=a)
+                torch.cuda.synchronize()
+                assert torch.equal(got, plain), names[tile]
+                n_pre += 1
+    assert n_pre > 0
+    # group convolution with a pre-processed filter, against the checker
+    d = _abi.make_conv_desc("NCHW32", 2, 128, 9, 9, 192, 3, pad=1, group=2, nonline="H_SWISH", has_z=True, **S)
+    src, flt, bias, zz = util.make_tensors(d, seed=777)
+    want = oracle.conv_bias(d, src, flt, bias, zz)
+    a, _ = ops.conv_bias_query(d)
+    pre = ops.conv_bias_preprocess(d, to_dev(flt), a)
+    assert pre is not None
+    got = ops.conv_bias_exec_preprocessed(d, to_dev(src), pre, to_dev(bias), to_dev(zz), algo=a)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+    # an algorithm without a pre-processed form
+    a, _ = ops.conv_bias_query(d, DIRECT)
+    assert ops.conv_bias_preprocess(d, to_dev(flt), a) is None
+
+
 # ---------------------------------------------------------------------------------------------
 # every tile configuration (register-staged and LDS-direct, 4- and 8-wave) on ragged shapes
 # ---------------------------------------------------------------------------------------------

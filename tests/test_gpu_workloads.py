@@ -27,16 +27,19 @@ def host(t):
 
 
 def run_plan(plan):
-    for p in plan:
-        p["algo"], _ = ops.conv_bias_query(p["desc"])
-        ops.conv_bias_exec(p["desc"], p["src"], p["flt"], p["bias"], p["z"], dst=p["dst"], algo=p["algo"])
+    """exactly what bench.py launches: the heuristic for pre-processing callers, filters pre-processed where the chosen
+    algorithm has such a form"""
+    workloads.choose_algorithms(plan)
+    for call in workloads.bind_plan(plan):
+        call()
     torch.cuda.synchronize()
 
 
 def check_layer(oracle, p, seed):
     l, d = p["layer"], p["desc"]
     say("layer", l.name, "ic", l.ic, "oc", l.oc, "hw", l.ih, "f", l.f, "s", l.stride, "g", l.group, "z", l.z is not None,
-        "algo", lib.algo_names()[p["algo"].id], lib.tile_names()[p["algo"].tile_cfg] if p["algo"].id == IGEMM else "")
+        "algo", lib.algo_names()[p["algo"].id], lib.tile_names()[p["algo"].tile_cfg] if p["algo"].id == IGEMM else "",
+        "pre-processed filter" if p.get("pre") is not None else "")
     got = p["dst"]
     idx = (util.splitmix64(seed, NPOINTS) % np.uint64(got.numel())).astype(np.int64)
     want = oracle.conv_bias_points(d, host(p["src"]), host(p["flt"]), host(p["bias"]), host(p["z"]), idx)
@@ -69,6 +72,12 @@ def test_config2_resnet50_stack(oracle, resnet_plan, part):
     assert len(plan) == 53
     for i in range(part, len(plan), 6):
         check_layer(oracle, plan[i], seed=1000 + i)
+
+
+def test_config2_uses_preprocessed_filters(resnet_plan):
+    n = sum(p.get("pre") is not None for p in resnet_plan)
+    say(n, "of 53 layers run with a pre-processed filter")
+    assert n >= 20
 
 
 def test_config2_requantisation_forms(resnet_plan):
