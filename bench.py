@@ -37,6 +37,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip the per-config side measurements")
+    ap.add_argument("--extras-only", action="store_true",
+                    help="side measurements only (short runs for profilers): prints their JSON, no headline")
+    ap.add_argument("--side-iters", type=int, default=50, help="launches per side measurement")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only")
     ap.add_argument("--no-preprocess", action="store_true", help="exec with the filters in the reference layout only")
@@ -62,6 +65,13 @@ def main():
     log("device: %s %s, %d CUs, %.0f MHz" % (info.name.decode(), info.arch.decode(), info.compute_units,
                                              info.clock_khz / 1e3))
     torch.manual_seed(1234)
+    if args.extras_only:
+        side = torch.cuda.Stream()
+        torch.cuda.set_stream(side)
+        print(json.dumps(dict(other_configs=run_extras(torch, np, _abi, lib, ops, workloads, args.side_iters))), flush=True)
+        if args.calib_copy:
+            calib_copy(torch)
+        return
     batch = 64
     layers = workloads.resnet50(batch)
     plan = workloads.build_stack(layers, 7)
@@ -168,7 +178,10 @@ def main():
     tr = os.path.join(ROOT, "profiles", "traffic_resnet50_stack.json")
     if os.path.exists(tr):
         try:
-            roofline["traffic"] = json.load(open(tr))["hbm_bytes_per_launch"]
+            trj = json.load(open(tr))
+            roofline["traffic"] = trj["hbm_bytes_per_launch"]
+            # not measured by this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes over this same command
+            roofline["traffic_source"] = "profiles/traffic_resnet50_stack.json (%s)" % trj.get("measured", "earlier counter pass")
         except Exception:
             pass
 
@@ -188,17 +201,12 @@ def main():
                roofline=roofline)
 
     if args.calib_copy:
-        a = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device="cuda")
-        b = torch.empty_like(a)
-        torch.cuda.synchronize()
-        torch.bitwise_not(a, out=b)     # reads 256 MiB, writes 256 MiB
-        torch.cuda.synchronize()
-        del a, b
+        calib_copy(torch)
 
     extras = {}
     if not args.no_extras:
         try:
-            extras = run_extras(torch, np, _abi, lib, ops, workloads)
+            extras = run_extras(torch, np, _abi, lib, ops, workloads, args.side_iters)
         except Exception as e:  # side measurements must not lose the headline
             extras = dict(error=repr(e))
         out["other_configs"] = extras
@@ -213,6 +221,17 @@ def main():
         for row in table:
             log(row)
     print(json.dumps(out), flush=True)
+
+
+def calib_copy(torch):
+    """One plain streaming kernel of known size (reads 256 MiB, writes 256 MiB): the reference point that scales the
+    profiler's FETCH_SIZE / WRITE_SIZE counters."""
+    a = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device="cuda")
+    b = torch.empty_like(a)
+    torch.cuda.synchronize()
+    torch.bitwise_not(a, out=b)
+    torch.cuda.synchronize()
+    del a, b
 
 
 class EventTimer:
@@ -266,8 +285,32 @@ def time_launches(torch, fn, iters=20, warm=3):
     return e0.elapsed_time(e1) / iters * 1e-3
 
 
-def run_extras(torch, np, _abi, lib, ops, workloads):
-    """Side measurements for the other workload configurations (not the headline value)."""
+_FLUSH = None
+
+
+def time_launches_cold(torch, fn, iters=8):
+    """Like time_launches, but L2 and the 256 MB last-level cache are flushed before every launch (a 512 MiB fill on
+    the same stream); only the launch itself is between the two events of an iteration."""
+    global _FLUSH
+    if _FLUSH is None:
+        _FLUSH = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream()
+    fn()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for e0, e1 in ev:
+        _FLUSH.fill_(1)
+        e0.record(st)
+        fn()
+        e1.record(st)
+    torch.cuda.synchronize()
+    t = sorted(e0.elapsed_time(e1) for e0, e1 in ev)
+    return t[len(t) // 2] * 1e-3
+
+
+def run_extras(torch, np, _abi, lib, ops, workloads, side_iters=50):
+    """Side measurements for the other workload configurations (not the headline value).  Every row carries two
+    times: "us" = the launch repeated back to back on the same tensors (operands warm in L2 / the last-level cache
+    when they fit), "us_cold" = median of launches that each follow a flush of both caches."""
     res = {}
 
     def measure(layers, seed):
@@ -276,11 +319,13 @@ def run_extras(torch, np, _abi, lib, ops, workloads):
         workloads.choose_algorithms(plan)
         # pre-marshalled launches: the per-call Python work of conv_bias_exec would floor short kernels
         for p, call in zip(plan, workloads.bind_plan(plan)):
-            t = time_launches(torch, call, iters=50)
+            t = time_launches(torch, call, iters=side_iters)
+            tc = time_launches_cold(torch, call, iters=max(3, min(8, side_iters)))
             l = p["layer"]
+            roof = max(l.ops / INT8_PEAK_OPS, l.bytes / HBM_PEAK)
             rows.append(dict(name=l.name, algo=lib.algo_names()[p["algo"].id], us=round(t * 1e6, 2),
-                             tops=round(l.ops / t / 1e12, 1), gbs=round(l.bytes / t / 1e9, 1),
-                             frac_roof=round(max(l.ops / INT8_PEAK_OPS, l.bytes / HBM_PEAK) / t, 3)))
+                             us_cold=round(tc * 1e6, 2), tops=round(l.ops / t / 1e12, 1), gbs=round(l.bytes / t / 1e9, 1),
+                             frac_roof=round(roof / t, 3), frac_roof_cold=round(roof / tc, 3)))
         return rows, plan
 
     rows, _ = measure([workloads.config0()], 1)
@@ -294,12 +339,17 @@ def run_extras(torch, np, _abi, lib, ops, workloads):
     pw = [(r, l) for r, l in zip(rows, mb) if l.group == 1]
     t_dw = sum(r["us"] for r, _ in dw) * 1e-6
     t_pw = sum(r["us"] for r, _ in pw) * 1e-6
+    tc_dw = sum(r["us_cold"] for r, _ in dw) * 1e-6
+    tc_pw = sum(r["us_cold"] for r, _ in pw) * 1e-6
     res["config3_mobilenetv2"] = dict(
         depthwise=dict(us=round(t_dw * 1e6, 1), gbs=round(sum(l.bytes for _, l in dw) / t_dw / 1e9, 1),
-                       frac_hbm=round(sum(l.bytes for _, l in dw) / t_dw / HBM_PEAK, 3)),
+                       frac_hbm=round(sum(l.bytes for _, l in dw) / t_dw / HBM_PEAK, 3), us_cold=round(tc_dw * 1e6, 1),
+                       frac_hbm_cold=round(sum(l.bytes for _, l in dw) / tc_dw / HBM_PEAK, 3),
+                       layers=[r for r, _ in dw]),
         pointwise=dict(us=round(t_pw * 1e6, 1), gbs=round(sum(l.bytes for _, l in pw) / t_pw / 1e9, 1),
                        tops=round(sum(l.ops for _, l in pw) / t_pw / 1e12, 1),
-                       frac_hbm=round(sum(l.bytes for _, l in pw) / t_pw / HBM_PEAK, 3)))
+                       frac_hbm=round(sum(l.bytes for _, l in pw) / t_pw / HBM_PEAK, 3), us_cold=round(tc_pw * 1e6, 1),
+                       frac_hbm_cold=round(sum(l.bytes for _, l in pw) / tc_pw / HBM_PEAK, 3)))
     torch.cuda.empty_cache()
     c4 = []
     for l in workloads.large_hswish():
@@ -316,10 +366,12 @@ def run_extras(torch, np, _abi, lib, ops, workloads):
             ops.conv_bias_exec(p["desc"], p["src"], p["flt"], p["bias"], p["z"], dst=p["dst"], algo=p["algo"])
             ops.relayout_exec(d_out, p["dst"], y_nchw)
 
-        t_full = time_launches(torch, full, iters=10)
-        t_in = time_launches(torch, lambda: ops.relayout_exec(d_in, x_nchw, p["src"]), iters=10)
-        t_out = time_launches(torch, lambda: ops.relayout_exec(d_out, p["dst"], y_nchw), iters=10)
+        n10 = max(2, min(10, side_iters))
+        t_full = time_launches(torch, full, iters=n10)
+        t_in = time_launches(torch, lambda: ops.relayout_exec(d_in, x_nchw, p["src"]), iters=n10)
+        t_out = time_launches(torch, lambda: ops.relayout_exec(d_out, p["dst"], y_nchw), iters=n10)
         rl_bytes_in, rl_bytes_out = 2 * x_nchw.numel(), 2 * y_nchw.numel()
+        # (these tensors are 67-134 MB each and stream through both caches: every launch is a cold one)
         c4.append(dict(conv=rows[0], total_us=round(t_full * 1e6, 1),
                        relayout_in_gbs=round(rl_bytes_in / t_in / 1e9, 1),
                        relayout_out_gbs=round(rl_bytes_out / t_out / 1e9, 1),
