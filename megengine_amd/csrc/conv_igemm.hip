@@ -483,6 +483,10 @@ const char* igemm_cfg_name(int cfg) {
 }
 int igemm_first_v2_cfg() { return kNumCfgs + igemm_dma_num_cfgs(); }
 
+static bool igemm_needs_general(const ConvProblem& p) {
+    return p.d.dst_dtype != MI355_DT_QS8 || p.d.bias_mode == MI355_BIAS_FULL || !p.epi.fast;
+}
+
 bool igemm_usable(const ConvProblem& p) {
     const mi355_conv_desc& d = p.d;
     if (p.dw4) return false;
@@ -492,8 +496,13 @@ bool igemm_usable(const ConvProblem& p) {
         d.format != MI355_FMT_NCHW32_NCHW4)
         return false;
     if (d.mode != MI355_MODE_CROSS_CORRELATION || d.dilate_h != 1 || d.dilate_w != 1) return false;
-    if (d.dst_dtype != MI355_DT_QS8 || d.bias_mode == MI355_BIAS_FULL) return false;
-    if (!p.epi.fast) return false;
+    // QuantizedS32 dst (without a residual), full-shape bias and scales outside the fast forms' envelope run the
+    // second-generation tiles with their general epilogue: 32-packed inputs only
+    if (igemm_needs_general(p)) {
+        if (p.pin != 32) return false;
+        if (d.dst_dtype == MI355_DT_QS32 && d.has_z) return false;
+        if (d.dst_dtype == MI355_DT_F32) return false;
+    }
     if (d.fh > 255 || d.fw > 255 || d.pad_h > 0xfff || d.pad_w > 0xfff || d.ih > 0x3000 || d.iw > 0x3000) return false;
     // 32-bit byte offsets and buffer descriptors
     const int64_t lim = (int64_t)1 << 31;
@@ -531,8 +540,8 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess) {
     const int64_t M = (int64_t)d.n * p.oh * p.ow;
     const int OC = d.oc;
     if (cu_count <= 0) cu_count = 256;
-    // group convolution: second-generation tiles only; a channel tile never spans two groups
-    if (d.group != 1) return igemm_first_v2_cfg() + (p.ocpg <= 64 ? 3 : 0);
+    // group convolution and the general epilogue: second-generation tiles only; a channel tile never spans two groups
+    if (d.group != 1 || igemm_needs_general(p)) return igemm_first_v2_cfg() + (p.ocpg <= 64 ? 3 : 0);
     auto tiles = [&](int cfg) { return ((OC + kCfgs[cfg].bm - 1) / kCfgs[cfg].bm) * ((M + kCfgs[cfg].bn - 1) / kCfgs[cfg].bn); };
     const int kbytes = d.ic * d.fh * d.fw;
     if (p.pin == 4 && p.pout == 4 && d.fh == 1 && d.fw == 1 && d.pad_h == 0 && d.pad_w == 0) {
@@ -637,8 +646,12 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
     a.src_sg = (p.icpg / p.pin) * a.src_scb;
     if (a.M == 0 || a.OC == 0) return 0;
     const int first_v2 = igemm_first_v2_cfg();
-    // group convolutions exist on the second-generation tiles only
-    if (d.group != 1 && cfg < first_v2) cfg = first_v2;
+    a.general = igemm_needs_general(p) ? 1 : 0;
+    a.dst_s32 = d.dst_dtype == MI355_DT_QS32;
+    a.bias_full = d.bias_mode == MI355_BIAS_FULL;
+    if (a.dst_s32) a.epi.s_b = a.epi.s_d;  // the sum lives in dst and is dequantised with the dtype of dst
+    // group convolutions and the general epilogue exist on the second-generation tiles only
+    if ((d.group != 1 || a.general) && cfg < first_v2) cfg = first_v2;
     if (cfg >= first_v2) {
         if (p.pin == 32) return launch_igemm2(st, a, p.pout, cfg - first_v2, cu_count);
         // 4-packed inputs: the register-staged tile of the same shape

@@ -348,7 +348,7 @@ struct Igemm2 {
         extern __shared__ __attribute__((aligned(16))) int8_t lds[];
         int* sBias = reinterpret_cast<int*>(lds + NS * STG);
         // [ring][bias][residual slots, only for launches with a residual][k-unit table]
-        const int zslots = a.epi.has_z ? a.zslots : 0;
+        const int zslots = a.zslots;
         KEntry* tab = reinterpret_cast<KEntry*>(lds + RING_BYTES + zslots * ZSLOT);
         const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)lds);
 
@@ -581,7 +581,10 @@ struct Igemm2 {
                 read_z(zr, zbuf + zslot * ZSLOT, lane);
                 if (zslots == 2) zslot ^= 1;
             }
-            igemm_run_epilogue<POUT, MT, NT, true>(a, acc, cur.oc0 + wm * WTM, cur.pix0 + wn * WTN, l32, lh, &zr, cur.oc_end);
+            if (a.general)
+                igemm_epilogue_general<POUT, MT, NT>(a, acc, cur.oc0 + wm * WTM, cur.pix0 + wn * WTN, l32, lh, cur.oc_end);
+            else
+                igemm_run_epilogue<POUT, MT, NT, true>(a, acc, cur.oc0 + wm * WTM, cur.pix0 + wn * WTN, l32, lh, &zr, cur.oc_end);
             c_tile += step;
             if (ti + 1 < my_tiles) {
                 if (nxt.oc0 != cur.oc0) {
@@ -647,7 +650,7 @@ int launch_k(hipStream_t st, IgemmArgs& a, int cu_count) {
     // tile to hide it behind (one slot, and room for a second workgroup per CU)
     const int fixed = K::RING_BYTES + tab_entries * 8;
     a.zslots = 0;
-    if (a.epi.has_z) {
+    if (a.epi.has_z && !a.general) {
         a.zslots = a.nstages <= 2 ? 2 : 1;
         if (fixed + a.zslots * K::ZSLOT > kLdsPerCu) a.zslots = 1;
     }

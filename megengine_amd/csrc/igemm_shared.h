@@ -41,6 +41,9 @@ struct IgemmArgs {
     // group convolution: ocpg output channels per group, src_sg bytes between the channel blocks of two groups
     int groups, ocpg, src_sg, tiles_m_pg;
     int zslots;  // residual slots in LDS: 0 (no residual), 1 or 2
+    // general epilogue (second-generation kernel): QuantizedS32 dst, full-shape bias, or scales outside the fast
+    // forms' envelope.  bias_full: a.bias has the shape of dst (contiguous) and has_bias is 0.
+    int general, dst_s32, bias_full;
 };
 
 struct KEntry {
@@ -184,6 +187,55 @@ __device__ __forceinline__ void igemm_run_epilogue(const IgemmArgs& a, v16i (&ac
             case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
             case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
             default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
+        }
+    }
+}
+
+// General epilogue of one wave tile: every dst dtype / bias shape / scale the operator accepts, with the literal
+// requantisation chain where the fast forms do not apply.  Register quad q of a 32x32 block holds channels
+// ocb + 8q + 4 (lane / 32) .. + 3 of pixel lane % 32: one dword of int8 results, or 16 bytes of int32 results.
+// QuantizedS32 dst (no residual here): the reference accumulates in dst itself, IDENTITY stores the raw sum, the
+// activations dequantise with the scale of dst (e.s_b holds it; naive/conv_bias/opr_impl.cpp:223-228,52,69-73,89-93).
+template <int POUT, int MT, int NT>
+__device__ __forceinline__ void igemm_epilogue_general(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w, int l32,
+                                                       int lh, int oc_end) {
+    const bool hz = a.epi.has_z != 0;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int m = pix_w + j * 32 + l32;
+        const bool pok = m < a.M;
+        const uint32_t mm = pok ? m : 0;
+        const uint32_t n = fdiv(mm, a.div_ohw), rem = mm - n * a.OHW;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int ocb = oc_w + i * 32;
+            if (ocb >= oc_end) continue;  // wave-uniform
+            const v16i& c = acc[i][j];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int oc4 = ocb + 8 * q + 4 * lh;
+                if (!(pok && oc4 < oc_end)) continue;
+                // element offsets inside one image (dst layout) and of the image
+                const int64_t in_img = (int64_t)(oc4 / POUT) * (a.OHW * POUT) + (int64_t)rem * POUT + (oc4 % POUT);
+                int v[4] = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
+                if (a.bias_full) {
+                    const v4i b = *reinterpret_cast<const v4i*>(a.bias + (int64_t)n * ((int64_t)a.OC * a.OHW) + in_img);
+                    v[0] += b[0]; v[1] += b[1]; v[2] += b[2]; v[3] += b[3];
+                }
+                if (a.dst_s32) {
+                    v4i o = {v[0], v[1], v[2], v[3]};
+                    if (a.epi.nonline != NL_IDENTITY) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[r] = requant_s32_exact(v[r], false, 0, a.epi);
+                    }
+                    *reinterpret_cast<v4i*>(reinterpret_cast<int*>(a.dst) + (int64_t)n * a.dst_sn + in_img) = o;
+                } else {
+                    uint32_t zw = 0;
+                    if (hz) zw = *reinterpret_cast<const uint32_t*>(a.z + (int64_t)n * a.z_sn + in_img);
+                    const uint32_t o = requant4(v[0], v[1], v[2], v[3], zw, a.epi);
+                    *reinterpret_cast<uint32_t*>(a.dst + (int64_t)n * a.dst_sn + in_img) = o;
+                }
+            }
         }
     }
 }

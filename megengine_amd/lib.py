@@ -20,7 +20,7 @@ EXPORTS = [
     "mi355_igemm_tile_count", "mi355_igemm_tile_name", "mi355_epilogue_linear_form",
     "mi355_relayout_deduce", "mi355_relayout_exec", "mi355_requant_s32_s8_exec", "mi355_requant_s8_s8_exec", "mi355_convbias_s8_profile",
     "mi355_pooling_deduce_out", "mi355_pooling_s8_exec", "mi355_typecvt_f32_s8_exec", "mi355_typecvt_s8_f32_exec",
-    "mi355_convbias_s8_preprocess_size", "mi355_convbias_s8_preprocess", "mi355_convbias_s8_exec_preprocessed",
+    "mi355_epilogue_quotient_form", "mi355_convbias_s8_preprocess_size", "mi355_convbias_s8_preprocess", "mi355_convbias_s8_exec_preprocessed",
 ]
 
 
@@ -67,6 +67,8 @@ def lib():
     L.mi355_igemm_tile_count.restype = C.c_int
     L.mi355_igemm_tile_name.restype = C.c_char_p
     L.mi355_igemm_tile_name.argtypes = [C.c_int]
+    L.mi355_epilogue_quotient_form.restype = C.c_int
+    L.mi355_epilogue_quotient_form.argtypes = [C.c_float, P(C.c_float), P(C.c_float)]
     L.mi355_epilogue_linear_form.restype = C.c_int
     L.mi355_epilogue_linear_form.argtypes = [C.c_float, C.c_float, C.c_uint32, P(C.c_float), P(C.c_float)]
     L.mi355_relayout_deduce.argtypes = [P(_abi.RelayoutDesc), P(C.c_uint32), P(C.c_uint32)]

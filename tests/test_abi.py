@@ -98,8 +98,12 @@ def test_query_chooser_and_workspace():
     assert (a.id, ws) == (igemm, 0)
     a, _ = ops.conv_bias_query(_abi.make_conv_desc("NCHW4", 1, 32, 8, 8, 32, 3, pad=1, group=32))
     assert a.id == dw
-    # scales outside the fast epilogue's envelope: MFMA algo is not usable, direct kernel runs it
+    # scales outside the fast epilogue's envelope: 32-packed inputs run the MFMA kernel with its general epilogue
+    # (a second-generation tile), 4-packed inputs the generic kernel
     d = _abi.make_conv_desc("NCHW32", 1, 32, 8, 8, 32, 3, pad=1, scale_dst=1e-30)
+    a, _ = ops.conv_bias_query(d)
+    assert a.id == igemm and lib.tile_names()[a.tile_cfg].startswith("v2_")
+    d = _abi.make_conv_desc("NCHW4", 1, 32, 8, 8, 32, 3, pad=1, scale_dst=1e-30)
     a, _ = ops.conv_bias_query(d)
     assert a.id == 0
     with pytest.raises(lib.Mi355Error) as e:

@@ -310,6 +310,40 @@ def test_heuristic_picks(oracle):
         assert a.id == IGEMM and names[a.tile_cfg] == want, (ic, hw, oc, names[a.tile_cfg])
 
 
+def test_general_epilogue_on_the_mfma_kernel(oracle):
+    """QuantizedS32 dst (the reference's default dst dtype for s8 x s8, dnn/src/common/convolution.cpp:555-574), full-shape
+    bias and scales outside the fast forms' envelope run the MFMA kernel (second-generation tiles) on 32-packed inputs."""
+    names = lib.tile_names()
+    v2 = [i for i, n in enumerate(names) if n.startswith("v2_")]
+    cases = [
+        dict(dst_dtype=_abi.DT_QS32, scale_bias=2e-4, scale_dst=2e-4),
+        dict(dst_dtype=_abi.DT_QS32, nonline="RELU", scale_bias=2e-4, scale_dst=2.0000001e-4),
+        dict(dst_dtype=_abi.DT_QS32, nonline="H_SWISH", scale_bias=2e-4, scale_dst=2e-4),
+        dict(bias_mode=_abi.BIAS_FULL, nonline="RELU", has_z=True, **S),
+        dict(bias_mode=_abi.BIAS_FULL, nonline="IDENTITY", scale_bias=1.3e-3, scale_dst=0.0271),
+        dict(nonline="H_SWISH", has_z=True, scale_bias=2e-4, scale_z=0.05, scale_dst=1e-20),
+        dict(nonline="RELU", scale_bias=2e-4, scale_dst=3e15),
+    ]
+    shapes = [("NCHW32", 2, 64, 9, 11, 96, 3, 1, 1, 1), ("NCHW32", 3, 128, 7, 7, 64, 1, 0, 1, 1), ("NCHW32", 2, 128, 8, 8, 128, 3, 1, 2, 2),
+              ("NCHW32_NCHW4", 2, 64, 8, 8, 24, 3, 1, 1, 1)]
+    for ci, kw in enumerate(cases):
+        for si, (fmt, n, ic, ih, iw, oc, f, pad, stride, group) in enumerate(shapes):
+            if fmt == "NCHW32_NCHW4" and kw.get("has_z"):
+                continue
+            d = _abi.make_conv_desc(fmt, n, ic, ih, iw, oc, f, pad=pad, stride=stride, group=group, **kw)
+            a, _ = ops.conv_bias_query(d)
+            assert a.id == IGEMM and names[a.tile_cfg].startswith("v2_"), (ci, si, names[a.tile_cfg])
+            big = dict(bias_range=(-(1 << 26), 1 << 26)) if kw.get("dst_dtype") == _abi.DT_QS32 else {}
+            check_case(oracle, d, seed=900 + 10 * ci + si, tag="general %d/%d heuristic" % (ci, si), **big)
+            for tile in v2[::3]:
+                check_case(oracle, d, seed=900 + 10 * ci + si, algo=IGEMM, tile=tile, tag="general %d/%d %s" % (ci, si, names[tile]), **big)
+    # QuantizedS32 dst with a residual, and 4-packed inputs, stay on the generic kernel
+    d = _abi.make_conv_desc("NCHW32", 1, 64, 6, 6, 64, 3, pad=1, has_z=True, dst_dtype=_abi.DT_QS32, scale_bias=2e-4, scale_dst=2e-4)
+    assert ops.conv_bias_query(d)[0].id == DIRECT
+    d = _abi.make_conv_desc("NCHW4", 1, 64, 6, 6, 64, 3, pad=1, dst_dtype=_abi.DT_QS32, scale_bias=2e-4, scale_dst=2e-4)
+    assert ops.conv_bias_query(d)[0].id == DIRECT
+
+
 def test_preprocessed_filter_equals_plain_filter(oracle):
     """exec with a PreprocessedFilter == exec with the filter, bit for bit, for every tile that has a pre-processed form;
     tiles without one report size 0 (nothing to hoist) and refuse exec_preprocessed."""
