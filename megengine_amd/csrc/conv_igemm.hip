@@ -522,8 +522,8 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess) {
     const mi355_conv_desc& d = p.d;
     if (will_preprocess && p.pin == 32 && p.pout == 32 && d.group == 1 && !d.has_z) {
         // The caller re-tiles the filter for the chosen algorithm (weight pre-processing): the second-generation tiles
-        // then copy whole kilobytes for both operands and win on the layers without a residual (in-stack sweep of
-        // every tile over the ResNet-50 shapes, plain and pre-processed filters).  Residual layers stay below.
+        // then copy whole kilobytes for both operands and win on the layers without a residual (every tile forced on every ResNet-50 shape in turn, timed as
+        // whole-stack replays of one captured graph against the unchanged stack in the same process).  Residual layers stay below.
         enum { V128x128x64r4 = 0, V64x128x128r3 = 3, V64x128x64r4 = 4, V64x64x128r4 = 8 };
         const int v2 = igemm_first_v2_cfg();
         const int cu = cu_count > 0 ? cu_count : 256;
@@ -531,11 +531,12 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess) {
         const int64_t t128 = ((d.oc + 127) / 128) * ((M + 127) / 128);
         const int kb = (int)(p.icpg * d.fh * d.fw);
         const bool pw = d.fh == 1 && d.fw == 1 && d.pad_h == 0 && d.pad_w == 0;
-        if (d.oc <= 64) return v2 + (pw && kb >= 256 ? V64x128x128r3 : V64x128x64r4);
+        if (d.oc <= 64) return v2 + V64x128x64r4;
         if (t128 >= cu) return v2 + V128x128x64r4;
         if (pw) return v2 + V64x128x128r3;
-        if (d.stride_h == 1 && d.stride_w == 1) return v2 + (kb >= 4608 ? V64x64x128r4 : V64x128x128r3);
-        // few tiles, strided 3x3: the first-generation tiles below
+        if (kb >= 4608) return v2 + V64x64x128r4;
+        if (d.stride_h == 1 && d.stride_w == 1) return v2 + V64x128x128r3;
+        // few tiles, strided 3x3 over at most 256 channels: the first-generation tiles below
     }
     const int64_t M = (int64_t)d.n * p.oh * p.ow;
     const int OC = d.oc;

@@ -342,8 +342,9 @@ struct Igemm2 {
         (f(std::integral_constant<int, C>{}), ...);
     }
 
-    // KT: the reduction is not a whole number of stages
-    template <bool KT>
+    // KT: the reduction is not a whole number of stages.  GEN: the general epilogue (its own instantiations: the fast
+    // epilogue's kernels carry none of its registers)
+    template <bool KT, bool GEN>
     __device__ static __forceinline__ void run(const IgemmArgs& a) {
         extern __shared__ __attribute__((aligned(16))) int8_t lds[];
         int* sBias = reinterpret_cast<int*>(lds + NS * STG);
@@ -581,7 +582,7 @@ struct Igemm2 {
                 read_z(zr, zbuf + zslot * ZSLOT, lane);
                 if (zslots == 2) zslot ^= 1;
             }
-            if (a.general)
+            if constexpr (GEN)
                 igemm_epilogue_general<POUT, MT, NT>(a, acc, cur.oc0 + wm * WTM, cur.pix0 + wn * WTN, l32, lh, cur.oc_end);
             else
                 igemm_run_epilogue<POUT, MT, NT, true>(a, acc, cur.oc0 + wm * WTM, cur.pix0 + wn * WTN, l32, lh, &zr, cur.oc_end);
@@ -603,13 +604,14 @@ struct Igemm2 {
     }
 };
 
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, bool KT>
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, bool KT, bool GEN>
 __global__ __launch_bounds__(WM * WN * 64, MINW) void igemm2_kernel(IgemmArgs a) {
-    Igemm2<POUT, BM, BN, WM, WN, KCH, NS, PW>::template run<KT>(a);
+    Igemm2<POUT, BM, BN, WM, WN, KCH, NS, PW>::template run<KT, GEN>(a);
 }
 
 constexpr int kLdsPerCu = 160 * 1024;
 constexpr int kNoFit = -1;  // not a hipError_t
+constexpr int kNoGen = -2;  // this tile has no instantiation with the general epilogue
 
 struct Cfg2 {
     const char* name;
@@ -633,7 +635,7 @@ const Cfg2 kCfg2[] = {
 };
 constexpr int kNumCfg2 = sizeof(kCfg2) / sizeof(kCfg2[0]);
 
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, bool KT>
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, bool KT, bool GEN>
 int launch_k(hipStream_t st, IgemmArgs& a, int cu_count) {
     using K = Igemm2<POUT, BM, BN, WM, WN, KCH, NS, PW>;
     a.tiles_m_pg = (a.ocpg + BM - 1) / BM;
@@ -656,7 +658,7 @@ int launch_k(hipStream_t st, IgemmArgs& a, int cu_count) {
     }
     const int lds = fixed + a.zslots * K::ZSLOT;
     if (lds > kLdsPerCu) return kNoFit;  // ring + residual slot of this tile do not fit: the caller takes a smaller tile
-    auto kern = igemm2_kernel<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW, KT>;
+    auto kern = igemm2_kernel<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW, KT, GEN>;
     // per-instantiation caches; atomics, because operators on different streams may launch from several threads
     static std::atomic<int> max_lds_set{0};
     if (lds > max_lds_set.load(std::memory_order_relaxed)) {
@@ -685,24 +687,36 @@ int launch_k(hipStream_t st, IgemmArgs& a, int cu_count) {
     return (int)hipGetLastError();
 }
 
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW>
-int launch_one(hipStream_t st, IgemmArgs& a, int cu) {
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool GEN>
+int launch_gen(hipStream_t st, IgemmArgs& a, int cu) {
     const bool pw = a.T == 1 && a.ph == 0 && a.pw == 0;
     const bool kt = a.KC % KCH != 0;
     if (pw)
-        return kt ? launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, true, true>(st, a, cu)
-                  : launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, true, false>(st, a, cu);
+        return kt ? launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, true, true, GEN>(st, a, cu)
+                  : launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, true, false, GEN>(st, a, cu);
     // the k-unit table carries the end of the reduction (padding entries)
-    return launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, false, false>(st, a, cu);
+    return launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, false, false, GEN>(st, a, cu);
+}
+
+// GENOK: the tile is also instantiated with the general epilogue (two tiles are: every general problem runs on one of them)
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool GENOK = false>
+int launch_one(hipStream_t st, IgemmArgs& a, int cu) {
+    if (a.general) {
+        if constexpr (GENOK)
+            return launch_gen<POUT, BM, BN, WM, WN, KCH, NS, MINW, true>(st, a, cu);
+        else
+            return kNoGen;
+    }
+    return launch_gen<POUT, BM, BN, WM, WN, KCH, NS, MINW, false>(st, a, cu);
 }
 
 template <int POUT>
 int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
     switch (cfg) {
-        case 0: return launch_one<POUT, 128, 128, 2, 2, 2, 4, 2>(st, a, cu);
+        case 0: return launch_one<POUT, 128, 128, 2, 2, 2, 4, 2, true>(st, a, cu);
         case 1: return launch_one<POUT, 128, 128, 2, 2, 2, 3, 2>(st, a, cu);
         case 2: return launch_one<POUT, 128, 128, 2, 2, 4, 3, 1>(st, a, cu);
-        case 3: return launch_one<POUT, 64, 128, 2, 2, 4, 3, 2>(st, a, cu);
+        case 3: return launch_one<POUT, 64, 128, 2, 2, 4, 3, 2, true>(st, a, cu);
         case 4: return launch_one<POUT, 64, 128, 2, 2, 2, 4, 2>(st, a, cu);
         case 5: return launch_one<POUT, 128, 64, 2, 2, 4, 3, 2>(st, a, cu);
         case 6: return launch_one<POUT, 128, 64, 2, 2, 2, 4, 2>(st, a, cu);
@@ -757,6 +771,11 @@ int launch_igemm2_preprocess(hipStream_t st, const int8_t* flt, int8_t* out, int
 
 int launch_igemm2(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count) {
     int rc = pout == 32 ? launch_fmt<32>(st, a, cfg, cu_count) : launch_fmt<4>(st, a, cfg, cu_count);
+    // the general epilogue exists on two tiles: the one with the asked tile's channel count, or the smaller one
+    if (rc == kNoGen) {
+        cfg = kCfg2[cfg].bm <= 64 ? 3 : 0;
+        rc = pout == 32 ? launch_fmt<32>(st, a, cfg, cu_count) : launch_fmt<4>(st, a, cfg, cu_count);
+    }
     // the large tiles with a residual need more LDS than a CU has: 128 x 128 x 64 with a ring of three always fits
     if (rc == kNoFit) rc = pout == 32 ? launch_fmt<32>(st, a, 1, cu_count) : launch_fmt<4>(st, a, 1, cu_count);
     return rc == kNoFit ? (int)hipErrorInvalidValue : rc;
