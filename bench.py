@@ -318,7 +318,8 @@ def run_extras(torch, np, _abi, lib, ops, workloads, side_iters=50):
         rows = []
         workloads.choose_algorithms(plan)
         # pre-marshalled launches: the per-call Python work of conv_bias_exec would floor short kernels
-        for p, call in zip(plan, workloads.bind_plan(plan)):
+        calls = workloads.bind_plan(plan)
+        for p, call in zip(plan, calls):
             t = time_launches(torch, call, iters=side_iters)
             tc = time_launches_cold(torch, call, iters=max(3, min(8, side_iters)))
             l = p["layer"]
@@ -326,15 +327,15 @@ def run_extras(torch, np, _abi, lib, ops, workloads, side_iters=50):
             rows.append(dict(name=l.name, algo=lib.algo_names()[p["algo"].id], us=round(t * 1e6, 2),
                              us_cold=round(tc * 1e6, 2), tops=round(l.ops / t / 1e12, 1), gbs=round(l.bytes / t / 1e9, 1),
                              frac_roof=round(roof / t, 3), frac_roof_cold=round(roof / tc, 3)))
-        return rows, plan
+        return rows, plan, calls
 
-    rows, _ = measure([workloads.config0()], 1)
+    rows, _, _ = measure([workloads.config0()], 1)
     res["config0"] = rows[0]
-    rows, _ = measure(workloads.pointwise_sweep(), 2)
+    rows, _, _ = measure(workloads.pointwise_sweep(), 2)
     res["config1_pointwise"] = rows
     torch.cuda.empty_cache()
     mb = workloads.mobilenet_v2()
-    rows, _ = measure(mb, 3)
+    rows, _, _ = measure(mb, 3)
     dw = [(r, l) for r, l in zip(rows, mb) if l.group > 1]
     pw = [(r, l) for r, l in zip(rows, mb) if l.group == 1]
     t_dw = sum(r["us"] for r, _ in dw) * 1e-6
@@ -353,8 +354,8 @@ def run_extras(torch, np, _abi, lib, ops, workloads, side_iters=50):
     torch.cuda.empty_cache()
     c4 = []
     for l in workloads.large_hswish():
-        rows, plan = measure([l], 4)
-        p = plan[0]
+        rows, plan, calls = measure([l], 4)
+        p, conv = plan[0], calls[0]
         # NCHW -> NCHW32 relayout of the input and NCHW32 -> NCHW of the output, timed with the conv
         x_nchw = torch.randint(-128, 128, (l.n, l.ic, l.ih, l.iw), dtype=torch.int8, device="cuda")
         y_nchw = torch.empty((l.n, l.oc, l.oh, l.ow), dtype=torch.int8, device="cuda")
@@ -363,7 +364,7 @@ def run_extras(torch, np, _abi, lib, ops, workloads, side_iters=50):
 
         def full():
             ops.relayout_exec(d_in, x_nchw, p["src"])
-            ops.conv_bias_exec(p["desc"], p["src"], p["flt"], p["bias"], p["z"], dst=p["dst"], algo=p["algo"])
+            conv()  # the heuristic's algorithm, with its pre-processed filter where it has one
             ops.relayout_exec(d_out, p["dst"], y_nchw)
 
         n10 = max(2, min(10, side_iters))

@@ -520,23 +520,32 @@ bool igemm_usable(const ConvProblem& p) {
 
 int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess) {
     const mi355_conv_desc& d = p.d;
-    if (will_preprocess && p.pin == 32 && p.pout == 32 && d.group == 1 && !d.has_z) {
+    if (will_preprocess && p.pin == 32 && p.pout == 32 && d.group == 1 && !igemm_needs_general(p)) {
         // The caller re-tiles the filter for the chosen algorithm (weight pre-processing): the second-generation tiles
-        // then copy whole kilobytes for both operands and win on the layers without a residual (every tile forced on every ResNet-50 shape in turn, timed as
-        // whole-stack replays of one captured graph against the unchanged stack in the same process).  Residual layers stay below.
-        enum { V128x128x64r4 = 0, V64x128x128r3 = 3, V64x128x64r4 = 4, V64x64x128r4 = 8 };
+        // then copy whole kilobytes for both operands.  Every tile was forced on every ResNet-50 shape in turn and timed
+        // as whole-stack replays of one captured graph, against the unchanged stack in the same process.
+        enum { V128x128x64r4 = 0, V64x128x128r3 = 3, V64x128x64r4 = 4, V64x64x128r4 = 8, V128x256x64w8 = 10, V256x256x64w8 = 11 };
         const int v2 = igemm_first_v2_cfg();
         const int cu = cu_count > 0 ? cu_count : 256;
         const int64_t M = (int64_t)d.n * p.oh * p.ow;
         const int64_t t128 = ((d.oc + 127) / 128) * ((M + 127) / 128);
         const int kb = (int)(p.icpg * d.fh * d.fw);
         const bool pw = d.fh == 1 && d.fw == 1 && d.pad_h == 0 && d.pad_w == 0;
-        if (d.oc <= 64) return v2 + V64x128x64r4;
-        if (t128 >= cu) return v2 + V128x128x64r4;
-        if (pw) return v2 + V64x128x128r3;
-        if (kb >= 4608) return v2 + V64x64x128r4;
-        if (d.stride_h == 1 && d.stride_w == 1) return v2 + V64x128x128r3;
-        // few tiles, strided 3x3 over at most 256 channels: the first-generation tiles below
+        // Large convolutions (six and more 128 x 128 tiles per CU, long reductions), with or without a residual: the
+        // 8-wave tiles of 256 rows or columns, which read a residual in the epilogue instead of staging it in LDS
+        // (1.8 / 2.2 / 2.1 Pop/s against 1.5 / 1.9 / 1.9 on the first-generation tiles for 3x3 256->256 at 64x64, 3x3
+        // stride 2 512->1024 at 32x32 and 5x5 128->128 at 80x80, batch 128, residual + H_SWISH).
+        if (t128 >= 6 * (int64_t)cu && kb >= 1024 && d.oc > 64) return v2 + (d.oc >= 256 ? V256x256x64w8 : V128x256x64w8);
+        if (!d.has_z) {
+            // the layers without a residual; the others stay on the first-generation tiles below, where the residual
+            // costs no LDS
+            if (d.oc <= 64) return v2 + V64x128x64r4;
+            if (t128 >= cu) return v2 + V128x128x64r4;
+            if (pw) return v2 + V64x128x128r3;
+            if (kb >= 4608) return v2 + V64x64x128r4;
+            if (d.stride_h == 1 && d.stride_w == 1) return v2 + V64x128x128r3;
+            // few tiles, strided 3x3 over at most 256 channels: the first-generation tiles below
+        }
     }
     const int64_t M = (int64_t)d.n * p.oh * p.ow;
     const int OC = d.oc;

@@ -50,6 +50,10 @@ struct Igemm2 {
     static constexpr int RB = NBB >= NW ? NBB / NW : 1;
     static constexpr int BIAS_BYTES = BM * 4;
     static constexpr int RING_BYTES = NS * STG + BIAS_BYTES;
+    // The 8-wave tiles of 256 x 128 outputs and more read the residual in the epilogue, straight from global memory:
+    // an LDS slot for it (BM * BN bytes) would cost them a workgroup per CU, and a tile of theirs runs long enough to
+    // hide the fetch of one block behind the requantisation of the previous one.
+    static constexpr bool ZD = BM * BN >= 256 * 128;
     static_assert(NW == 4 || NW == 8, "4 or 8 waves");
     static_assert(MT >= 1 && NT >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "wave tile");
     static_assert((KCH * NBA) % NW == 0 && (KCH * NBB) % NW == 0, "copies divide over the waves");
@@ -349,7 +353,7 @@ struct Igemm2 {
         extern __shared__ __attribute__((aligned(16))) int8_t lds[];
         int* sBias = reinterpret_cast<int*>(lds + NS * STG);
         // [ring][bias][residual slots, only for launches with a residual][k-unit table]
-        const int zslots = a.zslots;
+        const int zslots = ZD ? 0 : a.zslots;
         KEntry* tab = reinterpret_cast<KEntry*>(lds + RING_BYTES + zslots * ZSLOT);
         const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)lds);
 
@@ -584,6 +588,8 @@ struct Igemm2 {
             }
             if constexpr (GEN)
                 igemm_epilogue_general<POUT, MT, NT>(a, acc, cur.oc0 + wm * WTM, cur.pix0 + wn * WTN, l32, lh, cur.oc_end);
+            else if constexpr (ZD)
+                igemm_run_epilogue<POUT, MT, NT, false>(a, acc, cur.oc0 + wm * WTM, cur.pix0 + wn * WTN, l32, lh, nullptr, cur.oc_end);
             else
                 igemm_run_epilogue<POUT, MT, NT, true>(a, acc, cur.oc0 + wm * WTM, cur.pix0 + wn * WTN, l32, lh, &zr, cur.oc_end);
             c_tile += step;
@@ -652,7 +658,7 @@ int launch_k(hipStream_t st, IgemmArgs& a, int cu_count) {
     // tile to hide it behind (one slot, and room for a second workgroup per CU)
     const int fixed = K::RING_BYTES + tab_entries * 8;
     a.zslots = 0;
-    if (a.epi.has_z && !a.general) {
+    if (a.epi.has_z && !a.general && !K::ZD) {
         a.zslots = a.nstages <= 2 ? 2 : 1;
         if (fixed + a.zslots * K::ZSLOT > kLdsPerCu) a.zslots = 1;
     }

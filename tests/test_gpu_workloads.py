@@ -176,9 +176,20 @@ def test_config4_chain_at_batch_128(oracle, case):
     bias = torch.randint(-1000, 1001, bs, dtype=torch.int32, device="cuda", generator=g)
     z = torch.randint(-128, 128, ds, dtype=torch.int8, device="cuda", generator=g)
     src32 = ops.relayout_exec(ops.relayout_desc(_abi.RL_NCHW_NCHW32, tuple(x_nchw.shape)), x_nchw)
-    algo, _ = ops.conv_bias_query(d)
+    # what the bench launches: the heuristic for a caller that pre-processes weights (the 8-wave second-generation tiles,
+    # which read the residual in the epilogue), exec with the PreprocessedFilter
+    algo, _ = ops.conv_bias_query(d, _abi.ALGO_HEURISTIC_PREPROCESS)
     assert algo.id == IGEMM
-    dst32 = ops.conv_bias_exec(d, src32, flt, bias, z, algo=algo)
+    tile = lib.tile_names()[algo.tile_cfg]
+    say("tile", tile)
+    assert tile in ("v2_256x256x64r3w8", "v2_128x256x64r3w8")
+    pre = ops.conv_bias_preprocess(d, flt, algo)
+    assert pre is not None
+    dst32 = ops.conv_bias_exec_preprocessed(d, src32, pre, bias, z, algo=algo)
+    # ... and the choice of a caller that hands over the filter as it is
+    plain_algo, _ = ops.conv_bias_query(d)
+    assert plain_algo.id == IGEMM
+    dst_plain = ops.conv_bias_exec(d, src32, flt, bias, z, algo=plain_algo)
     y_nchw = ops.relayout_exec(ops.relayout_desc(_abi.RL_NCHW32_NCHW, tuple(dst32.shape)), dst32)
     torch.cuda.synchronize()
     assert tuple(y_nchw.shape) == (l.n, l.oc, l.oh, l.ow)
@@ -202,5 +213,6 @@ def test_config4_chain_at_batch_128(oracle, case):
     ref = ops.conv_bias_exec(d, src32, flt, bias, z, algo=DIRECT)
     torch.cuda.synchronize()
     assert torch.equal(dst32, ref)
-    del x_nchw, src32, dst32, y_nchw, ref, z
+    assert torch.equal(dst_plain, ref)
+    del x_nchw, src32, dst32, dst_plain, y_nchw, ref, z
     torch.cuda.empty_cache()
