@@ -582,6 +582,9 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess) {
         };
         if (OC <= 64) return kbytes <= 64 ? D128x128x64w8 : kbytes <= 256 ? D64x64x128r2 : D64x128x128r2;
         const int64_t t128 = tiles(0);
+        // layers with a residual and a short reduction (the expanding 1x1 of a bottleneck block) are bound by their
+        // epilogue: three 8-wave workgroups per CU at every size (whole-stack graph replays, each tile in turn)
+        if (d.has_z && kbytes <= 512 && t128 >= cu_count) return D128x128x64w8;
         if (t128 >= 4 * cu_count)
             return kbytes >= 1024 ? (OC >= 256 ? D256x128x64w8 : D128x128x128r2) : (kbytes <= 128 ? D128x128x64w8 : D128x128x128r2w8);
         if (t128 >= 2 * cu_count) return D128x64x128r2;
