@@ -91,8 +91,8 @@ struct Igemm2 {
 
     __device__ static __forceinline__ Tile tile_coords(const IgemmArgs& a, int tile) {
         Tile c;
-        const int tn = tile / a.tiles_m, tmg = tile - tn * a.tiles_m;
-        const int g = tmg / a.tiles_m_pg, tm = tmg - g * a.tiles_m_pg;
+        const int tn = (int)fdiv((uint32_t)tile, a.div_tiles_m), tmg = tile - tn * a.tiles_m;
+        const int g = (int)fdiv((uint32_t)tmg, a.div_tiles_m_pg), tm = tmg - g * a.tiles_m_pg;
         c.oc0 = g * a.ocpg + tm * BM;
         c.oc_end = (g + 1) * a.ocpg;
         c.pix0 = tn * BN;
@@ -100,8 +100,7 @@ struct Igemm2 {
         return c;
     }
 
-    __device__ static __forceinline__ void loader_enter_tile(const IgemmArgs& a, Loader& L, int tile, int w, int lane) {
-        const Tile c = tile_coords(a, tile);
+    __device__ static __forceinline__ void loader_enter_tile(const IgemmArgs& a, Loader& L, const Tile& c, int w, int lane) {
         const int rib = 16 * (lane >> 5) + (lane & 15);  // row inside a block
         const int half = (lane >> 4) & 1;
         int a_base[RA];
@@ -350,6 +349,17 @@ struct Igemm2 {
     // epilogue's kernels carry none of its registers)
     template <bool KT, bool GEN>
     __device__ static __forceinline__ void run(const IgemmArgs& a) {
+        // Every kernel argument that the path to the first copy reads is requested here, in one batch of scalar loads:
+        // left to itself the compiler fetches them where they are first used, behind branches, which made four
+        // dependent round trips to the argument segment (~500 clocks each) out of the first 2000 clocks of a workgroup.
+        asm volatile("" ::"s"(a.src), "s"(a.flt), "s"(a.bias), "s"(a.src_bytes), "s"(a.flt_bytes), "s"(a.M), "s"(a.OC),
+                     "s"(a.tiles), "s"(a.tiles_m), "s"(a.tiles_m_pg), "s"(a.nstages), "s"(a.KC), "s"(a.src_sn), "s"(a.src_scb),
+                     "s"(a.flt_rstride), "s"(a.flt_kstride), "s"(a.OHW), "s"(a.OW), "s"(a.IW), "s"(a.IH), "s"(a.sh), "s"(a.sw),
+                     "s"(a.ph), "s"(a.pw), "s"(a.ocpg), "s"(a.src_sg), "s"(a.has_bias), "s"(a.zslots), "s"(a.entries));
+        asm volatile("" ::"s"(a.div_ohw.m), "s"(a.div_ohw.s1), "s"(a.div_ohw.s2), "s"(a.div_ow.m), "s"(a.div_ow.s1),
+                     "s"(a.div_ow.s2), "s"(a.div_tiles_m.m), "s"(a.div_tiles_m.s1), "s"(a.div_tiles_m.s2),
+                     "s"(a.div_tiles_m_pg.m), "s"(a.div_tiles_m_pg.s1), "s"(a.div_tiles_m_pg.s2), "s"(a.div_step.m),
+                     "s"(a.div_step.s1), "s"(a.div_step.s2), "s"(a.z), "s"(a.z_bytes), "s"(a.epi.has_z));
         extern __shared__ __attribute__((aligned(16))) int8_t lds[];
         int* sBias = reinterpret_cast<int*>(lds + NS * STG);
         // [ring][bias][residual slots, only for launches with a residual][k-unit table]
@@ -378,7 +388,7 @@ struct Igemm2 {
                 first = b; step = G; last = a.tiles;
             }
         }
-        const int my_tiles = first < last ? (last - first + step - 1) / step : 0;
+        const int my_tiles = first < last ? (int)fdiv((uint32_t)(last - first + step - 1), a.div_step) : 0;
         if (my_tiles == 0) return;  // workgroup-uniform
         const int nst = a.nstages;
 
@@ -418,7 +428,7 @@ struct Igemm2 {
         L.kc0 = 0;
         L.kA = 0;
         L.kB = 0;
-        loader_enter_tile(a, L, first, wave, lane);
+        loader_enter_tile(a, L, cur, wave, lane);
         // after a stage was issued: the general step, which may move on to the workgroup's next tile or past its last
         auto advance = [&]() __attribute__((always_inline)) {
             L.kc0 += KCH;
@@ -430,7 +440,7 @@ struct Igemm2 {
                 L.kA = 0;
                 L.kB = 0;
                 if (++L.ti < my_tiles)
-                    loader_enter_tile(a, L, first + L.ti * step, wave, lane);
+                    loader_enter_tile(a, L, tile_coords(a, first + L.ti * step), wave, lane);
                 else
                     loader_kill(L);
             }
@@ -646,6 +656,8 @@ int launch_k(hipStream_t st, IgemmArgs& a, int cu_count) {
     using K = Igemm2<POUT, BM, BN, WM, WN, KCH, NS, PW>;
     a.tiles_m_pg = (a.ocpg + BM - 1) / BM;
     a.tiles_m = a.tiles_m_pg * a.groups;
+    a.div_tiles_m = make_fastdiv((uint32_t)a.tiles_m);
+    a.div_tiles_m_pg = make_fastdiv((uint32_t)a.tiles_m_pg);
     a.tiles_n = (a.M + BN - 1) / BN;
     const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
     if (tiles <= 0 || tiles > 0x3fffffff) return (int)hipErrorInvalidValue;
@@ -689,6 +701,7 @@ int launch_k(hipStream_t st, IgemmArgs& a, int cu_count) {
     int64_t grid = (int64_t)occ * cu_count;
     if (grid > tiles) grid = tiles;
     if (grid >= 8) grid &= ~(int64_t)7;
+    a.div_step = make_fastdiv((uint32_t)((grid & 7) == 0 ? grid >> 3 : grid));  // the kernel's tile stride
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(K::THREADS), lds, st, a);
     return (int)hipGetLastError();
 }

@@ -71,7 +71,7 @@ struct DmaKernel {
     };
 
     __device__ static __forceinline__ void tile_coords(const IgemmArgs& a, int tile, int& oc0, int& pix0) {
-        const int tn = tile / a.tiles_m, tm = tile - tn * a.tiles_m;
+        const int tn = (int)fdiv((uint32_t)tile, a.div_tiles_m), tm = tile - tn * a.tiles_m;
         oc0 = tm * BM;
         pix0 = tn * BN;
     }
@@ -220,7 +220,7 @@ struct DmaKernel {
                 first = b; step = G; last = a.tiles;
             }
         }
-        const int my_tiles = first < last ? (last - first + step - 1) / step : 0;
+        const int my_tiles = first < last ? (int)fdiv((uint32_t)(last - first + step - 1), a.div_step) : 0;
         const int total = my_tiles * a.nstages;
 
         // The bias of the workgroup's channel tile lives in LDS, written once after the prologue's copies are issued: workgroups
@@ -448,6 +448,7 @@ template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, b
 int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
     using K = DmaKernel<POUT, BM, BN, WM, WN, KCH, NS, PW, PIN>;
     a.tiles_m = (a.OC + BM - 1) / BM;
+    a.div_tiles_m = make_fastdiv((uint32_t)a.tiles_m);
     a.tiles_n = (a.M + BN - 1) / BN;
     const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
     if (tiles <= 0 || tiles > 0x3fffffff) return (int)hipErrorInvalidValue;
@@ -481,6 +482,7 @@ int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
     int64_t grid = (int64_t)occ * cu_count;
     if (grid > tiles) grid = tiles;
     if (grid >= 8) grid &= ~(int64_t)7;
+    a.div_step = make_fastdiv((uint32_t)((grid & 7) == 0 ? grid >> 3 : grid));  // the kernel's tile stride
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(K::THREADS), lds, st, a);
     return (int)hipGetLastError();
 }

@@ -44,6 +44,10 @@ struct IgemmArgs {
     // general epilogue (second-generation kernel): QuantizedS32 dst, full-shape bias, or scales outside the fast
     // forms' envelope.  bias_full: a.bias has the shape of dst (contiguous) and has_bias is 0.
     int general, dst_s32, bias_full;
+    // tile decoding of the LDS-direct kernels without run-time integer divisions (each costs ~30 scalar instructions and a
+    // reciprocal on the critical path from kernel entry to the first copy): by the number of channel tiles, by the
+    // channel tiles of a group, and by the tile stride of a workgroup (set by the launch code, which knows the grid)
+    FastDiv div_tiles_m, div_tiles_m_pg, div_step;
 };
 
 struct KEntry {
