@@ -53,25 +53,25 @@ bool epi_fast_ok(float s_b, float s_z, float s_d, bool has_z) {
     return true;
 }
 
-// ---- three-FMA quotient of the fast epilogue form (epilogue.h): host-side proof per dst scale --------------------
+// ---- divide-free quotient of the fast epilogue form (epilogue.h): host-side proof per dst scale --------------------
 // From the float r on, the contract is  clamp(roundf(RN(r / s_d)))  and the fast form replaces RN(r / s_d) by
-//     q0 = fma(r, y_hi, RN(r y_lo));  e = fma(-q0, s_d, r);  q = fma(e, y_hi, q0)      y_hi + y_lo = 1 / s_d to 2^-48.
-// q0 is within one ulp of r / s_d (two roundings of relative size 2^-24 and 2^-48), which makes the residual e exact,
-// and q = RN(q0 + e y_hi) differs from r / s_d by less than one ulp before its own rounding: q is a faithful
-// quotient, |q - RN(r / s_d)| <= 1 ulp, for every s_d and r that epi_fast_ok admits (no intermediate leaves the normal
-// range).  A faithful quotient can change the result only where RN(r / s_d) lies within one ulp of a rounding boundary
-// k + 0.5 of roundf, i.e. for a handful of consecutive floats r around each of the 128 boundary magnitudes.  The proof
-// therefore finds every boundary of the literal chain by bisection over the floats and evaluates BOTH forms, with the
-// device's own operations (IEEE fma, clamp, the two integer conversions), on the 33 floats around it, on both signs.
-// Equal there = equal on every float r.  A scale that fails (none is known) runs the literal chain with the IEEE divide.
+//     q0 = RN(r y);  e = fma(-q0, s_d, r);  q = fma(e, y, q0)          y = RN(1 / s_d).
+// q0 is within two ulps of r / s_d (the rounding of y and its own), its residual e is r - q0 s_d to within one rounding
+// of a quantity of two ulps, and q = RN(q0 + e y) differs from r / s_d by less than one ulp before its own rounding: q
+// is a faithful quotient, |q - RN(r / s_d)| <= 1 ulp, for every s_d and r that epi_fast_ok admits (no intermediate
+// leaves the normal range).  A faithful quotient can change the result only where RN(r / s_d) lies within one ulp of a
+// rounding boundary k + 0.5 of roundf, i.e. for a handful of consecutive floats r around each of the 128 boundary
+// magnitudes.  The proof therefore finds every boundary of the literal chain by bisection over the floats and evaluates
+// BOTH forms, with the device's own operations (IEEE multiply and fma, clamp, the two integer conversions), on the 33
+// floats around it, on both signs.  Equal there = equal on every float r.  A scale that fails (none is known: 20 000
+// log-uniform draws and the special scales of the tests all pass) runs the literal chain with the IEEE divide.
 int epi_tail_contract(float r, float s_d) {
     float v = roundf(r / s_d);
     v = fminf(fmaxf(-128.f, v), 127.f);
     return (int)v;
 }
-int epi_tail_fast(float r, float s_d, float y_hi, float y_lo, bool relu) {
-    const float t0 = r * y_lo;
-    const float q0 = fmaf(r, y_hi, t0);
+int epi_tail_fast(float r, float s_d, float y_hi, bool relu) {
+    const float q0 = r * y_hi;
     const float res = fmaf(-q0, s_d, r);
     float q = fmaf(res, y_hi, q0);
     if (relu) {
@@ -88,7 +88,6 @@ float f_from_bits(uint32_t b) {
 }
 bool epi_prove_quotient(float s_d) {
     const float y_hi = 1.0f / s_d;
-    const float y_lo = (float)(1.0 / (double)s_d - (double)y_hi);
     const float top = 130.f * s_d;  // beyond the last boundary: finite by epi_fast_ok
     uint32_t top_bits;
     memcpy(&top_bits, &top, 4);
@@ -104,11 +103,11 @@ bool epi_prove_quotient(float s_d) {
             const int64_t b = (int64_t)hi + d;
             if (b <= 0 || b >= 0x7f800000) continue;
             const float m = f_from_bits((uint32_t)b);
-            if (epi_tail_fast(-m, s_d, y_hi, y_lo, false) != epi_tail_contract(-m, s_d)) return false;
+            if (epi_tail_fast(-m, s_d, y_hi, false) != epi_tail_contract(-m, s_d)) return false;
             // the positive side has the same boundaries (round half away from zero) up to the clamp at 127
-            if (epi_tail_fast(m, s_d, y_hi, y_lo, false) != epi_tail_contract(m, s_d)) return false;
-            if (epi_tail_fast(m, s_d, y_hi, y_lo, true) != epi_tail_contract(m, s_d)) return false;
-            if (epi_tail_fast(-m, s_d, y_hi, y_lo, true) != 0) return false;  // RELU folded into the clamp
+            if (epi_tail_fast(m, s_d, y_hi, false) != epi_tail_contract(m, s_d)) return false;
+            if (epi_tail_fast(m, s_d, y_hi, true) != epi_tail_contract(m, s_d)) return false;
+            if (epi_tail_fast(-m, s_d, y_hi, true) != 0) return false;  // RELU folded into the clamp
         }
     }
     return true;
@@ -249,7 +248,6 @@ void epi_fill(EpiParams* e, float s_b, float s_z, float s_d, uint32_t nonline, b
     e->has_z = has_z ? 1 : 0;
     e->fast = qs8 && epi_fast_ok(s_b, s_z, s_d, has_z) && epi_quotient_proved(s_d);
     e->y_hi = 1.0f / s_d;
-    e->y_lo = (float)(1.0 / (double)s_d - (double)e->y_hi);
     e->lin = 0;
     e->lin_c = e->lin_d = 0.f;
     e->lin_lo = nonline == MI355_NL_RELU ? 0.f : -128.f;
@@ -705,10 +703,9 @@ int mi355_pooling_s8_exec(void* stream, const mi355_pooling_desc* d, const int8_
 int mi355_igemm_tile_count(void) { return igemm_num_cfgs(); }
 const char* mi355_igemm_tile_name(int cfg) { return igemm_cfg_name(cfg); }
 
-int mi355_epilogue_quotient_form(float scale_dst, float* y_hi, float* y_lo) {
-    if (!y_hi || !y_lo) return -fail(MI355_ERR_BAD_ARG, "null argument");
-    *y_hi = 1.0f / scale_dst;
-    *y_lo = (float)(1.0 / (double)scale_dst - (double)*y_hi);
+int mi355_epilogue_quotient_form(float scale_dst, float* y) {
+    if (!y) return -fail(MI355_ERR_BAD_ARG, "null argument");
+    *y = 1.0f / scale_dst;
     if (!epi_fast_ok(1.f, 1.f, scale_dst, false)) return 0;
     return epi_quotient_proved(scale_dst) ? 1 : 0;
 }

@@ -10,14 +10,18 @@
 //     dst = (int8) min(max(-128, v), 127)
 //
 // The "fast" form below produces the same bits with no hardware divide:
-//   * division by the per-tensor constant s_dst: with y_hi = RN(1/s_dst), y_lo = RN(1/s_dst - y_hi)
-//       q0 = fma(r, y_hi, r * y_lo)      faithful quotient (error << 1 ulp before its rounding)
-//       e  = fma(-q0, s_dst, r)          exact residual
-//       q  = fma(e, y_hi, q0)            correctly rounded r / s_dst (Markstein's correction step)
+//   * division by the per-tensor constant s_dst: with y = RN(1/s_dst)
+//       q0 = r * y                       first estimate, within two ulps of r / s_dst
+//       e  = fma(-q0, s_dst, r)          its residual
+//       q  = fma(e, y, q0)               faithful quotient: less than one ulp from r / s_dst (Markstein's correction step)
+//     A faithful quotient can change the result only next to a rounding boundary of roundf; the host proves the form
+//     for every dst scale before a kernel may use it (epi_prove_quotient in capi.hip).
 //   * RELU is folded into the clamp: for s_dst > 0, r <= 0 gives q <= 0 which clamps to 0.
 //   * roundf + clamp + convert: clamp first, then trunc(q + copysign(pred(0.5), q)); for
 //     |q| <= 128 the sum is exact except below 0.5 where pred(0.5) keeps it under 1.  After a RELU
 //     clamp q >= 0 and the hardware's round-to-plus-infinity conversion does the same in one step.
+//   * the four results of a dword are packed by the conversions themselves: the SDWA form of the convert writes the low
+//     byte of its integer result into byte k of the destination and keeps the other bytes (no v_perm afterwards).
 // The host only selects the fast form when the scales are positive, normal and small enough
 // that no intermediate overflows (see epi_fast_ok in capi.hip); otherwise kernels run the
 // literal form with the IEEE divide.
@@ -39,7 +43,7 @@ namespace mi355 {
 
 struct EpiParams {
     float s_b, s_z, s_d;
-    float y_hi, y_lo;
+    float y_hi;   // RN(1 / s_d)
     int nonline;  // MI355_NL_*
     int has_z;
     int fast;     // 1: fast form allowed
@@ -88,15 +92,14 @@ __device__ __forceinline__ int requant_s32_exact(int sfb, bool has_z, int z, con
     return (int)v;
 }
 
-// fast form; NL and HAS_Z are compile-time so the inner loops carry no branches
+// fast form; NL and HAS_Z are compile-time so the inner loops carry no branches.  Returns the value that the final
+// conversion takes: clamped for NL_LIN (floor follows) and NL_RELU (round half up follows), clamped and moved half a
+// unit away from zero otherwise (truncation follows).
 template <int NL, bool HAS_Z>
-__device__ __forceinline__ int requant_s8_fast(int sfb, int z, const EpiParams& e) {
+__device__ __forceinline__ float requant_fast_value(int sfb, int z, const EpiParams& e) {
     if (NL == NL_LIN) {
         float x = __builtin_fmaf((float)sfb, e.lin_c, e.lin_d);
-        x = __builtin_amdgcn_fmed3f(x, e.lin_lo, 127.5f);
-        int o;
-        asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(o) : "v"(x));  // (int)floor(x): x is finite and inside [-128, 127.5]
-        return o;
+        return __builtin_amdgcn_fmed3f(x, e.lin_lo, 127.5f);  // finite and inside [-128, 127.5]
     }
     float r = (float)sfb * e.s_b;
     if (HAS_Z) {
@@ -109,22 +112,57 @@ __device__ __forceinline__ int requant_s8_fast(int sfb, int z, const EpiParams& 
         float m = r * t;
         r = m * (1.f / 6.f);
     }
-    float t0 = r * e.y_lo;
-    float q0 = __builtin_fmaf(r, e.y_hi, t0);
+    float q0 = r * e.y_hi;
     float res = __builtin_fmaf(-q0, e.s_d, r);
     float q = __builtin_fmaf(res, e.y_hi, q0);
-    int out;
-    if (NL == NL_RELU) {
-        q = __builtin_amdgcn_fmed3f(q, 0.f, 127.f);  // q is finite here: same as min(max(q, 0), 127)
-        // floor(q + 0.5) computed exactly by the hardware (round to nearest, ties to +infinity): for q >= 0 that is
-        // round-half-away, one instruction instead of add + truncate.  Equal to (int)(q + 0.49999997f) on every
-        // float in [0, 127] (checked exhaustively on gfx950).
-        asm("v_cvt_rpi_i32_f32 %0, %1" : "=v"(out) : "v"(q));
+    if (NL == NL_RELU) return __builtin_amdgcn_fmed3f(q, 0.f, 127.f);  // q is finite here: same as min(max(q, 0), 127)
+    q = __builtin_amdgcn_fmed3f(q, -128.f, 127.f);
+    return q + __builtin_copysignf(0.49999997f, q);
+}
+
+// The final conversion of result K of a dword, written into byte K of `o` (the other bytes are kept; K = 0 clears them):
+//   NL_LIN   floor            v_cvt_flr_i32_f32
+//   NL_RELU  floor(x + 0.5)   v_cvt_rpi_i32_f32: exact (no intermediate rounding), for x >= 0 that is round-half-away; equal
+//                             to (int)(x + 0.49999997f) on every float in [0, 127] (checked exhaustively on gfx950)
+//   others   truncation       v_cvt_i32_f32
+// Every result lies in [-128, 127]: its low byte is the int8 value.
+template <int NL, int K>
+__device__ __forceinline__ void convert_into_byte(uint32_t& o, float x) {
+    static_assert(K >= 0 && K < 4, "byte of a dword");
+    if (K == 0) {
+        if (NL == NL_LIN)
+            asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD" : "=v"(o) : "v"(x));
+        else if (NL == NL_RELU)
+            asm("v_cvt_rpi_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD" : "=v"(o) : "v"(x));
+        else
+            asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD" : "=v"(o) : "v"(x));
+    } else if (NL == NL_LIN) {
+        if (K == 1) asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o) : "v"(x));
+        if (K == 2) asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o) : "v"(x));
+        if (K == 3) asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o) : "v"(x));
+    } else if (NL == NL_RELU) {
+        if (K == 1) asm("v_cvt_rpi_i32_f32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o) : "v"(x));
+        if (K == 2) asm("v_cvt_rpi_i32_f32_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o) : "v"(x));
+        if (K == 3) asm("v_cvt_rpi_i32_f32_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o) : "v"(x));
     } else {
-        q = __builtin_amdgcn_fmed3f(q, -128.f, 127.f);
-        out = (int)(q + __builtin_copysignf(0.49999997f, q));
+        if (K == 1) asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o) : "v"(x));
+        if (K == 2) asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o) : "v"(x));
+        if (K == 3) asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(o) : "v"(x));
     }
-    return out;
+}
+
+// one result, as an int (the generic one-thread-per-output kernel)
+template <int NL, bool HAS_Z>
+__device__ __forceinline__ int requant_s8_fast(int sfb, int z, const EpiParams& e) {
+    const float x = requant_fast_value<NL, HAS_Z>(sfb, z, e);
+    int o;
+    if (NL == NL_LIN)
+        asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(o) : "v"(x));
+    else if (NL == NL_RELU)
+        asm("v_cvt_rpi_i32_f32 %0, %1" : "=v"(o) : "v"(x));
+    else
+        o = (int)x;
+    return o;
 }
 
 __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
@@ -144,11 +182,16 @@ __device__ __forceinline__ uint32_t requant4_fast(int a0, int a1, int a2, int a3
         z2 = (int)(int8_t)(zw >> 16);
         z3 = (int)zw >> 24;
     }
-    int r0 = requant_s8_fast<NL, HAS_Z>(a0, z0, e);
-    int r1 = requant_s8_fast<NL, HAS_Z>(a1, z1, e);
-    int r2 = requant_s8_fast<NL, HAS_Z>(a2, z2, e);
-    int r3 = requant_s8_fast<NL, HAS_Z>(a3, z3, e);
-    return pack4(r0, r1, r2, r3);
+    const float x0 = requant_fast_value<NL, HAS_Z>(a0, z0, e);
+    const float x1 = requant_fast_value<NL, HAS_Z>(a1, z1, e);
+    const float x2 = requant_fast_value<NL, HAS_Z>(a2, z2, e);
+    const float x3 = requant_fast_value<NL, HAS_Z>(a3, z3, e);
+    uint32_t o;
+    convert_into_byte<NL, 0>(o, x0);
+    convert_into_byte<NL, 1>(o, x1);
+    convert_into_byte<NL, 2>(o, x2);
+    convert_into_byte<NL, 3>(o, x3);
+    return o;
 }
 
 __device__ __forceinline__ uint32_t requant4_exact(int a0, int a1, int a2, int a3, uint32_t zw,
