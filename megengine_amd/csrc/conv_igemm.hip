@@ -541,7 +541,9 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess) {
             // costs no LDS
             if (d.oc <= 64) return v2 + V64x128x64r4;
             if (t128 >= cu) return v2 + V128x128x64r4;
-            if (pw) return v2 + V64x128x128r3;
+            // pointwise: more pixels than channels per tile; with fewer tiles than CUs and a very long reduction the
+            // small tile with the deepest ring
+            if (pw) return v2 + (kb >= 2048 && t128 < cu ? V64x64x128r4 : V64x128x128r3);
             if (kb >= 4608) return v2 + V64x64x128r4;
             if (d.stride_h == 1 && d.stride_w == 1) return v2 + V64x128x128r3;
             // few tiles, strided 3x3 over at most 256 channels: the first-generation tiles below
@@ -584,7 +586,7 @@ int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess) {
         const int64_t t128 = tiles(0);
         // layers with a residual and a short reduction (the expanding 1x1 of a bottleneck block) are bound by their
         // epilogue: three 8-wave workgroups per CU at every size (whole-stack graph replays, each tile in turn)
-        if (d.has_z && kbytes <= 512 && t128 >= cu_count) return D128x128x64w8;
+        if (d.has_z && t128 >= cu_count && (kbytes <= 128 || (kbytes <= 512 && t128 < 2 * cu_count))) return D128x128x64w8;
         if (t128 >= 4 * cu_count)
             return kbytes >= 1024 ? (OC >= 256 ? D256x128x64w8 : D128x128x128r2) : (kbytes <= 128 ? D128x128x64w8 : D128x128x128r2w8);
         if (t128 >= 2 * cu_count) return D128x64x128r2;
