@@ -360,6 +360,9 @@ struct Igemm2 {
                      "s"(a.div_ow.s2), "s"(a.div_tiles_m.m), "s"(a.div_tiles_m.s1), "s"(a.div_tiles_m.s2),
                      "s"(a.div_tiles_m_pg.m), "s"(a.div_tiles_m_pg.s1), "s"(a.div_tiles_m_pg.s2), "s"(a.div_step.m),
                      "s"(a.div_step.s1), "s"(a.div_step.s2), "s"(a.z), "s"(a.z_bytes), "s"(a.epi.has_z));
+        if (!PW)  // the k-unit table
+            asm volatile("" ::"s"(a.div_t.m), "s"(a.div_t.s1), "s"(a.div_t.s2), "s"(a.div_fw.m), "s"(a.div_fw.s1), "s"(a.div_fw.s2),
+                         "s"(a.T), "s"(a.FW));
         extern __shared__ __attribute__((aligned(16))) int8_t lds[];
         int* sBias = reinterpret_cast<int*>(lds + NS * STG);
         // [ring][bias][residual slots, only for launches with a residual][k-unit table]
