@@ -9,7 +9,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int IG_THREADS = 256;
-constexpr int IG_MAX_ENTRIES = 2048;  // k-unit table capacity (entries of 8 bytes)
+constexpr int IG_MAX_ENTRIES = 4096;  // k-unit table capacity (entries of 8 bytes: 32 KiB of LDS when full)
 
 struct IgemmArgs {
     const int8_t* src;

@@ -207,6 +207,16 @@ def test_igemm_formats_and_tiles(oracle, i):
         check_case(oracle, d, seed=100 + i, algo=IGEMM, tile=tile, tag="igemm%d" % i)
 
 
+def test_igemm_long_k_table(oracle):
+    """3x3 over 1024 channels of a 4-packed tensor: 2304 k-units, beyond the first 2048 table entries."""
+    d = _abi.make_conv_desc("NCHW4", 1, 1024, 6, 6, 64, 3, pad=1, nonline="RELU", **S)
+    a, _ = ops.conv_bias_query(d)
+    assert a.id == IGEMM
+    check_case(oracle, d, seed=77, algo=IGEMM, tag="longk4")
+    d = _abi.make_conv_desc("NCHW32", 1, 8192, 3, 3, 32, 3, pad=1, nonline="IDENTITY", **S)
+    check_case(oracle, d, seed=78, algo=IGEMM, tag="longk32")
+
+
 def test_igemm_nonlines_z_bias(oracle):
     for nl in ("IDENTITY", "RELU", "H_SWISH"):
         for has_z in (False, True):
