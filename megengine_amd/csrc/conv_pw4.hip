@@ -27,8 +27,6 @@ __global__ __launch_bounds__(256) void pw4s_kernel(IgemmArgs a, int n_ocg, int n
     const int t = threadIdx.x;
     const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
-    for (int i = t; i < PW4_MAX_OC + 96; i += 256) sBias[i] = (a.has_bias && i < a.OC) ? a.bias[i] : 0;
-    __syncthreads();
 
     const int gw = blockIdx.x * 4 + wave, GW = gridDim.x * 4;  // GW is a multiple of n_ocg
     const int pb0 = gw / n_ocg, ocg = gw - pb0 * n_ocg, step = GW / n_ocg;
@@ -66,6 +64,10 @@ __global__ __launch_bounds__(256) void pw4s_kernel(IgemmArgs a, int n_ocg, int n
     ZRegs<HZ ? MT : 1, 1> zr, nz;
     load_b(pb0, fb);
     if constexpr (HZ) igemm_load_z<4, MT, 1>(a, zr, oc_w, pb0 * 32, l32, lh);
+    // the bias goes to LDS after the filter rows and the first block are requested: one memory round trip before the
+    // first multiply instead of two (the barrier waits for everything outstanding)
+    for (int i = t; i < PW4_MAX_OC + 96; i += 256) sBias[i] = (a.has_bias && i < a.OC) ? a.bias[i] : 0;
+    __syncthreads();
     for (int pb = pb0; pb < n_pb; pb += step) {
         // the next block's pixels and residual are in flight during the multiply and the epilogue
         load_b(pb + step, nb);
