@@ -649,12 +649,14 @@ int oracle_relayout(const mi355_relayout_desc* d, const void* src, void* dst) {
 /* helpers for tests of the device epilogue's division scheme                            */
 /* ------------------------------------------------------------------------------------ */
 
-/* The device epilogue divides by the (per-tensor constant) dst scale without a hardware
- * divide: with y_hi = RN(1/b), y_lo = RN(1/b - y_hi),
+/* Division by a constant without a hardware divide, in its correctly rounded form: with y_hi = RN(1/b),
+ * y_lo = RN(1/b - y_hi),
  *   q0 = fma(a, y_hi, a * y_lo)   (faithful quotient)
  *   r  = fma(-q0, b, a)           (exact residual)
  *   q  = fma(r, y_hi, q0)         (correctly rounded a / b)
- * This host copy lets a CPU test sweep it against the C '/' operator. */
+ * This host copy lets a CPU test sweep it against the C '/' operator.  The device epilogue runs the cheaper variant
+ * q0 = a * y_hi (a faithful quotient, not always the correctly rounded one), which is checked differently: at every
+ * rounding boundary of the final roundf, per dst scale (tests/test_epilogue_quotient.py and the library's own proof). */
 float oracle_fastdiv(float a, float b, float y_hi, float y_lo) {
     float t = a * y_lo;
     float q0 = fmaf(a, y_hi, t);
