@@ -185,6 +185,17 @@ def main():
         except Exception:
             pass
 
+    # ---- what the launches and the memory traffic alone cost here: the same 53 dependent launches as plain streaming
+    # kernels that read and write each layer's bytes (mi355_stream_probe), replayed from a captured graph like the stack
+    if not args.no_graph:
+        try:
+            chain_ms = streaming_chain_ms(torch, L, layers, side, stream, max(20, args.steps // 4))
+            roofline["streaming_chain_ms"] = round(chain_ms, 4)
+            roofline["vs_streaming_chain"] = round(ms_per_step / chain_ms, 3)
+        except Exception as e:  # a measuring stick must not lose the headline
+            roofline["streaming_chain_ms"] = None
+            log("streaming chain: %r" % (e,))
+
     out = dict(metric="ResNet-50 int8 conv-stack throughput @ bs64 (53 ConvBias layers)", value=round(img_s, 1),
                unit="img/s", n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_per_step, 4),
                higher_is_better=True, scaling="weak", vs_baseline=None, dtype="s8",
@@ -283,6 +294,40 @@ def time_launches(torch, fn, iters=20, warm=3):
     e1.record(st)
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) / iters * 1e-3
+
+
+def streaming_chain_ms(torch, L, layers, side, stream, reps):
+    """One pass over the layer list as plain streaming launches: layer i reads src + filter + bias (+ residual) bytes and
+    writes dst bytes, ping-ponging between two buffers; captured once, replayed `reps` times."""
+    rd = [((l.bytes - l.n * l.oc * l.oh * l.ow) + 15) // 16 * 16 for l in layers]
+    wr = [(l.n * l.oc * l.oh * l.ow + 15) // 16 * 16 for l in layers]
+    cap = max(max(rd), max(wr))
+    a = torch.ones(cap, dtype=torch.uint8, device="cuda")
+    b = torch.ones(cap, dtype=torch.uint8, device="cuda")
+    raw = stream.cuda_stream
+
+    def chain():
+        for i in range(len(layers)):
+            s, d = (a, b) if i % 2 == 0 else (b, a)
+            st = L.mi355_stream_probe(raw, s.data_ptr(), rd[i], d.data_ptr(), wr[i])
+            if st:
+                raise RuntimeError("mi355_stream_probe: status %d" % st)
+
+    chain()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        chain()
+    for _ in range(3):
+        g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(reps):
+        g.replay()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
 
 
 _FLUSH = None

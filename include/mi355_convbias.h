@@ -157,6 +157,13 @@ typedef struct mi355_device_info {
 } mi355_device_info;
 int mi355_get_device_info(int device, mi355_device_info* out);
 
+/* A measuring stick, not an operator: launches one plain streaming kernel on `stream` that reads read_bytes from src and
+ * writes write_bytes to dst in 16-byte accesses (buffers 16-byte aligned, counts multiples of 16; the bytes written are
+ * a function of the bytes read).  A chain of such launches with the byte counts of a network's layers shows what the
+ * launches and the memory traffic alone cost on this device, which is what bench.py reports beside the data-sheet
+ * roofline.  No counterpart in the reference. */
+int mi355_stream_probe(void* stream, const void* src, uint64_t read_bytes, void* dst, uint64_t write_bytes);
+
 /* ---- ConvBias ---- */
 /* output spatial size: floor((i + 2p - ((f-1)d+1)) / s) + 1  (dnn/src/common/utils.cpp:130-138) */
 int mi355_convbias_deduce_out(const mi355_conv_desc* d, uint32_t* oh, uint32_t* ow);

@@ -597,6 +597,15 @@ int mi355_convbias_s8_profile(void* stream, const mi355_conv_desc* d, const mi35
     return MI355_OK;
 }
 
+int mi355_stream_probe(void* stream, const void* src, uint64_t read_bytes, void* dst, uint64_t write_bytes) {
+    if ((read_bytes && !src) || (write_bytes && !dst)) return fail(MI355_ERR_BAD_ARG, "null buffer");
+    if ((read_bytes | write_bytes) & 15) return fail(MI355_ERR_BAD_ARG, "byte counts must be multiples of 16");
+    if (!aligned16(src) || !aligned16(dst)) return fail(MI355_ERR_BAD_ARG, "buffers need 16-byte alignment");
+    hipError_t e = (hipError_t)launch_stream_probe(reinterpret_cast<hipStream_t>(stream), src, read_bytes, dst, write_bytes, cu_count());
+    if (e != hipSuccess) return fail(MI355_ERR_LAUNCH, "stream probe: %s", hipGetErrorString(e));
+    return MI355_OK;
+}
+
 int mi355_requant_s32_s8_exec(void* stream, const mi355_requant_desc* d, const int32_t* src, const int8_t* z, int8_t* dst) {
     if (!d) return fail(MI355_ERR_BAD_ARG, "null descriptor");
     if (d->nonline == MI355_NL_SIGMOID || d->nonline > MI355_NL_H_SWISH)

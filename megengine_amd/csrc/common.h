@@ -60,6 +60,8 @@ int launch_requant(hipStream_t st, const EpiParams& e, const int32_t* src, const
 int launch_requant8(hipStream_t st, const EpiParams& e, const int8_t* src, const int8_t* z, int8_t* dst, uint64_t count,
                     int cu_count);
 
+// plain streaming kernel: reads read_bytes from src and writes write_bytes to dst in 16-byte accesses (a measuring stick)
+int launch_stream_probe(hipStream_t st, const void* src, uint64_t read_bytes, void* dst, uint64_t write_bytes, int cu_count);
 int launch_cvt_f32_s8(hipStream_t st, float scale, const float* src, int8_t* dst, uint64_t count, int cu_count);
 int launch_cvt_s8_f32(hipStream_t st, float scale, const int8_t* src, float* dst, uint64_t count, int cu_count);
 

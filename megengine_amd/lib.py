@@ -14,7 +14,7 @@ _LIB = None
 
 # every symbol declared in include/mi355_convbias.h
 EXPORTS = [
-    "mi355_abi_version", "mi355_status_string", "mi355_last_error", "mi355_get_device_info",
+    "mi355_abi_version", "mi355_status_string", "mi355_last_error", "mi355_get_device_info", "mi355_stream_probe",
     "mi355_convbias_deduce_out", "mi355_convbias_algo_count", "mi355_convbias_algo_name",
     "mi355_convbias_algo_usable", "mi355_convbias_s8_query", "mi355_convbias_s8_exec",
     "mi355_igemm_tile_count", "mi355_igemm_tile_name", "mi355_epilogue_linear_form",
@@ -49,6 +49,8 @@ def lib():
     L.mi355_status_string.argtypes = [C.c_int]
     L.mi355_last_error.restype = C.c_char_p
     L.mi355_get_device_info.argtypes = [C.c_int, P(_abi.DeviceInfo)]
+    L.mi355_stream_probe.restype = C.c_int
+    L.mi355_stream_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64]
     L.mi355_convbias_deduce_out.argtypes = [P(_abi.ConvDesc), P(C.c_uint32), P(C.c_uint32)]
     L.mi355_convbias_algo_count.restype = C.c_int
     L.mi355_convbias_algo_name.restype = C.c_char_p
