@@ -133,3 +133,12 @@ def test_exec_rejects_host_tensors():
     x = torch.zeros(1, 2, 4, 4, 4, dtype=torch.int8)
     with pytest.raises(RuntimeError):
         ops.conv_bias_exec(d, x, x, None, None)
+
+
+def test_stream_probe_argument_checks():
+    L = lib.lib()
+    assert L.mi355_stream_probe(None, None, 16, None, 0) == _abi.ERR_BAD_ARG       # bytes to read but no buffer
+    assert L.mi355_stream_probe(None, None, 0, None, 16) == _abi.ERR_BAD_ARG
+    assert L.mi355_stream_probe(None, 4096, 24, 8192, 16) == _abi.ERR_BAD_ARG      # not a multiple of 16
+    assert L.mi355_stream_probe(None, 4100, 16, 8192, 16) == _abi.ERR_BAD_ARG      # misaligned
+    assert L.mi355_stream_probe(None, None, 0, None, 0) == 0                       # nothing to do

@@ -170,3 +170,21 @@ def test_linear_form_on_every_int32():
                     raise AssertionError("x=%d: linear %d, multi-step %d (scales %r %r, %s)" % (
                         int(x[bad]), int(lin[bad]), int(ref[bad]), s_src, s_dst, nl))
     assert checked >= 18, checked
+
+
+def test_stream_probe_moves_the_bytes():
+    """The bench's measuring stick: reads every input vector, writes every output vector (each output is the running
+    XOR of the inputs its thread has read, so an output equals its input wherever the launch gives a thread one unit)."""
+    import ctypes as C
+    from megengine_amd import lib
+    n = 1 << 20
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda")
+    dst = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    st = lib.lib().mi355_stream_probe(C.c_void_p(torch.cuda.current_stream().cuda_stream), src.data_ptr(), n, dst.data_ptr(), n)
+    assert st == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src)      # 65536 units on at least as many threads: one unit per thread
+    dst.zero_()
+    assert lib.lib().mi355_stream_probe(C.c_void_p(torch.cuda.current_stream().cuda_stream), src.data_ptr(), n, dst.data_ptr(), n // 4) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dst[: n // 4], src[: n // 4]) and int(dst[n // 4:].max()) == 0
