@@ -159,7 +159,7 @@ int mi355_get_device_info(int device, mi355_device_info* out);
 
 /* A measuring stick, not an operator: launches one plain streaming kernel on `stream` that reads read_bytes from src and
  * writes write_bytes to dst in 16-byte accesses (buffers 16-byte aligned, counts multiples of 16; the bytes written are
- * a function of the bytes read).  A chain of such launches with the byte counts of a network's layers shows what the
+ * a function of the bytes read; a probe that reads must write at least 16 bytes, which is what keeps its loads).  A chain of such launches with the byte counts of a network's layers shows what the
  * launches and the memory traffic alone cost on this device, which is what bench.py reports beside the data-sheet
  * roofline.  No counterpart in the reference. */
 int mi355_stream_probe(void* stream, const void* src, uint64_t read_bytes, void* dst, uint64_t write_bytes);
@@ -214,6 +214,12 @@ int mi355_convbias_s8_profile(void* stream, const mi355_conv_desc* d, const mi35
 /* tile configurations of the MFMA implicit-GEMM algorithm (values of mi355_algo.tile_cfg) */
 int mi355_igemm_tile_count(void);
 const char* mi355_igemm_tile_name(int tile_cfg);
+/* MI355_OK if the MFMA algorithm runs descriptor `d` on exactly this tile (AlgoBase::is_available of the reference's
+ * algorithm packs, dnn/src/cuda/conv_bias/algo.h: each tile is one algorithm there too).  A tile can be unavailable
+ * for a packing (the LDS-direct tiles need 32-packed inputs), a dst dtype or bias shape (two tiles carry the general
+ * epilogue) or a residual (ring + residual slot beyond the LDS of a CU).  exec() with such a tile: MI355_ERR_ALGO when the
+ * caller named it, the tile that can run when the heuristic did (MI355_ALGO_FLAG_HEURISTIC). */
+int mi355_igemm_tile_usable(const mi355_conv_desc* d, int tile_cfg);
 
 /* The requantisation without z, dst = quantize_s8(act(float(sfb) * scale_bias)) with act IDENTITY or RELU
  * (dnn/src/naive/conv_bias/opr_impl.cpp:52,69-73,89-93; dnn/include/megdnn/dtype.h:845-853), is a step

@@ -7,6 +7,8 @@
 #include <string.h>
 
 #include <mutex>
+#include <shared_mutex>
+#include <unordered_map>
 
 #include "common.h"
 
@@ -113,25 +115,45 @@ bool epi_prove_quotient(float s_d) {
     return true;
 }
 
-struct QuotEntry {
-    uint32_t kd;
-    int state;  // 0 empty, 1 proved, 2 failed
+// Verdicts are kept for the life of the process, one per dst scale: a proof costs ~0.15 ms of host time and an operator
+// asks for it on every call, so an entry, once made, is never evicted (a growing hash map; readers share the lock).
+// Beyond kProofCacheCap entries -- a caller cycling through millions of distinct scales -- new verdicts are computed
+// but no longer stored.
+constexpr size_t kProofCacheCap = 1u << 20;
+
+template <class V>
+class ProofCache {
+public:
+    bool find(uint64_t key, V* out) {
+        std::shared_lock<std::shared_mutex> lk(mu_);
+        auto it = map_.find(key);
+        if (it == map_.end()) return false;
+        *out = it->second;
+        return true;
+    }
+    void insert(uint64_t key, const V& v) {
+        std::unique_lock<std::shared_mutex> lk(mu_);
+        if (map_.size() < kProofCacheCap) map_.emplace(key, v);
+    }
+    size_t size() {
+        std::shared_lock<std::shared_mutex> lk(mu_);
+        return map_.size();
+    }
+
+private:
+    std::shared_mutex mu_;
+    std::unordered_map<uint64_t, V> map_;
 };
-QuotEntry g_quot[256];
-std::mutex g_quot_mu;
+
+ProofCache<bool> g_quot;
 
 bool epi_quotient_proved(float s_d) {
     uint32_t kd;
     memcpy(&kd, &s_d, 4);
-    const uint32_t slot = (kd * 2654435761u) >> 24;
-    {
-        std::lock_guard<std::mutex> lk(g_quot_mu);
-        if (g_quot[slot].state && g_quot[slot].kd == kd) return g_quot[slot].state == 1;
-    }
-    const bool ok = epi_prove_quotient(s_d);
-    std::lock_guard<std::mutex> lk(g_quot_mu);
-    g_quot[slot].kd = kd;
-    g_quot[slot].state = ok ? 1 : 2;
+    bool ok;
+    if (g_quot.find(kd, &ok)) return ok;
+    ok = epi_prove_quotient(s_d);
+    g_quot.insert(kd, ok);
     return ok;
 }
 
@@ -206,37 +228,28 @@ bool epi_solve_linear(float s_b, float s_d, bool relu, float* c_out, float* d_ou
     return false;
 }
 
-// Results are kept per (s_b, s_d, activation): a search is ~0.1 ms of host time, a hit a few dozen ns.
+// Results are kept per (s_b, s_d, activation) for the life of the process (never evicted, see ProofCache): a search is
+// ~0.1 ms of host time, a hit a hash lookup.
 struct LinEntry {
-    uint32_t kb, kd;
-    int relu, state;  // state: 0 empty, 1 solved, 2 no solution
+    bool solved;
     float c, d;
 };
-LinEntry g_lin[256];
-std::mutex g_lin_mu;
+ProofCache<LinEntry> g_lin[2];  // [relu]
 
 bool epi_linear_cached(float s_b, float s_d, bool relu, float* c, float* d) {
     uint32_t kb, kd;
     memcpy(&kb, &s_b, 4);
     memcpy(&kd, &s_d, 4);
-    const uint32_t slot = ((kb * 2654435761u) ^ (kd * 40503u) ^ (uint32_t)relu) >> 5 & 255u;
-    {
-        std::lock_guard<std::mutex> lk(g_lin_mu);
-        const LinEntry& e = g_lin[slot];
-        if (e.state && e.kb == kb && e.kd == kd && e.relu == (int)relu) {
-            *c = e.c;
-            *d = e.d;
-            return e.state == 1;
-        }
+    const uint64_t key = ((uint64_t)kb << 32) | kd;
+    LinEntry e;
+    if (!g_lin[relu].find(key, &e)) {
+        e.c = e.d = 0.f;
+        e.solved = epi_solve_linear(s_b, s_d, relu, &e.c, &e.d);
+        g_lin[relu].insert(key, e);
     }
-    LinEntry n;
-    n.kb = kb; n.kd = kd; n.relu = relu; n.c = n.d = 0.f;
-    n.state = epi_solve_linear(s_b, s_d, relu, &n.c, &n.d) ? 1 : 2;
-    std::lock_guard<std::mutex> lk(g_lin_mu);
-    g_lin[slot] = n;
-    *c = n.c;
-    *d = n.d;
-    return n.state == 1;
+    *c = e.c;
+    *d = e.d;
+    return e.solved;
 }
 
 // All epilogue parameters of one launch.  qs8: the destination is QuantizedS8 (the only dtype with the fast forms).
@@ -258,8 +271,7 @@ void epi_fill(EpiParams* e, float s_b, float s_z, float s_d, uint32_t nonline, b
 // Validation of a descriptor: the checks of ConvolutionBase::deduce_layout_fwd
 // (dnn/src/common/convolution.cpp:633-1049) and do_check_exec_common
 // (dnn/src/common/conv_bias.cpp:8-133) that survive the translation to a flat descriptor.
-int canonize(const mi355_conv_desc* d, ConvProblem* p) {
-    if (!d) return fail(MI355_ERR_BAD_ARG, "null descriptor");
+int canonize_checked(const mi355_conv_desc* d, ConvProblem* p) {
     const int pi = in_pack(d->format), po = out_pack(d->format);
     if (!pi) return fail(MI355_ERR_UNSUPPORTED, "format %u not supported by this backend", d->format);
     if (d->sparse > MI355_SPARSE_GROUP) return fail(MI355_ERR_BAD_ARG, "invalid convolution sparse type");
@@ -317,6 +329,26 @@ int canonize(const mi355_conv_desc* d, ConvProblem* p) {
     epi_fill(&p->epi, d->scale_bias, d->scale_z, d->scale_dst, d->nonline, d->has_z != 0, d->dst_dtype == MI355_DT_QS8);
     if (d->dst_dtype == MI355_DT_F32) p->epi.s_b = d->scale_bias * d->scale_z;
     return MI355_OK;
+}
+
+// An operator call canonizes the same descriptor several times in a row (get_workspace_in_bytes, the algorithm
+// choice, exec): each thread remembers the last descriptor that passed and its canonical form.  Equal bytes mean an
+// equal descriptor; different padding bytes only cost the full path.
+int canonize(const mi355_conv_desc* d, ConvProblem* p) {
+    if (!d) return fail(MI355_ERR_BAD_ARG, "null descriptor");
+    thread_local bool have = false;
+    thread_local ConvProblem last;
+    if (have && memcmp(d, &last.d, sizeof(*d)) == 0) {
+        *p = last;
+        return MI355_OK;
+    }
+    const int st = canonize_checked(d, p);
+    if (st == MI355_OK) {
+        last = *p;
+        memcpy(&last.d, d, sizeof(*d));  // padding bytes included, so that the comparison above can hit
+        have = true;
+    }
+    return st;
 }
 
 struct DevInfo {
@@ -471,7 +503,20 @@ static int exec_impl(void* stream, const mi355_conv_desc* d, const mi355_algo* a
     }
     if (id < 0 || id >= ALGO_COUNT) return fail(MI355_ERR_ALGO, "unknown algorithm id %d", id);
     if (!algo_usable(p, id)) return fail(MI355_ERR_ALGO, "%s cannot run this problem", kAlgoNames[id]);
-    if (id == ALGO_IGEMM_MFMA && (cfg < 0 || cfg >= igemm_num_cfgs())) cfg = igemm_pick_cfg(p, cu_count());
+    const bool by_heuristic = !algo || algo->id == MI355_ALGO_HEURISTIC || (algo->reserved & MI355_ALGO_FLAG_HEURISTIC);
+    if (id == ALGO_IGEMM_MFMA) {
+        if (cfg < 0 || cfg >= igemm_num_cfgs()) {
+            cfg = igemm_pick_cfg(p, cu_count());
+        } else {
+            // the tile that runs is the tile that was named: a tile the caller forced and that cannot run this problem is an
+            // error (a fast-run chooser must not time one kernel under two names); a choice of the heuristic is replaced
+            const int runs = igemm_resolve_cfg(p, cfg);
+            if (runs != cfg && !by_heuristic)
+                return fail(MI355_ERR_ALGO, "tile %s cannot run this problem (%s would)", igemm_cfg_name(cfg),
+                            runs >= 0 ? igemm_cfg_name(runs) : "none");
+            cfg = runs;
+        }
+    }
     if (preprocessed && (id != ALGO_IGEMM_MFMA || igemm_preprocessed_bytes(p, cfg) == 0))
         return fail(MI355_ERR_ALGO, "this algorithm has no pre-processed filter form");
     // the tiled kernels use 16-byte vector accesses; misaligned tensors take the generic kernel
@@ -482,7 +527,7 @@ static int exec_impl(void* stream, const mi355_conv_desc* d, const mi355_algo* a
                   (!z || aligned16(z)) && p.src_sn % sa == 0 && p.dst_sn % da == 0 && p.z_sn % da == 0;
         if (!al) {
             // the generic kernel reads the reference filter layout only
-            if (preprocessed || (algo && algo->id != MI355_ALGO_HEURISTIC && !(algo->reserved & MI355_ALGO_FLAG_HEURISTIC)))
+            if (preprocessed || !by_heuristic)
                 return fail(MI355_ERR_ALGO, "%s needs 16-byte aligned tensors", kAlgoNames[id]);
             id = ALGO_DIRECT;
         }
@@ -600,6 +645,8 @@ int mi355_convbias_s8_profile(void* stream, const mi355_conv_desc* d, const mi35
 int mi355_stream_probe(void* stream, const void* src, uint64_t read_bytes, void* dst, uint64_t write_bytes) {
     if ((read_bytes && !src) || (write_bytes && !dst)) return fail(MI355_ERR_BAD_ARG, "null buffer");
     if ((read_bytes | write_bytes) & 15) return fail(MI355_ERR_BAD_ARG, "byte counts must be multiples of 16");
+    // loads whose values reach no store may be dropped by the compiler: a read-only probe would move nothing
+    if (read_bytes && !write_bytes) return fail(MI355_ERR_BAD_ARG, "a probe that reads must write at least 16 bytes");
     if (!aligned16(src) || !aligned16(dst)) return fail(MI355_ERR_BAD_ARG, "buffers need 16-byte alignment");
     hipError_t e = (hipError_t)launch_stream_probe(reinterpret_cast<hipStream_t>(stream), src, read_bytes, dst, write_bytes, cu_count());
     if (e != hipSuccess) return fail(MI355_ERR_LAUNCH, "stream probe: %s", hipGetErrorString(e));
@@ -711,6 +758,19 @@ int mi355_pooling_s8_exec(void* stream, const mi355_pooling_desc* d, const int8_
 
 int mi355_igemm_tile_count(void) { return igemm_num_cfgs(); }
 const char* mi355_igemm_tile_name(int cfg) { return igemm_cfg_name(cfg); }
+
+int mi355_igemm_tile_usable(const mi355_conv_desc* d, int tile_cfg) {
+    ConvProblem p;
+    int st = canonize(d, &p);
+    if (st) return st;
+    if (!igemm_usable(p)) return fail(MI355_ERR_ALGO, "%s cannot run this problem", kAlgoNames[ALGO_IGEMM_MFMA]);
+    if (tile_cfg < 0 || tile_cfg >= igemm_num_cfgs()) return fail(MI355_ERR_ALGO, "unknown tile configuration %d", tile_cfg);
+    const int runs = igemm_resolve_cfg(p, tile_cfg);
+    if (runs != tile_cfg)
+        return fail(MI355_ERR_ALGO, "tile %s cannot run this problem (%s would)", igemm_cfg_name(tile_cfg),
+                    runs >= 0 ? igemm_cfg_name(runs) : "none");
+    return MI355_OK;
+}
 
 int mi355_epilogue_quotient_form(float scale_dst, float* y) {
     if (!y) return -fail(MI355_ERR_BAD_ARG, "null argument");

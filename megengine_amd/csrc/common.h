@@ -39,6 +39,10 @@ const char* igemm_cfg_name(int cfg);
 bool igemm_usable(const ConvProblem& p);
 // will_preprocess: the caller will hand exec the filter pre-processed for the chosen tile
 int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess = false);
+// The tile that runs when tile_cfg is asked for: tile_cfg itself when that kernel can run the problem as it is, else
+// the tile the launch code takes in its place (another kernel generation for this packing, a tile that has the general
+// epilogue, a ring that fits the LDS).  A choice of the heuristic is replaced silently; a tile the caller forced is not.
+int igemm_resolve_cfg(const ConvProblem& p, int tile_cfg);
 // flt_preprocessed: flt points to the artefact of launch_igemm_preprocess (only tiles with igemm_preprocessed_bytes > 0)
 int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int tile_cfg, int cu_count, const int8_t* src,
                       const int8_t* flt, const int32_t* bias, const int8_t* z, int8_t* dst, bool flt_preprocessed = false);

@@ -21,6 +21,8 @@
 // oc = 8*(v/4) + 4*(l/32) + v%4.  NCHW4 output stores one dword (4 channels) per register quad;
 // NCHW32 output first exchanges quads between lanes l and l+32 (v_permlane32_swap) so that each
 // lane owns 16 consecutive channels of one pixel and stores 16 bytes.
+#include <string.h>
+
 #include <atomic>
 
 #include "igemm_shared.h"
@@ -518,7 +520,7 @@ bool igemm_usable(const ConvProblem& p) {
     return true;
 }
 
-int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess) {
+static int pick_cfg_by_shape(const ConvProblem& p, int cu_count, bool will_preprocess) {
     const mi355_conv_desc& d = p.d;
     if (will_preprocess && p.pin == 32 && p.pout == 32 && d.group == 1 && !igemm_needs_general(p)) {
         // The caller re-tiles the filter for the chosen algorithm (weight pre-processing): the second-generation tiles
@@ -619,11 +621,17 @@ int launch_igemm_preprocess(hipStream_t st, const ConvProblem& p, const int8_t* 
     return launch_igemm2_preprocess(st, flt, out, (int)p.d.oc, (int)(p.icpg * p.d.fh * p.d.fw));
 }
 
-int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_count, const int8_t* src,
-                      const int8_t* flt, const int32_t* bias, const int8_t* z, int8_t* dst, bool flt_preprocessed) {
+// The chooser's tile, as the launch code will run it: what query() hands out names the kernel that executes.
+int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess) {
+    const int c = pick_cfg_by_shape(p, cu_count, will_preprocess);
+    const int r = igemm_resolve_cfg(p, c);
+    return r >= 0 ? r : c;
+}
+
+// everything of IgemmArgs that follows from the problem alone (no tensor pointers, no tile)
+static void igemm_fill_args(const ConvProblem& p, IgemmArgs& a) {
     const mi355_conv_desc& d = p.d;
-    IgemmArgs a;
-    a.src = src; a.flt = flt; a.bias = bias; a.z = z; a.dst = dst;
+    memset(&a, 0, sizeof(a));
     a.IH = d.ih; a.IW = d.iw; a.OH = p.oh; a.OW = p.ow; a.OHW = p.oh * p.ow;
     a.FH = d.fh; a.FW = d.fw; a.T = d.fh * d.fw;
     a.sh = d.stride_h; a.sw = d.stride_w; a.ph = d.pad_h; a.pw = d.pad_w;
@@ -649,6 +657,73 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
     a.epi = p.epi;
     a.flt_rstride = a.kbytes;
     a.flt_kstride = 32;
+    a.groups = d.group;
+    a.ocpg = p.ocpg;
+    a.src_sg = (p.icpg / p.pin) * a.src_scb;
+    a.general = igemm_needs_general(p) ? 1 : 0;
+    a.dst_s32 = d.dst_dtype == MI355_DT_QS32;
+    a.bias_full = d.bias_mode == MI355_BIAS_FULL;
+    if (a.dst_s32) a.epi.s_b = a.epi.s_d;  // the sum lives in dst and is dequantised with the dtype of dst
+}
+
+static int staged_tile_of_shape(int bm, int bn, int kch) {
+    int cfg = 0;
+    for (int i = 0; i < kNumCfgs; ++i)
+        if (kCfgs[i].bm == bm && kCfgs[i].bn == bn && kCfgs[i].kch == kch) cfg = i;
+    return cfg;
+}
+
+int igemm_resolve_cfg(const ConvProblem& p, int cfg) {
+    if (cfg < 0 || cfg >= igemm_num_cfgs()) return -1;
+    const mi355_conv_desc& d = p.d;
+    IgemmArgs a;
+    igemm_fill_args(p, a);
+    if (a.M == 0 || a.OC == 0) return cfg;  // nothing is launched
+    const int first_v2 = igemm_first_v2_cfg();
+    // group convolutions and the general epilogue exist on the second-generation tiles only
+    if ((d.group != 1 || a.general) && cfg < first_v2) cfg = first_v2 + (p.ocpg <= 64 ? 3 : 0);
+    if (cfg >= first_v2) {
+        if (p.pin == 32) {
+            int v = cfg - first_v2;
+            if (igemm2_can_run(a, p.pout, v)) return cfg;
+            int bm, bn, kch;
+            igemm2_cfg_shape(v, &bm, &bn, &kch);
+            // the general epilogue exists on two tiles: the one with the asked tile's channel count, or the smaller one
+            if (a.general) v = bm <= 64 ? 3 : 0;
+            if (igemm2_can_run(a, p.pout, v)) return first_v2 + v;
+            // ring + residual slots beyond the LDS of a CU: 128 x 128 x 64 with a ring of three always fits
+            return first_v2 + 1;
+        }
+        // 4-packed inputs: the register-staged tile of the same shape
+        int bm, bn, kch;
+        igemm2_cfg_shape(cfg - first_v2, &bm, &bn, &kch);
+        return staged_tile_of_shape(bm, bn, kch);
+    }
+    if (cfg >= kNumCfgs) {
+        const int dcfg = cfg - kNumCfgs;
+        const bool c4 = igemm_dma_cfg_is_pin4(dcfg);
+        if (!c4 && p.pin == 32) return cfg;
+        if (c4 && p.pin == 4 && p.pout == 4 && a.T == 1 && a.ph == 0 && a.pw == 0) {
+            // the streaming kernel where it applies, else the 128 x 128 x 64 tile
+            if (dcfg == igemm_dma_num_cfgs() - 1 && !pw4s_usable(a)) return kNumCfgs + igemm_dma_first_pin4_cfg();
+            return cfg;
+        }
+        // no LDS-direct kernel for this packing / filter: the register-staged tile of the same shape
+        int bm, bn, kch;
+        igemm_dma_cfg_shape(dcfg, &bm, &bn, &kch);
+        return staged_tile_of_shape(bm, bn, kch);
+    }
+    return cfg;
+}
+
+int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_count, const int8_t* src,
+                      const int8_t* flt, const int32_t* bias, const int8_t* z, int8_t* dst, bool flt_preprocessed) {
+    IgemmArgs a;
+    igemm_fill_args(p, a);
+    a.src = src; a.flt = flt; a.bias = bias; a.z = z; a.dst = dst;
+    if (a.M == 0 || a.OC == 0) return 0;
+    cfg = igemm_resolve_cfg(p, cfg);
+    if (cfg < 0) return (int)hipErrorInvalidValue;
     if (flt_preprocessed) {
         if (igemm_preprocessed_bytes(p, cfg) == 0) return (int)hipErrorInvalidValue;
         const int ocp = (a.OC + 31) / 32 * 32;
@@ -656,40 +731,9 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
         a.flt_kstride = ocp * 32;
         a.flt_bytes = (uint32_t)igemm_preprocessed_bytes(p, cfg);
     }
-    a.groups = d.group;
-    a.ocpg = p.ocpg;
-    a.src_sg = (p.icpg / p.pin) * a.src_scb;
-    if (a.M == 0 || a.OC == 0) return 0;
     const int first_v2 = igemm_first_v2_cfg();
-    a.general = igemm_needs_general(p) ? 1 : 0;
-    a.dst_s32 = d.dst_dtype == MI355_DT_QS32;
-    a.bias_full = d.bias_mode == MI355_BIAS_FULL;
-    if (a.dst_s32) a.epi.s_b = a.epi.s_d;  // the sum lives in dst and is dequantised with the dtype of dst
-    // group convolutions and the general epilogue exist on the second-generation tiles only
-    if ((d.group != 1 || a.general) && cfg < first_v2) cfg = first_v2;
-    if (cfg >= first_v2) {
-        if (p.pin == 32) return launch_igemm2(st, a, p.pout, cfg - first_v2, cu_count);
-        // 4-packed inputs: the register-staged tile of the same shape
-        int bm, bn, kch;
-        igemm2_cfg_shape(cfg - first_v2, &bm, &bn, &kch);
-        cfg = 0;
-        for (int i = 0; i < kNumCfgs; ++i)
-            if (kCfgs[i].bm == bm && kCfgs[i].bn == bn && kCfgs[i].kch == kch) cfg = i;
-    }
-    if (cfg >= kNumCfgs) {
-        const int dcfg = cfg - kNumCfgs;
-        if (dcfg >= igemm_dma_num_cfgs()) return (int)hipErrorInvalidValue;
-        const bool c4 = igemm_dma_cfg_is_pin4(dcfg);
-        if (!c4 && p.pin == 32) return launch_igemm_dma(st, a, p.pout, dcfg, cu_count);
-        if (c4 && p.pin == 4 && p.pout == 4 && a.T == 1 && a.ph == 0 && a.pw == 0)
-            return launch_igemm_dma(st, a, 4, dcfg, cu_count);
-        // no LDS-direct kernel for this packing / filter: run the register-staged tile of the same shape
-        int bm, bn, kch;
-        igemm_dma_cfg_shape(dcfg, &bm, &bn, &kch);
-        cfg = 0;
-        for (int i = 0; i < kNumCfgs; ++i)
-            if (kCfgs[i].bm == bm && kCfgs[i].bn == bn && kCfgs[i].kch == kch) cfg = i;
-    }
+    if (cfg >= first_v2) return launch_igemm2(st, a, p.pout, cfg - first_v2, cu_count);
+    if (cfg >= kNumCfgs) return launch_igemm_dma(st, a, p.pout, cfg - kNumCfgs, cu_count);
     if (p.pin == 32 && p.pout == 32) return launch_fmt<32, 32>(st, a, cfg, cu_count);
     if (p.pin == 4 && p.pout == 4) return launch_fmt<4, 4>(st, a, cfg, cu_count);
     if (p.pin == 4 && p.pout == 32) return launch_fmt<4, 32>(st, a, cfg, cu_count);

@@ -678,7 +678,8 @@ int launch_k(hipStream_t st, IgemmArgs& a, int cu_count) {
         if (fixed + a.zslots * K::ZSLOT > kLdsPerCu) a.zslots = 1;
     }
     const int lds = fixed + a.zslots * K::ZSLOT;
-    if (lds > kLdsPerCu) return kNoFit;  // ring + residual slot of this tile do not fit: the caller takes a smaller tile
+    if (lds > kLdsPerCu) return kNoFit;  // ring + residual slot of this tile do not fit
+    if (a.dry_run) return 0;             // the question was only whether this tile can run the problem
     auto kern = igemm2_kernel<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW, KT, GEN>;
     // per-instantiation caches; atomics, because operators on different streams may launch from several threads
     static std::atomic<int> max_lds_set{0};
@@ -791,16 +792,17 @@ int launch_igemm2_preprocess(hipStream_t st, const int8_t* flt, int8_t* out, int
     return (int)hipGetLastError();
 }
 
+// A tile that cannot run the problem (no instantiation with the general epilogue, or ring + residual slot beyond the
+// LDS of a CU) is an error here: igemm_resolve_cfg (conv_igemm.hip) names the tile that runs before anything is launched.
 int launch_igemm2(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count) {
-    int rc = pout == 32 ? launch_fmt<32>(st, a, cfg, cu_count) : launch_fmt<4>(st, a, cfg, cu_count);
-    // the general epilogue exists on two tiles: the one with the asked tile's channel count, or the smaller one
-    if (rc == kNoGen) {
-        cfg = kCfg2[cfg].bm <= 64 ? 3 : 0;
-        rc = pout == 32 ? launch_fmt<32>(st, a, cfg, cu_count) : launch_fmt<4>(st, a, cfg, cu_count);
-    }
-    // the large tiles with a residual need more LDS than a CU has: 128 x 128 x 64 with a ring of three always fits
-    if (rc == kNoFit) rc = pout == 32 ? launch_fmt<32>(st, a, 1, cu_count) : launch_fmt<4>(st, a, 1, cu_count);
-    return rc == kNoFit ? (int)hipErrorInvalidValue : rc;
+    const int rc = pout == 32 ? launch_fmt<32>(st, a, cfg, cu_count) : launch_fmt<4>(st, a, cfg, cu_count);
+    return rc == kNoFit || rc == kNoGen ? (int)hipErrorInvalidConfiguration : rc;
+}
+
+bool igemm2_can_run(const IgemmArgs& a, int pout, int cfg) {
+    IgemmArgs t = a;
+    t.dry_run = 1;
+    return (pout == 32 ? launch_fmt<32>(nullptr, t, cfg, 256) : launch_fmt<4>(nullptr, t, cfg, 256)) == 0;
 }
 
 }  // namespace mi355

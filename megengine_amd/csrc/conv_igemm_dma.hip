@@ -54,7 +54,8 @@ struct DmaKernel {
     static constexpr int NOFF = PIN == 4 ? (NB64 > 0 ? NB64 : 1) : UB32;  // per-lane activation offsets kept by the loader
     static constexpr int U = UA + UB;
     static_assert(PIN == 32 || (PIN == 4 && PW && BN % 64 == 0 && CB % NW == 0), "4-packed inputs: pointwise tiles of whole 64-pixel blocks");
-    static constexpr int BIAS_BYTES = BM * 4;  // bias of the workgroup's channel tile
+    // bias of the workgroup's channel tile; it arrives by whole-wave copies of 64 dwords (a 32-row tile leaves half of one unused)
+    static constexpr int BIAS_BYTES = (BM < 64 ? 64 : BM) * 4;
     static constexpr int RING_BYTES = NS * STG + BIAS_BYTES;
     static_assert(NW == 4 || NW == 8, "4 or 8 waves");
     static_assert(UA >= 1 && UB >= 1 && BM % (RPL * NW) == 0 && (PIN == 4 || BN % (RPL * NW) == 0), "tile vs copy granularity");
@@ -223,16 +224,18 @@ struct DmaKernel {
         const int my_tiles = first < last ? (int)fdiv((uint32_t)(last - first + step - 1), a.div_step) : 0;
         const int total = my_tiles * a.nstages;
 
-        // The bias of the workgroup's channel tile lives in LDS, written once after the prologue's copies are issued: workgroups
-        // mostly stay on one channel tile (their tile stride is a multiple of the number of channel tiles whenever
-        // that is a power of two), so the copy is read at every tile start and almost never rewritten.
+        // The bias of the workgroup's channel tile lives in LDS, copied there once: workgroups mostly stay on one channel
+        // tile (their tile stride is a multiple of the number of channel tiles whenever that is a power of two), so the
+        // copy is read at every tile start and almost never rewritten.
         int* sBias = reinterpret_cast<int*>(lds + NS * STG);
         int c_tile = first, c_oc0, c_pix0;
         tile_coords(a, c_tile, c_oc0, c_pix0);
-        // requested now, written to LDS only after the prologue's copies are on their way: the first touch of the bias
-        // (a cold miss) overlaps theirs instead of preceding it.  Without a bias the buffer has no bytes: every lane reads 0
+        // An LDS-direct copy like the operands' (no register is the target of a load the compiler does not know about),
+        // requested before the prologue's copies: its cold miss overlaps theirs, and it is older than all of them.
+        // Without a bias the buffer has no bytes: every lane writes 0, and so do channels past the last one.
         const v4i rs_bias = uniform_rsrc(a.bias, a.has_bias ? (uint32_t)a.OC * 4u : 0u);
-        int bias_reg = load_dword_async(t < BM ? (c_oc0 + t) * 4 : SENT, rs_bias);
+        const bool bias_wave = wave * 64 < BM;  // wave-uniform
+        if (total != 0 && bias_wave) lds_copy64x4(lds0 + (uint32_t)(NS * STG + wave * 256), (c_oc0 + t) * 4, rs_bias);
 
         if (!PW) {
             const int cap = a.nstages * KCH;
@@ -282,10 +285,9 @@ struct DmaKernel {
             advance();
         }
         v16i acc[MT][NT];
-        // older than every copy of the prologue (the counter holds at most 63: with more copies than that in the
-        // prologue the oldest operations, this one first, have completed by the time the last copy was accepted)
-        wait_vmcnt_for<((NS - 1) * U < 63 ? (NS - 1) * U : 63)>(bias_reg);
-        if (t < BM) sBias[t] = bias_reg;
+        // the bias copy is older than every copy of the prologue (the counter holds at most 63: with more copies than
+        // that in the prologue the oldest operations, this one first, have completed by the time the last copy was accepted)
+        wait_vmcnt<((NS - 1) * U < 63 ? (NS - 1) * U : 63)>();
         __syncthreads();
         init_acc_lds(acc, sBias, wm, lh);
         int rd_off = 0;                                     // byte offset of the stage being multiplied
@@ -534,6 +536,7 @@ void igemm_dma_cfg_shape(int cfg, int* bm, int* bn, int* kch) {
 }
 
 bool igemm_dma_cfg_is_pin4(int cfg) { return cfg >= kFirstDma4; }
+int igemm_dma_first_pin4_cfg() { return kFirstDma4; }
 
 int launch_igemm_dma(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count) {
     return pout == 32 ? launch_fmt<32>(st, a, cfg, cu_count) : launch_fmt<4>(st, a, cfg, cu_count);

@@ -48,6 +48,7 @@ struct IgemmArgs {
     // reciprocal on the critical path from kernel entry to the first copy): by the number of channel tiles, by the
     // channel tiles of a group, and by the tile stride of a workgroup (set by the launch code, which knows the grid)
     FastDiv div_tiles_m, div_tiles_m_pg, div_step;
+    int dry_run;  // host only: the launch code stops before anything is launched and reports whether the tile fits
 };
 
 struct KEntry {
@@ -249,6 +250,7 @@ int igemm_dma_num_cfgs();
 const char* igemm_dma_cfg_name(int cfg);
 void igemm_dma_cfg_shape(int cfg, int* bm, int* bn, int* kch);
 bool igemm_dma_cfg_is_pin4(int cfg);  // a 4-packed pointwise tile (NCHW4 in and out, 1x1, no padding)
+int igemm_dma_first_pin4_cfg();       // the first of them (128 x 128 x 64)
 int launch_igemm_dma(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count);
 
 // second-generation kernel for 32-packed inputs (conv_igemm2.hip): chunk-major LDS stages, software-pipelined k-loop,
@@ -257,6 +259,8 @@ int igemm2_num_cfgs();
 const char* igemm2_cfg_name(int cfg);
 void igemm2_cfg_shape(int cfg, int* bm, int* bn, int* kch);
 int launch_igemm2(hipStream_t st, IgemmArgs& a, int pout, int cfg, int cu_count);
+// whether second-generation tile `cfg` runs this problem as itself (general epilogue instantiated, LDS fits); no launch
+bool igemm2_can_run(const IgemmArgs& a, int pout, int cfg);
 int igemm_first_v2_cfg();  // tile_cfg of the first second-generation tile
 // pre-processed filter of the second-generation kernel: [k-chunk][channel padded to 32][32 bytes]
 size_t igemm2_preprocessed_bytes(int oc, int kbytes);

@@ -39,28 +39,6 @@ __device__ __forceinline__ void wait_vmcnt() {
 
 __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
-// loads the compiler does not wait for: the value is valid only after wait_vmcnt_for on it
-__device__ __forceinline__ int load_dword_async(int voff, const v4i& rsrc) {
-    int v;
-    asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=v"(v) : "v"(voff), "s"(rsrc) : "memory");
-    return v;
-}
-__device__ __forceinline__ v4i load_b128_async(int voff, const v4i& rsrc) {
-    v4i v;
-    asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(v) : "v"(voff), "s"(rsrc) : "memory");
-    return v;
-}
-template <int N>
-__device__ __forceinline__ void wait_vmcnt_for(int& v) {
-    static_assert(N >= 0 && N < 64, "vmcnt range");
-    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N) : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_vmcnt_for(v4i& v) {
-    static_assert(N >= 0 && N < 64, "vmcnt range");
-    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N) : "memory");
-}
-
 // a buffer descriptor held in scalar registers (the inline assembly takes it as an "s" operand)
 __device__ __forceinline__ v4i uniform_rsrc(const void* p, uint32_t bytes) {
     const uint64_t a = (uint64_t)(uintptr_t)p;

@@ -489,7 +489,8 @@ std::vector<AlgorithmInfo> ConvBiasForward::get_all_algorithms_info(const Tensor
         r.push_back(AlgorithmInfo{AlgorithmDesc{id, -1}, base, true});
         if (base.find("IGEMM") != std::string::npos)
             for (int t = 0; t < mi355_igemm_tile_count(); ++t)
-                r.push_back(AlgorithmInfo{AlgorithmDesc{id, t}, base + ":" + mi355_igemm_tile_name(t), true});
+                if (mi355_igemm_tile_usable(&c.d, t) == MI355_OK)  // one kernel, one name
+                    r.push_back(AlgorithmInfo{AlgorithmDesc{id, t}, base + ":" + mi355_igemm_tile_name(t), true});
     }
     return r;
 }

@@ -17,7 +17,7 @@ EXPORTS = [
     "mi355_abi_version", "mi355_status_string", "mi355_last_error", "mi355_get_device_info", "mi355_stream_probe",
     "mi355_convbias_deduce_out", "mi355_convbias_algo_count", "mi355_convbias_algo_name",
     "mi355_convbias_algo_usable", "mi355_convbias_s8_query", "mi355_convbias_s8_exec",
-    "mi355_igemm_tile_count", "mi355_igemm_tile_name", "mi355_epilogue_linear_form",
+    "mi355_igemm_tile_count", "mi355_igemm_tile_name", "mi355_igemm_tile_usable", "mi355_epilogue_linear_form",
     "mi355_relayout_deduce", "mi355_relayout_exec", "mi355_requant_s32_s8_exec", "mi355_requant_s8_s8_exec", "mi355_convbias_s8_profile",
     "mi355_pooling_deduce_out", "mi355_pooling_s8_exec", "mi355_typecvt_f32_s8_exec", "mi355_typecvt_s8_f32_exec",
     "mi355_epilogue_quotient_form", "mi355_convbias_s8_preprocess_size", "mi355_convbias_s8_preprocess", "mi355_convbias_s8_exec_preprocessed",
@@ -69,6 +69,7 @@ def lib():
     L.mi355_igemm_tile_count.restype = C.c_int
     L.mi355_igemm_tile_name.restype = C.c_char_p
     L.mi355_igemm_tile_name.argtypes = [C.c_int]
+    L.mi355_igemm_tile_usable.argtypes = [P(_abi.ConvDesc), C.c_int]
     L.mi355_epilogue_quotient_form.restype = C.c_int
     L.mi355_epilogue_quotient_form.argtypes = [C.c_float, P(C.c_float)]
     L.mi355_epilogue_linear_form.restype = C.c_int
@@ -100,6 +101,11 @@ def algo_names():
 def tile_names():
     L = lib()
     return [L.mi355_igemm_tile_name(i).decode() for i in range(L.mi355_igemm_tile_count())]
+
+
+def tile_usable(desc, tile):
+    """True if the MFMA algorithm runs `desc` on exactly this tile (a forced tile that cannot is MI355_ERR_ALGO at exec)"""
+    return lib().mi355_igemm_tile_usable(C.byref(desc), tile) == 0
 
 
 def device_info(device=0):

@@ -142,3 +142,42 @@ def test_stream_probe_argument_checks():
     assert L.mi355_stream_probe(None, 4096, 24, 8192, 16) == _abi.ERR_BAD_ARG      # not a multiple of 16
     assert L.mi355_stream_probe(None, 4100, 16, 8192, 16) == _abi.ERR_BAD_ARG      # misaligned
     assert L.mi355_stream_probe(None, None, 0, None, 0) == 0                       # nothing to do
+    assert L.mi355_stream_probe(None, 4096, 64, 8192, 0) == _abi.ERR_BAD_ARG       # reads that reach no store
+
+
+def test_tile_usable_names_the_kernel_that_runs():
+    """Every tile is an algorithm of its own (cf. the per-tile algorithm packs of dnn/src/cuda/conv_bias/algo.cpp:216-253):
+    a tile is usable only when exec would run that very kernel, and what the heuristic hands out is always usable."""
+    names = lib.tile_names()
+    igemm = lib.algo_names().index("MI355_IGEMM_MFMA_I8")
+
+    def usable(d):
+        return {names[t] for t in range(len(names)) if lib.tile_usable(d, t)}
+
+    d4 = _abi.make_conv_desc("NCHW4", 2, 64, 14, 14, 64, 3, pad=1, scale_bias=2e-4, scale_dst=0.05)
+    u = usable(d4)
+    assert "128x128x64" in u and not any(n.startswith(("v2_", "dma")) or n == "pw4_stream" for n in u), u
+    d32 = _abi.make_conv_desc("NCHW32", 2, 64, 14, 14, 64, 3, pad=1, has_z=True, scale_bias=2e-4, scale_z=0.05, scale_dst=0.05)
+    u = usable(d32)
+    assert {"128x128x64", "dma128x128x64", "v2_128x128x64r4", "v2_256x256x64r3w8"} <= u and not any(n.startswith("dma4_") for n in u), u
+    # 4-packed pointwise: the 4-packed LDS-direct tiles, and the streaming kernel only where it applies
+    dpw = _abi.make_conv_desc("NCHW4", 2, 16, 14, 14, 96, 1, scale_bias=2e-4, scale_dst=0.05)
+    assert {"dma4_128x128x64", "pw4_stream"} <= usable(dpw)
+    dpw2 = _abi.make_conv_desc("NCHW4", 2, 256, 14, 14, 96, 1, scale_bias=2e-4, scale_dst=0.05)
+    u = usable(dpw2)
+    assert "dma4_128x128x64" in u and "pw4_stream" not in u
+    # the general epilogue (here: a dst scale outside the fast forms) is instantiated on two second-generation tiles
+    dg = _abi.make_conv_desc("NCHW32", 1, 64, 8, 8, 64, 3, pad=1, scale_dst=1e-30)
+    assert usable(dg) == {"v2_128x128x64r4", "v2_64x128x128r3"}
+    dgrp = _abi.make_conv_desc("NCHW32", 1, 128, 8, 8, 128, 3, pad=1, group=2, scale_bias=2e-4, scale_dst=0.05)
+    u = usable(dgrp)
+    assert u and all(n.startswith("v2_") for n in u), u
+    # not an MFMA problem at all
+    ddw = _abi.make_conv_desc("NCHW4", 1, 32, 8, 8, 32, 3, pad=1, group=32)
+    assert lib.lib().mi355_igemm_tile_usable(C.byref(ddw), 0) == _abi.ERR_ALGO
+    assert lib.lib().mi355_igemm_tile_usable(C.byref(d32), len(names)) == _abi.ERR_ALGO
+    for d in (d4, d32, dpw, dpw2, dg, dgrp):
+        for req in (_abi.ALGO_HEURISTIC, _abi.ALGO_HEURISTIC_PREPROCESS, igemm):
+            a, _ = ops.conv_bias_query(d, req)
+            if a.id == igemm:
+                assert lib.tile_usable(d, a.tile_cfg), (names[a.tile_cfg], req)

@@ -77,6 +77,8 @@ def test_igemm_full_size(oracle, case):
     assert torch.equal(got, ref)
     # every tile configuration must give the same tensor
     for tile in range(len(lib.tile_names())):
+        if not lib.tile_usable(d, tile):
+            continue
         a2, _ = ops.conv_bias_query(d, IGEMM)
         a2.tile_cfg = tile
         say("  tile", lib.tile_names()[tile])

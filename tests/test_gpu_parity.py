@@ -367,6 +367,8 @@ def test_preprocessed_filter_equals_plain_filter(oracle):
             src, flt, bias, zz = util.make_tensors(d, seed=700 + ci)
             dev = [to_dev(x) for x in (src, flt, bias, zz)]
             for tile in range(len(names)):
+                if not lib.tile_usable(d, tile):
+                    continue
                 a, _ = ops.conv_bias_query(d, IGEMM)
                 a.tile_cfg = tile
                 pre = ops.conv_bias_preprocess(d, dev[1], a)
@@ -394,6 +396,30 @@ def test_preprocessed_filter_equals_plain_filter(oracle):
     # an algorithm without a pre-processed form
     a, _ = ops.conv_bias_query(d, DIRECT)
     assert ops.conv_bias_preprocess(d, to_dev(flt), a) is None
+
+
+def test_forced_tile_that_cannot_run_is_an_error(oracle):
+    """exec runs the tile it is given or refuses: a tile the caller named and that is no algorithm for the problem is
+    MI355_ERR_ALGO (so a fast-run chooser never times one kernel under two names); the same tile under the heuristic's
+    flag is replaced by the one that can run."""
+    names = lib.tile_names()
+    d = _abi.make_conv_desc("NCHW4", 2, 64, 9, 9, 64, 3, pad=1, nonline="RELU", **S)
+    src, flt, bias, z = util.make_tensors(d, seed=31)
+    want = oracle.conv_bias(d, src, flt, bias, z)
+    dev = [to_dev(x) for x in (src, flt, bias, z)]
+    bad = names.index("v2_128x128x64r4")
+    assert not lib.tile_usable(d, bad)
+    forced, _ = ops.conv_bias_query(d, IGEMM)
+    forced.tile_cfg = bad
+    with pytest.raises(lib.Mi355Error) as e:
+        ops.conv_bias_exec(d, *dev, algo=forced)
+    assert e.value.status == _abi.ERR_ALGO
+    heur, _ = ops.conv_bias_query(d)
+    assert heur.id == IGEMM
+    heur.tile_cfg = bad
+    got = ops.conv_bias_exec(d, *dev, algo=heur)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -522,7 +548,8 @@ def test_random_descriptors_every_kernel_family(oracle):
         if it % 5 == 0:
             torch.cuda.synchronize()
             assert np.array_equal(ref.cpu().numpy(), oracle.conv_bias(d, src, flt, bias, z))
-        for tile in rnd.sample(range(len(names)), 4) + [None]:
+        usable = [t for t in range(len(names)) if lib.tile_usable(d, t)]
+        for tile in rnd.sample(usable, min(4, len(usable))) + [None]:
             a, _ = ops.conv_bias_query(d, IGEMM)
             if tile is not None:
                 a.tile_cfg = tile

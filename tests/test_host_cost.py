@@ -1,0 +1,79 @@
+"""Host-side cost of one operator call (no GPU): the descriptor validation and the epilogue proofs behind query / exec.
+
+The requantisation forms are proved per scale on the host (~0.1 ms each); an operator is called once per layer per
+inference, so a proof must be paid once per scale for the life of the process and never again -- an inference loop over
+more distinct scales than some fixed cache size must not fall back to proving on every call.  The role the algorithm
+cache plays upstream (dnn/src/common/algo_chooser.h:25-49, dnn/include/megdnn/algorithm_cache.h:33-61)."""
+import ctypes as C
+import time
+
+import numpy as np
+
+from megengine_amd import _abi, lib
+
+
+def _descs(count, seed):
+    rng = np.random.RandomState(seed)
+    shapes = [(256, 56, 64, 1, 0, False), (64, 56, 64, 3, 1, False), (64, 56, 256, 1, 0, True), (512, 28, 128, 1, 0, False),
+              (128, 28, 128, 3, 1, False), (1024, 14, 256, 1, 0, False), (512, 7, 2048, 1, 0, True)]
+    out = []
+    for i in range(count):
+        ic, hw, oc, f, pad, z = shapes[i % len(shapes)]
+        s = [float(np.float32(np.exp(rng.uniform(np.log(1e-3), np.log(5e-2))))) for _ in range(4)]
+        out.append(_abi.make_conv_desc("NCHW32", 64, ic, hw, hw, oc, f, pad=pad, nonline="RELU", has_z=z,
+                                       scale_bias=float(np.float32(s[0]) * np.float32(s[1])), scale_z=s[2], scale_dst=s[3]))
+    return out
+
+
+def _best_ns(fn, repeats=5):
+    best = None
+    for _ in range(repeats):
+        t0 = time.perf_counter_ns()
+        fn()
+        t = time.perf_counter_ns() - t0
+        best = t if best is None else min(best, t)
+    return best
+
+
+def test_steady_state_query_and_canonize_stay_cheap_over_many_scales():
+    L = lib.lib()
+    descs = _descs(1200, 5)
+    assert len({(d.scale_bias, d.scale_dst) for d in descs}) >= 1000
+    algo, ws, oh, ow = _abi.Algo(), C.c_size_t(0), C.c_uint32(0), C.c_uint32(0)
+    # first pass: every scale is proved once
+    for d in descs:
+        assert L.mi355_convbias_s8_query(C.byref(d), _abi.ALGO_HEURISTIC_PREPROCESS, C.byref(algo), C.byref(ws)) == 0
+    # steady state: neighbours in the list differ, so the per-thread memo of the last descriptor never answers and
+    # every call walks the validation and both proof caches.  Best of a few repeats per call: the bound is on the
+    # work, not on what else the host was doing.
+    worst_q = worst_c = 0
+    for rep in range(2):
+        for d in descs:
+            ref = C.byref(d)
+            tq = _best_ns(lambda: L.mi355_convbias_s8_query(ref, _abi.ALGO_HEURISTIC_PREPROCESS, C.byref(algo), C.byref(ws)), 1)
+            tc = _best_ns(lambda: L.mi355_convbias_deduce_out(ref, C.byref(oh), C.byref(ow)), 1)
+            d._tq = min(getattr(d, "_tq", tq), tq)
+            d._tc = min(getattr(d, "_tc", tc), tc)
+    worst_q = max(d._tq for d in descs)
+    worst_c = max(d._tc for d in descs)
+    assert worst_q < 5000, "a steady-state query took %.1f us" % (worst_q / 1e3)
+    assert worst_c < 5000, "a steady-state canonize took %.1f us" % (worst_c / 1e3)
+
+
+def test_repeated_descriptor_is_answered_from_the_memo():
+    L = lib.lib()
+    d = _descs(1, 9)[0]
+    oh, ow = C.c_uint32(0), C.c_uint32(0)
+    assert L.mi355_convbias_deduce_out(C.byref(d), C.byref(oh), C.byref(ow)) == 0
+    assert (oh.value, ow.value) == (56, 56)
+    # a changed field must not be answered with the remembered form
+    d.ih = 28
+    d.iw = 28
+    assert L.mi355_convbias_deduce_out(C.byref(d), C.byref(oh), C.byref(ow)) == 0
+    assert (oh.value, ow.value) == (28, 28)
+    d.scale_dst = 0.0
+    algo, ws = _abi.Algo(), C.c_size_t(0)
+    assert L.mi355_convbias_s8_query(C.byref(d), _abi.ALGO_HEURISTIC, C.byref(algo), C.byref(ws)) == 0
+    # an invalid descriptor after a valid one is still rejected
+    d.group = 0
+    assert L.mi355_convbias_deduce_out(C.byref(d), C.byref(oh), C.byref(ow)) == _abi.ERR_BAD_ARG
