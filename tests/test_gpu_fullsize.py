@@ -18,13 +18,13 @@ pytestmark = pytest.mark.gpu
 DIRECT, IGEMM, DW, C4 = 0, 1, 2, 3
 
 
-def dev_tensors(d, seed):
+def dev_tensors(d, seed, bias_range=(-1000, 1000)):
     g = torch.Generator(device="cuda")
     g.manual_seed(seed)
     ss, fs, bs, ds = _abi.conv_shapes(d)
     src = torch.randint(-128, 128, ss, dtype=torch.int8, device="cuda", generator=g)
     flt = torch.randint(-127, 128, fs, dtype=torch.int8, device="cuda", generator=g)
-    bias = torch.randint(-1000, 1001, bs, dtype=torch.int32, device="cuda", generator=g)
+    bias = torch.randint(int(bias_range[0]), int(bias_range[1]) + 1, bs, dtype=torch.int32, device="cuda", generator=g)
     z = torch.randint(-128, 128, ds, dtype=torch.int8, device="cuda", generator=g) if d.has_z else None
     return src, flt, bias, z
 
@@ -94,6 +94,49 @@ def test_igemm_full_size(oracle, case):
         assert torch.equal(noz, zero)
 
 
+def live_scales(k, nonline):
+    """Scales and a bias range that keep most outputs strictly inside the int8 range: uniform int8 operands give an
+    accumulator of spread sigma = 73.9 * 73.3 * sqrt(K); the dst scale puts sigma at 25 output steps, the bias sits
+    around +1.6 sigma (so that RELU keeps most values), the residual contributes at most +-32 steps."""
+    sigma = 73.9 * 73.3 * k ** 0.5
+    s_bias = 2e-4
+    s_dst = float(np.float32(s_bias * sigma / 25.0))
+    return dict(scale_bias=s_bias, scale_dst=s_dst, scale_z=0.25 * s_dst), (1.3 * sigma, 1.9 * sigma)
+
+
+@pytest.mark.parametrize("case", FULL_CASES, ids=[c[0] for c in FULL_CASES])
+def test_igemm_full_size_on_live_values(oracle, case):
+    """The full-size cases again with scales derived from the reduction length: with the fixed 2e-4 / 0.05 pair a long
+    reduction saturates most outputs, and a wrong accumulator in a few lanes would hide behind the clamp."""
+    name, fmt, n, ic, hw, oc, f, stride, pad, nl, z = case
+    scales, bias_range = live_scales(ic * f * f, nl)
+    d = _abi.make_conv_desc(fmt, n, ic, hw, hw, oc, f, stride=stride, pad=pad, nonline=nl, has_z=z, **scales)
+    say("full-size live", case, scales)
+    src, flt, bias, zt = dev_tensors(d, 19, bias_range)
+    ref = ops.conv_bias_exec(d, src, flt, bias, zt, algo=DIRECT)
+    torch.cuda.synchronize()
+    lo = 0 if nl == "RELU" else -128
+    live = float(((ref > lo) & (ref < 127)).float().mean())
+    say("  live outputs %.3f" % live)
+    assert live >= 0.75
+    spot_check(oracle, d, src, flt, bias, zt, ref)
+    algo, _ = ops.conv_bias_query(d)
+    got = ops.conv_bias_exec(d, src, flt, bias, zt, algo=algo)
+    torch.cuda.synchronize()
+    assert torch.equal(got, ref)
+    if algo.id != IGEMM:
+        return
+    for tile in range(len(lib.tile_names())):
+        if not lib.tile_usable(d, tile):
+            continue
+        a2, _ = ops.conv_bias_query(d, IGEMM)
+        a2.tile_cfg = tile
+        say("  tile", lib.tile_names()[tile])
+        out = ops.conv_bias_exec(d, src, flt, bias, zt, algo=a2)
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref), lib.tile_names()[tile]
+
+
 def test_relu_property_full_size():
     d_id = _abi.make_conv_desc("NCHW32", 64, 64, 56, 56, 64, 3, pad=1, nonline="IDENTITY", scale_bias=2e-4, scale_dst=0.05)
     d_re = _abi.make_conv_desc("NCHW32", 64, 64, 56, 56, 64, 3, pad=1, nonline="RELU", scale_bias=2e-4, scale_dst=0.05)
@@ -119,4 +162,16 @@ def test_depthwise_full_size(oracle):
         spot_check(oracle, d, src, flt, bias, None, got, npoints=20000)
         ref = ops.conv_bias_exec(d, src, flt, bias, None, algo=DIRECT)
         torch.cuda.synchronize()
+        assert torch.equal(got, ref)
+        # the same layer on live values (9 taps: sigma = 16 250; a bias around +1.6 sigma keeps RELU from zeroing half)
+        scales, bias_range = live_scales(9, "RELU")
+        d = _abi.make_conv_desc("NCHW4", 64, c, hw, hw, c, 3, group=c, stride=stride, pad=1, nonline="RELU", **scales)
+        src, flt, bias, _ = dev_tensors(d, 29, bias_range)
+        got = ops.conv_bias_exec(d, src, flt, bias, None, algo=algo)
+        ref = ops.conv_bias_exec(d, src, flt, bias, None, algo=DIRECT)
+        torch.cuda.synchronize()
+        live = float(((ref > 0) & (ref < 127)).float().mean())
+        say("  live outputs %.3f" % live)
+        assert live >= 0.75
+        spot_check(oracle, d, src, flt, bias, None, got, npoints=20000)
         assert torch.equal(got, ref)

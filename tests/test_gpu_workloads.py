@@ -74,6 +74,29 @@ def test_config2_resnet50_stack(oracle, resnet_plan, part):
         check_layer(oracle, plan[i], seed=1000 + i)
 
 
+@pytest.fixture(scope="module")
+def resnet_live_plan():
+    """The same 53 layers, tensors and algorithm choices with scales and biases calibrated layer by layer so that the
+    compared bytes are live values: with the bench's scale recipe most outputs of a long reduction sit at a clamp (0 or
+    127), where a wrong accumulator in a minority of lanes would hide."""
+    torch.manual_seed(1234)
+    plan = workloads.build_stack(workloads.resnet50(64), 7)
+    live = workloads.run_calibrated(plan, 77)
+    yield plan, live
+    del plan
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("part", range(6))
+def test_config2_resnet50_stack_on_live_values(oracle, resnet_live_plan, part):
+    plan, live = resnet_live_plan
+    assert len(plan) == 53
+    for i in range(part, len(plan), 6):
+        say("live outputs", plan[i]["layer"].name, "%.3f" % live[i])
+        assert live[i] >= 0.75, (plan[i]["layer"].name, live[i])
+        check_layer(oracle, plan[i], seed=5000 + i)
+
+
 def test_config2_uses_preprocessed_filters(resnet_plan):
     n = sum(p.get("pre") is not None for p in resnet_plan)
     say(n, "of 53 layers run with a pre-processed filter")
@@ -145,6 +168,29 @@ def mobilenet_plan():
     yield plan
     del plan
     torch.cuda.empty_cache()
+
+
+@pytest.fixture(scope="module")
+def mobilenet_live_plan():
+    torch.manual_seed(4321)
+    plan = workloads.build_stack(workloads.mobilenet_v2(), 3)
+    live = workloads.run_calibrated(plan, 33)
+    yield plan, live
+    del plan
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("part", range(4))
+def test_config3_mobilenetv2_on_live_values(oracle, mobilenet_live_plan, part):
+    """Calibrated scales: the depthwise kernel, the 4-packed pointwise tiles and the streaming kernel at full size on
+    values inside the int8 range."""
+    plan, live = mobilenet_live_plan
+    for i in range(part, len(plan), 4):
+        p = plan[i]
+        say("live outputs", p["layer"].name, "%.3f" % live[i])
+        assert live[i] >= 0.75, (p["layer"].name, live[i])
+        assert p["algo"].id == (DW if p["layer"].group > 1 else IGEMM)
+        check_layer(oracle, p, seed=6000 + i)
 
 
 @pytest.mark.parametrize("part", range(4))
