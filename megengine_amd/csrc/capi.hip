@@ -372,7 +372,7 @@ int cu_count() {
 }
 
 const char* kAlgoNames[ALGO_COUNT] = {"MI355_DIRECT_DOT4", "MI355_IGEMM_MFMA_I8", "MI355_DEPTHWISE_DOT4",
-                                      "MI355_C4_MFMA_I8"};
+                                      "MI355_C4_MFMA_I8", "MI355_NCHW_RELAYOUT_MFMA_I8"};
 
 bool algo_usable(const ConvProblem& p, int id) {
     switch (id) {
@@ -380,19 +380,28 @@ bool algo_usable(const ConvProblem& p, int id) {
         case ALGO_IGEMM_MFMA: return igemm_usable(p);
         case ALGO_DEPTHWISE: return depthwise_usable(p);
         case ALGO_C4_MFMA: return c4_usable(p);
+        case ALGO_NCHW_MFMA: return nchw_mfma_usable(p);
         default: return false;
     }
 }
 
 // Heuristic order (cf. the reference's per-backend get_algorithm_heuristic, e.g.
 // dnn/src/cuda/conv_bias/opr_impl.cpp:44-238): channel-wise kernel, the 4-channel first-layer kernel,
-// then the MFMA implicit GEMM, then the generic direct kernel.
-int pick_algo(const ConvProblem& p) {
+// then the MFMA implicit GEMM, then the generic direct kernel.  Plain NCHW takes the relayout + MFMA algorithm once
+// the problem is large enough to pay for its five extra launches (the generic kernel runs ~4 M multiply-adds in the time
+// those take); workspace_limit is get_algorithm_heuristic's (dnn/include/megdnn/oprs/base.h:595-614).
+int pick_algo(const ConvProblem& p, size_t workspace_limit = SIZE_MAX) {
     if (depthwise_usable(p)) return ALGO_DEPTHWISE;
     if (c4_usable(p)) return ALGO_C4_MFMA;
     if (igemm_usable(p)) return ALGO_IGEMM_MFMA;
+    if (p.d.format == MI355_FMT_NCHW) {
+        const uint64_t macs = (uint64_t)p.d.n * p.d.oc * p.oh * p.ow * p.icpg * p.d.fh * p.d.fw;
+        if (macs >= (1ull << 22) && nchw_mfma_usable(p) && nchw_mfma_workspace(p) <= workspace_limit) return ALGO_NCHW_MFMA;
+    }
     return ALGO_DIRECT;
 }
+
+size_t algo_workspace(const ConvProblem& p, int id) { return id == ALGO_NCHW_MFMA ? nchw_mfma_workspace(p) : 0; }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -481,14 +490,15 @@ int mi355_convbias_s8_query(const mi355_conv_desc* d, int algo_request, mi355_al
         // one the caller asked for by id may not
         algo_out->reserved = algo_request == MI355_ALGO_HEURISTIC || pre ? MI355_ALGO_FLAG_HEURISTIC : 0;
     }
-    // every kernel reads the reference layouts in place: no filter repack, no float staging
-    if (workspace_bytes) *workspace_bytes = 0;
+    // the packed-format kernels read the reference layouts in place (no filter repack, no float staging): 0 bytes;
+    // the plain-NCHW algorithm keeps its packed intermediates in the workspace
+    if (workspace_bytes) *workspace_bytes = algo_workspace(p, id);
     return MI355_OK;
 }
 
 // filter: the reference layout, or (preprocessed) the artefact of mi355_convbias_s8_preprocess for this algorithm
 static int exec_impl(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src, const int8_t* filter,
-                     bool preprocessed, const int32_t* bias, const int8_t* z, void* dst) {
+                     bool preprocessed, const int32_t* bias, const int8_t* z, void* dst, void* workspace, size_t workspace_bytes) {
     ConvProblem p;
     int st = canonize(d, &p);
     if (st) return st;
@@ -498,11 +508,19 @@ static int exec_impl(void* stream, const mi355_conv_desc* d, const mi355_algo* a
     int id = algo ? algo->id : MI355_ALGO_HEURISTIC;
     int cfg = algo ? algo->tile_cfg : -1;
     if (id == MI355_ALGO_HEURISTIC) {
-        id = pick_algo(p);
+        id = pick_algo(p, workspace ? workspace_bytes : 0);  // whatever fits the workspace the caller brought
         cfg = -1;
     }
     if (id < 0 || id >= ALGO_COUNT) return fail(MI355_ERR_ALGO, "unknown algorithm id %d", id);
     if (!algo_usable(p, id)) return fail(MI355_ERR_ALGO, "%s cannot run this problem", kAlgoNames[id]);
+    // check_exec's workspace rule (dnn/src/common/conv_bias.cpp:32-37)
+    const size_t ws_need = algo_workspace(p, id);
+    if (ws_need) {
+        if (!workspace || workspace_bytes < ws_need)
+            return fail(MI355_ERR_WORKSPACE, "workspace of %zu bytes, %s needs %zu", workspace ? workspace_bytes : (size_t)0,
+                        kAlgoNames[id], ws_need);
+        if (!aligned16(workspace)) return fail(MI355_ERR_BAD_ARG, "the workspace needs 16-byte alignment");
+    }
     const bool by_heuristic = !algo || algo->id == MI355_ALGO_HEURISTIC || (algo->reserved & MI355_ALGO_FLAG_HEURISTIC);
     if (id == ALGO_IGEMM_MFMA) {
         if (cfg < 0 || cfg >= igemm_num_cfgs()) {
@@ -520,7 +538,7 @@ static int exec_impl(void* stream, const mi355_conv_desc* d, const mi355_algo* a
     if (preprocessed && (id != ALGO_IGEMM_MFMA || igemm_preprocessed_bytes(p, cfg) == 0))
         return fail(MI355_ERR_ALGO, "this algorithm has no pre-processed filter form");
     // the tiled kernels use 16-byte vector accesses; misaligned tensors take the generic kernel
-    if (id != ALGO_DIRECT) {
+    if (id != ALGO_DIRECT && id != ALGO_NCHW_MFMA) {  // (the relayouts of plain NCHW tensors take any pointer)
         // (pack-32 tensors move as 16-byte vectors, pack-4 tensors as dwords)
         const int sa = p.pin == 32 ? 16 : 4, da = p.pout == 32 ? 16 : 4;
         bool al = aligned16(src) && aligned16(filter) && aligned16(dst) && (!bias || aligned16(bias)) &&
@@ -547,6 +565,9 @@ static int exec_impl(void* stream, const mi355_conv_desc* d, const mi355_algo* a
         case ALGO_C4_MFMA:
             rc = launch_conv_c4(hs, p, cu_count(), src, filter, bias, z, reinterpret_cast<int8_t*>(dst));
             break;
+        case ALGO_NCHW_MFMA:
+            rc = launch_conv_nchw_mfma(hs, p, cu_count(), src, filter, bias, z, reinterpret_cast<int8_t*>(dst), workspace);
+            break;
     }
     if (rc) return fail(MI355_ERR_LAUNCH, "%s: %s", kAlgoNames[id], hipGetErrorString((hipError_t)rc));
     return MI355_OK;
@@ -555,9 +576,7 @@ static int exec_impl(void* stream, const mi355_conv_desc* d, const mi355_algo* a
 int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src,
                            const int8_t* filter, const int32_t* bias, const int8_t* z, void* dst, void* workspace,
                            size_t workspace_bytes) {
-    (void)workspace;
-    (void)workspace_bytes;
-    return exec_impl(stream, d, algo, src, filter, false, bias, z, dst);
+    return exec_impl(stream, d, algo, src, filter, false, bias, z, dst, workspace, workspace_bytes);
 }
 
 // ---- weight pre-processing ----
@@ -599,8 +618,6 @@ int mi355_convbias_s8_preprocess(void* stream, const mi355_conv_desc* d, const m
 int mi355_convbias_s8_exec_preprocessed(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src,
                                         const void* preprocessed, size_t preprocessed_bytes, const int32_t* bias,
                                         const int8_t* z, void* dst, void* workspace, size_t workspace_bytes) {
-    (void)workspace;
-    (void)workspace_bytes;
     ConvProblem p;
     size_t need = 0;
     int st = preprocess_problem(d, algo, &p, &need);
@@ -608,7 +625,8 @@ int mi355_convbias_s8_exec_preprocessed(void* stream, const mi355_conv_desc* d, 
     if (need == 0) return fail(MI355_ERR_ALGO, "this algorithm has no pre-processed filter form");
     if (preprocessed_bytes < need)
         return fail(MI355_ERR_WORKSPACE, "pre-processed filter of %zu bytes, %zu needed", preprocessed_bytes, need);
-    return exec_impl(stream, d, algo, src, reinterpret_cast<const int8_t*>(preprocessed), true, bias, z, dst);
+    return exec_impl(stream, d, algo, src, reinterpret_cast<const int8_t*>(preprocessed), true, bias, z, dst, workspace,
+                     workspace_bytes);
 }
 
 int mi355_convbias_s8_profile(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src,

@@ -15,7 +15,8 @@ enum AlgoId {
     ALGO_IGEMM_MFMA = 1,   // dense implicit GEMM on int8 MFMA (NCHW4 / NCHW32 / mixed)
     ALGO_DEPTHWISE = 2,    // channel-wise, bandwidth bound (NCHW4-packed and NCHW)
     ALGO_C4_MFMA = 3,      // first layers: NCHW4 with 4 input channels, patch-staged MFMA
-    ALGO_COUNT = 4
+    ALGO_NCHW_MFMA = 4,    // plain NCHW: relayout into the workspace, the NCHW32 MFMA kernel, relayout back
+    ALGO_COUNT = 5
 };
 
 // Canonical problem description used by every launcher (derived from mi355_conv_desc)
@@ -58,6 +59,12 @@ int launch_conv_depthwise(hipStream_t st, const ConvProblem& p, const int8_t* sr
 bool c4_usable(const ConvProblem& p);
 int launch_conv_c4(hipStream_t st, const ConvProblem& p, int cu_count, const int8_t* src, const int8_t* flt,
                    const int32_t* bias, const int8_t* z, int8_t* dst);
+
+// plain NCHW through the caller's workspace (conv_nchw.hip); nchw_mfma_workspace is 0 when the algorithm cannot run
+bool nchw_mfma_usable(const ConvProblem& p);
+size_t nchw_mfma_workspace(const ConvProblem& p);
+int launch_conv_nchw_mfma(hipStream_t st, const ConvProblem& p, int cu_count, const int8_t* src, const int8_t* flt,
+                          const int32_t* bias, const int8_t* z, int8_t* dst, void* workspace);
 
 int launch_requant(hipStream_t st, const EpiParams& e, const int32_t* src, const int8_t* z, int8_t* dst, uint64_t count,
                    int cu_count);

@@ -489,11 +489,32 @@ static bool igemm_needs_general(const ConvProblem& p) {
     return p.d.dst_dtype != MI355_DT_QS8 || p.d.bias_mode == MI355_BIAS_FULL || !p.epi.fast;
 }
 
+// NCHW4 group convolution with whole channel blocks of 4 per group on both sides (the reference's NCHW4 group filter
+// (G, OCpg, ICpg/4, FH, FW, 4), dnn/src/common/convolution.cpp:392-407): every group is a dense NCHW4 convolution on
+// batch-strided views of src, dst and z, with its own contiguous piece of filter and bias -- one launch of the dense
+// tiles per group, the way the reference's CUDA backend runs group convolutions over a dense algorithm
+// (dnn/src/cuda/conv_bias/group_conv.cpp:10-44,76-104).
+constexpr uint32_t kMaxGroupLaunches = 1024;
+static bool igemm_group_by_launch(const ConvProblem& p) {
+    const mi355_conv_desc& d = p.d;
+    return d.format == MI355_FMT_NCHW4 && d.group > 1 && d.group <= kMaxGroupLaunches && !p.dw4 && p.icpg % 4 == 0 &&
+           p.ocpg % 4 == 0 && !igemm_needs_general(p);
+}
+static ConvProblem igemm_group_view(const ConvProblem& p) {
+    ConvProblem q = p;
+    q.d.group = 1;
+    q.d.sparse = MI355_SPARSE_DENSE;
+    q.d.ic = p.icpg;
+    q.d.oc = p.ocpg;
+    return q;  // batch strides stay those of the whole tensors
+}
+
 bool igemm_usable(const ConvProblem& p) {
     const mi355_conv_desc& d = p.d;
     if (p.dw4) return false;
-    // group convolution: 32-packed tensors whose groups are whole channel blocks (second-generation tiles only)
-    if (d.group != 1 && !(p.pin == 32 && p.icpg % 32 == 0 && p.ocpg % 32 == 0)) return false;
+    // group convolution: 32-packed tensors whose groups are whole channel blocks (second-generation tiles only), or
+    // NCHW4 with whole blocks of 4 on both sides, one dense launch per group (igemm_group_view)
+    if (d.group != 1 && !(p.pin == 32 && p.icpg % 32 == 0 && p.ocpg % 32 == 0) && !igemm_group_by_launch(p)) return false;
     if (d.format != MI355_FMT_NCHW4 && d.format != MI355_FMT_NCHW32 && d.format != MI355_FMT_NCHW4_NCHW32 &&
         d.format != MI355_FMT_NCHW32_NCHW4)
         return false;
@@ -502,7 +523,6 @@ bool igemm_usable(const ConvProblem& p) {
     // second-generation tiles with their general epilogue: 32-packed inputs only
     if (igemm_needs_general(p)) {
         if (p.pin != 32) return false;
-        if (d.dst_dtype == MI355_DT_QS32 && d.has_z) return false;
         if (d.dst_dtype == MI355_DT_F32) return false;
     }
     if (d.fh > 255 || d.fw > 255 || d.pad_h > 0xfff || d.pad_w > 0xfff || d.ih > 0x3000 || d.iw > 0x3000) return false;
@@ -623,6 +643,7 @@ int launch_igemm_preprocess(hipStream_t st, const ConvProblem& p, const int8_t* 
 
 // The chooser's tile, as the launch code will run it: what query() hands out names the kernel that executes.
 int igemm_pick_cfg(const ConvProblem& p, int cu_count, bool will_preprocess) {
+    if (igemm_group_by_launch(p)) return igemm_pick_cfg(igemm_group_view(p), cu_count, will_preprocess);
     const int c = pick_cfg_by_shape(p, cu_count, will_preprocess);
     const int r = igemm_resolve_cfg(p, c);
     return r >= 0 ? r : c;
@@ -675,6 +696,7 @@ static int staged_tile_of_shape(int bm, int bn, int kch) {
 
 int igemm_resolve_cfg(const ConvProblem& p, int cfg) {
     if (cfg < 0 || cfg >= igemm_num_cfgs()) return -1;
+    if (igemm_group_by_launch(p)) return igemm_resolve_cfg(igemm_group_view(p), cfg);
     const mi355_conv_desc& d = p.d;
     IgemmArgs a;
     igemm_fill_args(p, a);
@@ -718,6 +740,20 @@ int igemm_resolve_cfg(const ConvProblem& p, int cfg) {
 
 int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_count, const int8_t* src,
                       const int8_t* flt, const int32_t* bias, const int8_t* z, int8_t* dst, bool flt_preprocessed) {
+    if (igemm_group_by_launch(p)) {
+        if (flt_preprocessed) return (int)hipErrorInvalidValue;
+        const ConvProblem q = igemm_group_view(p);
+        const mi355_conv_desc& d = p.d;
+        const int64_t src_g = (int64_t)p.icpg * d.ih * d.iw, dst_g = (int64_t)p.ocpg * p.oh * p.ow;
+        const int64_t flt_g = (int64_t)p.ocpg * p.icpg * d.fh * d.fw;
+        for (uint32_t g = 0; g < d.group; ++g) {
+            const int rc = launch_conv_igemm(st, q, cfg, cu_count, src + g * src_g, flt + g * flt_g,
+                                             bias ? bias + (int64_t)g * p.ocpg : nullptr, z ? z + g * dst_g : nullptr,
+                                             dst + g * dst_g, false);
+            if (rc) return rc;
+        }
+        return 0;
+    }
     IgemmArgs a;
     igemm_fill_args(p, a);
     a.src = src; a.flt = flt; a.bias = bias; a.z = z; a.dst = dst;

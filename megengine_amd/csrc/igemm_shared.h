@@ -199,7 +199,7 @@ __device__ __forceinline__ void igemm_run_epilogue(const IgemmArgs& a, v16i (&ac
 // General epilogue of one wave tile: every dst dtype / bias shape / scale the operator accepts, with the literal
 // requantisation chain where the fast forms do not apply.  Register quad q of a 32x32 block holds channels
 // ocb + 8q + 4 (lane / 32) .. + 3 of pixel lane % 32: one dword of int8 results, or 16 bytes of int32 results.
-// QuantizedS32 dst (no residual here): the reference accumulates in dst itself, IDENTITY stores the raw sum, the
+// QuantizedS32 dst: the reference accumulates in dst itself, IDENTITY stores the raw sum, the
 // activations dequantise with the scale of dst (e.s_b holds it; naive/conv_bias/opr_impl.cpp:223-228,52,69-73,89-93).
 template <int POUT, int MT, int NT>
 __device__ __forceinline__ void igemm_epilogue_general(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w, int l32,
@@ -229,9 +229,12 @@ __device__ __forceinline__ void igemm_epilogue_general(const IgemmArgs& a, v16i 
                 }
                 if (a.dst_s32) {
                     v4i o = {v[0], v[1], v[2], v[3]};
-                    if (a.epi.nonline != NL_IDENTITY) {
+                    if (hz || a.epi.nonline != NL_IDENTITY) {
+                        // a residual of a QuantizedS32 dst is QuantizedS32 itself (z has the dtype of dst)
+                        v4i zq = {0, 0, 0, 0};
+                        if (hz) zq = *reinterpret_cast<const v4i*>(reinterpret_cast<const int*>(a.z) + (int64_t)n * a.z_sn + in_img);
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) o[r] = requant_s32_exact(v[r], false, 0, a.epi);
+                        for (int r = 0; r < 4; ++r) o[r] = requant_s32_exact(v[r], hz, zq[r], a.epi);
                     }
                     *reinterpret_cast<v4i*>(reinterpret_cast<int*>(a.dst) + (int64_t)n * a.dst_sn + in_img) = o;
                 } else {

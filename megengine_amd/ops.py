@@ -57,7 +57,7 @@ def conv_bias_exec(desc, src, flt, bias=None, z=None, dst=None, algo=None, works
     elif isinstance(algo, int):
         algo, ws_bytes = conv_bias_query(desc, algo)
     else:
-        ws_bytes = 0
+        ws_bytes = conv_bias_query(desc, algo.id)[1] if workspace is None and algo.id >= 0 else 0
     if dst is None:
         shape = _abi.conv_shapes(desc)[3]
         dt = {_abi.DT_QS8: torch.int8, _abi.DT_QS32: torch.int32, _abi.DT_F32: torch.float32}[desc.dst_dtype]

@@ -13,6 +13,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <functional>
 #include <string>
 #include <vector>
@@ -118,6 +119,9 @@ static std::vector<Case> cases() {
          2, 16, 8, 8, 10, 3, 3, 1},
         {"nchw dense", F::NCHW, S::DENSE, N::RELU, {2, 5, 9, 9}, {7, 5, 3, 3}, 1, 1, true, true, false,
          2, 5, 9, 9, 7, 3, 3, 1},
+        // large enough for the heuristic to take the relayout + MFMA algorithm, which needs a workspace
+        {"nchw dense, workspace", F::NCHW, S::DENSE, N::RELU, {4, 24, 28, 28}, {40, 24, 3, 3}, 1, 1, true, true, false,
+         4, 24, 28, 28, 40, 3, 3, 1},
         {"nchw depthwise", F::NCHW, S::GROUP, N::RELU, {2, 6, 9, 9}, {6, 1, 1, 3, 3}, 1, 2, true, false, false,
          2, 6, 9, 9, 6, 3, 3, 6},
         {"nchw44 channel-wise", F::NCHW44, S::GROUP, N::RELU, {2, 3, 9, 9, 4}, {3, 1, 1, 3, 3, 4}, 1, 1, true, false, false,
@@ -180,6 +184,24 @@ static void run_conv_case(Handle* h, const Case& c, bool on_gpu) {
     bool listed = false;
     for (auto& a : algos) listed = listed || a.desc.id == heur.desc.id;
     EXPECT(listed, "heuristic algorithm %s is not in the list", heur.name.c_str());
+    {
+        // get_workspace_in_bytes is the C ABI's number for the heuristic's algorithm; only the plain-NCHW relayout
+        // algorithm needs one
+        size_t abi_ws = 0;
+        mi355_algo qa;
+        EXPECT(mi355_convbias_s8_query(&d, MI355_ALGO_HEURISTIC, &qa, &abi_ws) == MI355_OK && abi_ws == ws,
+               "workspace: C++ %zu, C ABI %zu", ws, abi_ws);
+        const bool relayout_algo = heur.name.find("NCHW_RELAYOUT") != std::string::npos;
+        EXPECT((ws > 0) == relayout_algo, "workspace %zu for %s", ws, heur.name.c_str());
+        if (!strcmp(c.name, "nchw dense, workspace")) EXPECT(relayout_algo, "heuristic for a large NCHW problem: %s", heur.name.c_str());
+    }
+    // the largest workspace any listed algorithm asks for
+    size_t ws_all = ws;
+    for (auto& a : algos) {
+        opr->execution_policy().algo = a.desc;
+        ws_all = std::max(ws_all, opr->get_workspace_in_bytes(src, flt, bias, z, dst));
+    }
+    opr->execution_policy().algo = AlgorithmDesc{};
     if (!on_gpu) return;
 
     std::vector<int8_t> hsrc(src.total_nr_elems()), hflt(flt.total_nr_elems()), hz(z.total_nr_elems());
@@ -194,7 +216,7 @@ static void run_conv_case(Handle* h, const Case& c, bool on_gpu) {
                                 c.has_z ? hz.data() : nullptr, expect.data());
     EXPECT(st == 0, "CPU checker refused the case: %d", st);
 
-    DevBuf dsrc(hsrc.size()), dflt(hflt.size()), dbias(hbias.size() * 4), dz(hz.size()), ddst(dst_bytes), dws(ws);
+    DevBuf dsrc(hsrc.size()), dflt(hflt.size()), dbias(hbias.size() * 4), dz(hz.size()), ddst(dst_bytes), dws(ws_all);
     HIP_OK(hipMemcpy(dsrc.p, hsrc.data(), hsrc.size(), hipMemcpyHostToDevice));
     HIP_OK(hipMemcpy(dflt.p, hflt.data(), hflt.size(), hipMemcpyHostToDevice));
     if (c.has_bias) HIP_OK(hipMemcpy(dbias.p, hbias.data(), hbias.size() * 4, hipMemcpyHostToDevice));
@@ -205,9 +227,15 @@ static void run_conv_case(Handle* h, const Case& c, bool on_gpu) {
         HIP_OK(hipMemset(ddst.p, 0x5a, dst_bytes));
         opr->execution_policy().algo = a.desc;
         size_t need = opr->get_workspace_in_bytes(src, flt, bias, z, dst);
-        EXPECT(need <= ws || need == 0, "algorithm %s wants a larger workspace", a.name.c_str());
+        if (need > 0) {
+            // check_exec's rule (dnn/src/common/conv_bias.cpp:32-37): a workspace smaller than reported is an error
+            EXPECT(throws([&] {
+                       opr->exec(TensorND(dsrc.p, src), TensorND(dflt.p, flt), TensorND(dbias.p, bias), TensorND(dz.p, z),
+                                 TensorND(ddst.p, dst), nullptr, Workspace(dws.p, need - 1));
+                   }, MI355_ERR_WORKSPACE), "%s must refuse a short workspace", a.name.c_str());
+        }
         opr->exec(TensorND(dsrc.p, src), TensorND(dflt.p, flt), TensorND(dbias.p, bias), TensorND(dz.p, z),
-                  TensorND(ddst.p, dst), nullptr, Workspace(dws.p, ws));
+                  TensorND(ddst.p, dst), nullptr, Workspace(dws.p, need));
         HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
         HIP_OK(hipMemcpy(got.data(), ddst.p, dst_bytes, hipMemcpyDeviceToHost));
         size_t bad = 0;

@@ -39,7 +39,8 @@ def test_status_strings():
 
 def test_algorithm_table():
     names = lib.algo_names()
-    assert names == ["MI355_DIRECT_DOT4", "MI355_IGEMM_MFMA_I8", "MI355_DEPTHWISE_DOT4", "MI355_C4_MFMA_I8"]
+    assert names == ["MI355_DIRECT_DOT4", "MI355_IGEMM_MFMA_I8", "MI355_DEPTHWISE_DOT4", "MI355_C4_MFMA_I8",
+                     "MI355_NCHW_RELAYOUT_MFMA_I8"]
     assert lib.lib().mi355_convbias_algo_name(17) is None
     assert len(lib.tile_names()) >= 3
 
@@ -181,3 +182,34 @@ def test_tile_usable_names_the_kernel_that_runs():
             a, _ = ops.conv_bias_query(d, req)
             if a.id == igemm:
                 assert lib.tile_usable(d, a.tile_cfg), (names[a.tile_cfg], req)
+
+
+def test_plain_nchw_reports_a_workspace():
+    """Format::NCHW runs relayout -> NCHW32 MFMA kernel -> relayout through the caller's workspace: query reports its
+    size (get_workspace_in_bytes, dnn/include/megdnn/oprs/nn.h:419-422), the packed-format algorithms report 0."""
+    names = lib.algo_names()
+    nchw = names.index("MI355_NCHW_RELAYOUT_MFMA_I8")
+    up = lambda x: (x + 255) // 256 * 256
+    d = _abi.make_conv_desc("NCHW", 4, 24, 28, 28, 40, 3, pad=1, nonline="RELU", has_z=True, scale_bias=2e-4, scale_z=0.05,
+                            scale_dst=0.05)
+    a, ws = ops.conv_bias_query(d)
+    assert a.id == nchw
+    # src and filter with 24 -> 32 channels, dst and z with 40 -> 64 channels, the padded bias
+    assert ws == up(4 * 32 * 28 * 28) + up(64 * 32 * 9) + 2 * up(4 * 64 * 28 * 28) + up(64 * 4)
+    assert ops.conv_bias_query(d, 0)[1] == 0
+    # whole blocks on both sides, no residual: three tensors
+    d = _abi.make_conv_desc("NCHW", 4, 64, 14, 14, 128, 1, scale_bias=2e-4, scale_dst=0.05)
+    a, ws = ops.conv_bias_query(d)
+    assert a.id == nchw and ws == up(4 * 64 * 196) + up(128 * 64) + up(4 * 128 * 196)
+    # small problems, dilation, flipped filters, groups that split a channel block, QuantizedS32 dst: the generic kernel
+    for kw in (dict(n=1, ic=8, hw=8, oc=8), dict(dilate=2), dict(mode=_abi.MODE_CONVOLUTION), dict(group=2, ic=32, oc=32),
+               dict(dst_dtype=_abi.DT_QS32)):
+        kw = dict(kw)
+        n, ic, hw, oc = kw.pop("n", 4), kw.pop("ic", 24), kw.pop("hw", 28), kw.pop("oc", 40)
+        d = _abi.make_conv_desc("NCHW", n, ic, hw, hw, oc, 3, pad=1, scale_bias=2e-4, scale_dst=0.05, **kw)
+        a, ws = ops.conv_bias_query(d)
+        assert (a.id, ws) == (0, 0), kw
+    # groups of whole 32-channel blocks stay on the MFMA path
+    d = _abi.make_conv_desc("NCHW", 2, 64, 14, 14, 128, 3, pad=1, group=2, scale_bias=2e-4, scale_dst=0.05)
+    assert ops.conv_bias_query(d)[0].id == nchw
+    assert lib.lib().mi355_convbias_algo_usable(C.byref(_abi.make_conv_desc("NCHW32", 2, 64, 14, 14, 128, 1)), nchw) == _abi.ERR_ALGO

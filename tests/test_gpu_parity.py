@@ -309,8 +309,14 @@ def test_heuristic_picks(oracle):
     d = _abi.make_conv_desc("NCHW32", 1, 64, 8, 8, 64, 3, pad=1, group=2)
     a = ops.conv_bias_query(d)[0]
     assert a.id == IGEMM and lib.tile_names()[a.tile_cfg].startswith("v2_")
+    # NCHW4 groups of whole blocks of 4: the dense MFMA tiles, one launch per group; groups that split a block of 4 do
+    # not exist in the format (dnn/src/common/convolution.cpp:392-407)
     d = _abi.make_conv_desc("NCHW4", 1, 32, 8, 8, 32, 3, pad=1, group=4)
-    assert ops.conv_bias_query(d)[0].id == DIRECT
+    assert ops.conv_bias_query(d)[0].id == IGEMM
+    # plain NCHW: relayout + MFMA through the workspace once the problem pays for the extra launches
+    d = _abi.make_conv_desc("NCHW", 8, 64, 28, 28, 64, 3, pad=1)
+    a, ws = ops.conv_bias_query(d)
+    assert lib.algo_names()[a.id] == "MI355_NCHW_RELAYOUT_MFMA_I8" and ws > 0
     # 4-packed pointwise layers at batch 64: streaming kernel for the expansions and the narrow projections, LDS-direct
     # tiles for the long reductions on few pixels, register-staged tiles elsewhere
     names = lib.tile_names()
@@ -333,6 +339,9 @@ def test_general_epilogue_on_the_mfma_kernel(oracle):
         dict(bias_mode=_abi.BIAS_FULL, nonline="IDENTITY", scale_bias=1.3e-3, scale_dst=0.0271),
         dict(nonline="H_SWISH", has_z=True, scale_bias=2e-4, scale_z=0.05, scale_dst=1e-20),
         dict(nonline="RELU", scale_bias=2e-4, scale_dst=3e15),
+        # a QuantizedS32 residual on a QuantizedS32 dst (z has the dtype of dst, dnn/src/common/conv_bias.cpp:127-132)
+        dict(dst_dtype=_abi.DT_QS32, has_z=True, scale_bias=2e-4, scale_z=3e-4, scale_dst=2e-4),
+        dict(dst_dtype=_abi.DT_QS32, has_z=True, nonline="RELU", scale_bias=2e-4, scale_z=1e-4, scale_dst=2e-4),
     ]
     shapes = [("NCHW32", 2, 64, 9, 11, 96, 3, 1, 1, 1), ("NCHW32", 3, 128, 7, 7, 64, 1, 0, 1, 1), ("NCHW32", 2, 128, 8, 8, 128, 3, 1, 2, 2),
               ("NCHW32_NCHW4", 2, 64, 8, 8, 24, 3, 1, 1, 1)]
@@ -343,13 +352,11 @@ def test_general_epilogue_on_the_mfma_kernel(oracle):
             d = _abi.make_conv_desc(fmt, n, ic, ih, iw, oc, f, pad=pad, stride=stride, group=group, **kw)
             a, _ = ops.conv_bias_query(d)
             assert a.id == IGEMM and names[a.tile_cfg].startswith("v2_"), (ci, si, names[a.tile_cfg])
-            big = dict(bias_range=(-(1 << 26), 1 << 26)) if kw.get("dst_dtype") == _abi.DT_QS32 else {}
+            big = dict(bias_range=(-(1 << 26), 1 << 26), z_range=(-(1 << 24), 1 << 24)) if kw.get("dst_dtype") == _abi.DT_QS32 else {}
             check_case(oracle, d, seed=900 + 10 * ci + si, tag="general %d/%d heuristic" % (ci, si), **big)
             for tile in v2[::3]:
                 check_case(oracle, d, seed=900 + 10 * ci + si, algo=IGEMM, tile=tile, tag="general %d/%d %s" % (ci, si, names[tile]), **big)
-    # QuantizedS32 dst with a residual, and 4-packed inputs, stay on the generic kernel
-    d = _abi.make_conv_desc("NCHW32", 1, 64, 6, 6, 64, 3, pad=1, has_z=True, dst_dtype=_abi.DT_QS32, scale_bias=2e-4, scale_dst=2e-4)
-    assert ops.conv_bias_query(d)[0].id == DIRECT
+    # 4-packed inputs with a QuantizedS32 dst stay on the generic kernel
     d = _abi.make_conv_desc("NCHW4", 1, 64, 6, 6, 64, 3, pad=1, dst_dtype=_abi.DT_QS32, scale_bias=2e-4, scale_dst=2e-4)
     assert ops.conv_bias_query(d)[0].id == DIRECT
 
@@ -396,6 +403,101 @@ def test_preprocessed_filter_equals_plain_filter(oracle):
     # an algorithm without a pre-processed form
     a, _ = ops.conv_bias_query(d, DIRECT)
     assert ops.conv_bias_preprocess(d, to_dev(flt), a) is None
+
+
+NCHW_MFMA_CASES = [
+    # the generic kernel's NCHW shapes (DIRECT_CASES) scaled up until the relayout + MFMA algorithm is the heuristic's
+    # choice; channel counts that are no multiple of 32 (zero-padded blocks on either side), ragged images
+    dict(n=4, ic=24, ih=28, iw=28, oc=40, fh=3, pad=1),
+    dict(n=16, ic=3, ih=57, iw=49, oc=5, fh=3, pad=1),                     # DIRECT_CASES[0] at 8x the image and the batch
+    dict(n=3, ic=64, ih=14, iw=14, oc=128, fh=1),                           # whole blocks, 196 pixels (no vector path)
+    dict(n=2, ic=32, ih=32, iw=32, oc=64, fh=3, pad=1, stride=2),           # every relayout on its vector path
+    dict(n=2, ic=20, ih=19, iw=23, oc=36, fh=5, fw=3, pad=(2, 1), stride=(2, 1)),
+    dict(n=2, ic=64, ih=16, iw=16, oc=128, fh=3, pad=1, group=2),           # groups of whole 32-channel blocks
+    dict(n=1, ic=100, ih=30, iw=30, oc=7, fh=3),
+]
+
+
+@pytest.mark.parametrize("i", range(len(NCHW_MFMA_CASES)))
+def test_plain_nchw_on_the_mfma_kernel(oracle, i):
+    """Format::NCHW through relayout -> NCHW32 MFMA kernel -> relayout in the caller's workspace, against the checker's
+    NCHW path, every activation, with and without a residual; the generic kernel must give the same tensor."""
+    c = NCHW_MFMA_CASES[i]
+    nchw = lib.algo_names().index("MI355_NCHW_RELAYOUT_MFMA_I8")
+    for nl, has_z in (("RELU", True), ("IDENTITY", False), ("H_SWISH", True)):
+        d = mk(dict(c, fmt="NCHW"), nonline=nl, has_z=has_z, **S)
+        a, ws = ops.conv_bias_query(d)
+        assert a.id == nchw and ws > 0, (i, a.id, ws)
+        want = check_case(oracle, d, seed=1200 + i, algo=nchw, tag="nchw-mfma %d" % i)
+        check_case(oracle, d, seed=1200 + i, algo=DIRECT, tag="nchw-direct %d" % i)
+        assert want is not None
+
+
+def test_plain_nchw_workspace_contract(oracle):
+    """check_exec's workspace rule (dnn/src/common/conv_bias.cpp:32-37): exec with less than query reported is
+    MI355_ERR_WORKSPACE and launches nothing; a caller without a workspace gets the generic kernel from the heuristic;
+    exactly the reported size is enough, and a larger, offset workspace works as well."""
+    nchw = lib.algo_names().index("MI355_NCHW_RELAYOUT_MFMA_I8")
+    d = _abi.make_conv_desc("NCHW", 4, 24, 28, 28, 40, 3, pad=1, nonline="RELU", has_z=True, **S)
+    src, flt, bias, z = util.make_tensors(d, seed=77)
+    want = oracle.conv_bias(d, src, flt, bias, z)
+    dev = [to_dev(x) for x in (src, flt, bias, z)]
+    a, ws = ops.conv_bias_query(d)
+    assert a.id == nchw
+    L = lib.lib()
+    dst = torch.full(want.shape, 99, dtype=torch.int8, device="cuda")
+    short = torch.empty(ws - 256, dtype=torch.uint8, device="cuda")
+    rc = L.mi355_convbias_s8_exec(ops._stream(), d, a, *[ops._ptr(t) for t in dev], ops._ptr(dst), ops._ptr(short), short.numel())
+    assert rc == _abi.ERR_WORKSPACE, L.mi355_last_error()
+    rc = L.mi355_convbias_s8_exec(ops._stream(), d, a, *[ops._ptr(t) for t in dev], ops._ptr(dst), None, 0)
+    assert rc == _abi.ERR_WORKSPACE
+    torch.cuda.synchronize()
+    assert int((dst != 99).sum()) == 0          # nothing was launched
+    # no algorithm given and no workspace: the heuristic inside exec stays within what the caller brought
+    rc = L.mi355_convbias_s8_exec(ops._stream(), d, None, *[ops._ptr(t) for t in dev], ops._ptr(dst), None, 0)
+    assert rc == 0, L.mi355_last_error()
+    torch.cuda.synchronize()
+    assert np.array_equal(dst.cpu().numpy(), want)
+    exact = torch.empty(ws, dtype=torch.uint8, device="cuda")
+    got = ops.conv_bias_exec(d, *dev, algo=a, workspace=exact)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+    big = torch.empty(ws + 4096, dtype=torch.uint8, device="cuda")
+    got = ops.conv_bias_exec(d, *dev, algo=a, workspace=big[1024:])
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+    # tensors that are not 16-byte aligned: the relayouts take any pointer
+    flat = torch.zeros(src.size + 64, dtype=torch.int8, device="cuda")
+    flat[4:4 + src.size] = dev[0].reshape(-1)
+    got = ops.conv_bias_exec(d, flat[4:4 + src.size].view(*src.shape), dev[1], dev[2], dev[3], algo=a)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+NCHW4_GROUP_CASES = [
+    dict(n=1, ic=60, ih=9, iw=9, oc=20, fh=3, group=5, pad=1),      # shape family of dnn/test/naive/convolution.cpp:141-220
+    dict(n=20, ic=60, ih=30, iw=30, oc=20, fh=3, group=5),          # ... at the reference's own size {20,15,30,30,4} x {5,4,3,3,3,4}
+    dict(n=2, ic=32, ih=14, iw=14, oc=64, fh=3, group=4, pad=1, stride=2),
+    dict(n=3, ic=48, ih=10, iw=12, oc=24, fh=1, group=2),
+    dict(n=2, ic=256, ih=8, iw=8, oc=256, fh=3, group=8, pad=1),
+]
+
+
+@pytest.mark.parametrize("i", range(len(NCHW4_GROUP_CASES)))
+def test_nchw4_group_convolution_one_dense_launch_per_group(oracle, i):
+    c = NCHW4_GROUP_CASES[i]
+    for nl, has_z in (("RELU", True), ("IDENTITY", False), ("H_SWISH", True)):
+        d = mk(dict(c, fmt="NCHW4"), nonline=nl, has_z=has_z, **S)
+        assert ops.conv_bias_query(d)[0].id == IGEMM
+        check_case(oracle, d, seed=1300 + i, tag="nchw4 group %d heuristic" % i)
+        names = lib.tile_names()
+        for tile in range(0, len(names), 5):
+            check_case(oracle, d, seed=1300 + i, algo=IGEMM, tile=tile, tag="nchw4 group %d %s" % (i, names[tile]))
+    # batch-strided views of a group convolution: the per-group views keep the strides of the whole tensors
+    ss, fs, bs, ds = _abi.conv_shapes(mk(dict(c, fmt="NCHW4")))
+    kw = dict(src_stride_n=int(np.prod(ss[1:])) + 32, dst_stride_n=int(np.prod(ds[1:])) + 16, z_stride_n=int(np.prod(ds[1:])) + 48)
+    d = mk(dict(c, fmt="NCHW4"), nonline="RELU", has_z=True, **S, **kw)
+    check_case(oracle, d, seed=1350 + i, tag="nchw4 group %d strided batch" % i)
 
 
 def test_forced_tile_that_cannot_run_is_an_error(oracle):
