@@ -184,6 +184,23 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
                            const int8_t* src, const int8_t* filter, const int32_t* bias,
                            const int8_t* z, void* dst, void* workspace, size_t workspace_bytes);
 
+/* exec for callers that cannot allocate a workspace -- code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  No counterpart in the reference (its operators always take the caller's Workspace).  Same
+ * arguments, algorithms and results as mi355_convbias_s8_exec, minus the workspace: the algorithms that need one (plain
+ * NCHW through relayout + MFMA) use an array of MI355_STATIC_WORKSPACE_BYTES that is part of the library's own device
+ * image, one per GPU, held from the first use of the library on that GPU until the process ends.  The call allocates
+ * nothing (no hipMalloc / hipFree, no allocating library routine); the first call on a device looks the array's address
+ * up once (not under stream capture: make one call per device before capturing).  An algorithm that needs more than the
+ * array holds is MI355_ERR_WORKSPACE; without an algorithm the heuristic only considers what fits.  All calls on one
+ * GPU share the one array: calls that overlap in time on the same GPU (different streams, different threads) race --
+ * serialise them, or give all but one a workspace of their own through mi355_convbias_s8_exec.  Nothing in the array
+ * needs to survive between calls, and nothing in it is assumed to be zero. */
+#define MI355_STATIC_WORKSPACE_BYTES (32u << 20)
+size_t mi355_static_workspace_bytes(void);
+int mi355_convbias_s8_exec_static_workspace(void* stream, const mi355_conv_desc* d, const mi355_algo* algo,
+                                            const int8_t* src, const int8_t* filter, const int32_t* bias,
+                                            const int8_t* z, void* dst);
+
 /* Weight pre-processing: ConvBiasForward::deduce_preprocessed_filter_layout / get_preprocess_workspace_in_bytes /
  * exec_preprocess and the PreprocessedFilter argument of exec (dnn/include/megdnn/oprs/nn.h:381-385,400-447; CUDA
  * precedent dnn/src/cuda/conv_bias/implicit_gemm_int8_nchw32_imma.cpp:164-198: the filter re-ordered once for the

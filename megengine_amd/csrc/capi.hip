@@ -579,6 +579,58 @@ int mi355_convbias_s8_exec(void* stream, const mi355_conv_desc* d, const mi355_a
     return exec_impl(stream, d, algo, src, filter, false, bias, z, dst, workspace, workspace_bytes);
 }
 
+// ---- exec for callers that cannot allocate: the workspace is an array of the library's own --------------------------
+// One array per GPU, alive from the moment the code object is loaded on that GPU until the process ends.  In host code
+// the array's name is a stand-in, not a device address: its address on the CURRENT device comes from
+// hipGetSymbolAddress, once per device, and only that pointer is ever handed to a kernel.
+constexpr size_t kStaticWorkspaceBytes = (size_t)MI355_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticWorkspaceBytes];
+
+namespace {
+void* g_scratch_ptr[64];  // per device, under g_dev_mu
+int static_workspace(void** out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        (void)hipGetLastError();
+        return fail(MI355_ERR_NO_DEVICE, "no current device");
+    }
+    std::lock_guard<std::mutex> lk(g_dev_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return fail(MI355_ERR_LAUNCH, "address of the static workspace on device %d: %s", dev, hipGetErrorString(e));
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return MI355_OK;
+}
+}  // namespace
+
+size_t mi355_static_workspace_bytes(void) { return kStaticWorkspaceBytes; }
+
+int mi355_convbias_s8_exec_static_workspace(void* stream, const mi355_conv_desc* d, const mi355_algo* algo, const int8_t* src,
+                                            const int8_t* filter, const int32_t* bias, const int8_t* z, void* dst) {
+    // sizes first: a problem beyond the array is refused before anything touches the device
+    ConvProblem p;
+    int st = canonize(d, &p);
+    if (st) return st;
+    if (algo && algo->id != MI355_ALGO_HEURISTIC) {
+        if (algo->id < 0 || algo->id >= ALGO_COUNT) return fail(MI355_ERR_ALGO, "unknown algorithm id %d", algo->id);
+        const size_t need = algo_usable(p, algo->id) ? algo_workspace(p, algo->id) : 0;
+        if (need > kStaticWorkspaceBytes)
+            return fail(MI355_ERR_WORKSPACE, "%s needs a workspace of %zu bytes, the static workspace holds %zu", kAlgoNames[algo->id],
+                        need, kStaticWorkspaceBytes);
+    }
+    void* ws = nullptr;
+    st = static_workspace(&ws);
+    if (st) return st;
+    // no algorithm given: the heuristic stays within the array (exec_impl passes the size on as its workspace limit)
+    return exec_impl(stream, d, algo, src, filter, false, bias, z, dst, ws, kStaticWorkspaceBytes);
+}
+
 // ---- weight pre-processing ----
 static int preprocess_problem(const mi355_conv_desc* d, const mi355_algo* algo, ConvProblem* p, size_t* bytes) {
     int st = canonize(d, p);

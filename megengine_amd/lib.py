@@ -20,6 +20,7 @@ EXPORTS = [
     "mi355_igemm_tile_count", "mi355_igemm_tile_name", "mi355_igemm_tile_usable", "mi355_epilogue_linear_form",
     "mi355_relayout_deduce", "mi355_relayout_exec", "mi355_requant_s32_s8_exec", "mi355_requant_s8_s8_exec", "mi355_convbias_s8_profile",
     "mi355_pooling_deduce_out", "mi355_pooling_s8_exec", "mi355_typecvt_f32_s8_exec", "mi355_typecvt_s8_f32_exec",
+    "mi355_static_workspace_bytes", "mi355_convbias_s8_exec_static_workspace",
     "mi355_epilogue_quotient_form", "mi355_convbias_s8_preprocess_size", "mi355_convbias_s8_preprocess", "mi355_convbias_s8_exec_preprocessed",
 ]
 
@@ -59,6 +60,9 @@ def lib():
     L.mi355_convbias_s8_query.argtypes = [P(_abi.ConvDesc), C.c_int, P(_abi.Algo), P(C.c_size_t)]
     L.mi355_convbias_s8_exec.argtypes = [C.c_void_p, P(_abi.ConvDesc), P(_abi.Algo), C.c_void_p, C.c_void_p,
                                          C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    L.mi355_static_workspace_bytes.restype = C.c_size_t
+    L.mi355_convbias_s8_exec_static_workspace.argtypes = [C.c_void_p, P(_abi.ConvDesc), P(_abi.Algo), C.c_void_p, C.c_void_p,
+                                                          C.c_void_p, C.c_void_p, C.c_void_p]
     L.mi355_convbias_s8_preprocess_size.argtypes = [P(_abi.ConvDesc), P(_abi.Algo), P(C.c_size_t)]
     L.mi355_convbias_s8_preprocess.argtypes = [C.c_void_p, P(_abi.ConvDesc), P(_abi.Algo), C.c_void_p, C.c_void_p, C.c_size_t]
     L.mi355_convbias_s8_exec_preprocessed.argtypes = [C.c_void_p, P(_abi.ConvDesc), P(_abi.Algo), C.c_void_p, C.c_void_p,
