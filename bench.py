@@ -282,12 +282,34 @@ class EventTimer:
         return ms.value
 
 
-def time_launches(torch, fn, iters=20, warm=3):
+def time_launches(torch, fn, iters=20, warm=3, graph=True):
+    """Seconds per call of fn (one or more launches on the current stream), `iters` calls back to back.  With `graph`
+    the calls are captured once into a HIP graph and the graph is replayed: eager launches through Python cost ~6 us
+    of host time each, which would be the figure reported for every kernel shorter than that (the depthwise layers at
+    14x14 and 7x7 run 3.6-5.5 us).  Falls back to eager launches if the capture fails."""
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
     st = torch.cuda.current_stream()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    if graph:
+        try:
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=st):
+                for _ in range(iters):
+                    fn()
+            g.replay()
+            torch.cuda.synchronize()
+            reps = 3
+            e0.record(st)
+            for _ in range(reps):
+                g.replay()
+            e1.record(st)
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / (iters * reps) * 1e-3
+        except Exception as e:  # capture is an optimisation of the launch path only
+            log("graph capture of a side measurement failed (%r): eager launches" % (e,))
+            torch.cuda.synchronize()
     e0.record(st)
     for _ in range(iters):
         fn()
@@ -354,8 +376,9 @@ def time_launches_cold(torch, fn, iters=8):
 
 def run_extras(torch, np, _abi, lib, ops, workloads, side_iters=50):
     """Side measurements for the other workload configurations (not the headline value).  Every row carries two
-    times: "us" = the launch repeated back to back on the same tensors (operands warm in L2 / the last-level cache
-    when they fit), "us_cold" = median of launches that each follow a flush of both caches."""
+    times: "us" = the launch repeated back to back on the same tensors as replays of a captured HIP graph (operands warm
+    in L2 / the last-level cache when they fit; the dependent-launch gap of ~1.8 us is part of it, the host's launch
+    cost is not), "us_cold" = median of eager launches that each follow a flush of both caches."""
     res = {}
 
     def measure(layers, seed):

@@ -161,6 +161,13 @@ __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel)
     return __builtin_amdgcn_perm(hi, lo, sel);
 }
 
+// c + dot(a, b) over four signed bytes, written to a fresh register
+__device__ __forceinline__ int dot4_from(uint32_t a, int b, int c) {
+    int r;
+    asm("v_dot4_i32_i8 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // pixels (dwords of 4 channels) p[0..3]  ->  t[c] = {p0.c, p1.c, p2.c, p3.c}
 __device__ __forceinline__ void transpose4(const uint32_t p[4], uint32_t t[4]) {
     const uint32_t a = perm(p[1], p[0], 0x05010400u), b = perm(p[1], p[0], 0x07030602u);
@@ -220,8 +227,21 @@ __device__ __forceinline__ void dw3_store(const Dw3Args& a, const int (&acc)[R][
     }
 }
 
-template <int S, int R>
+// EPI: the requantisation form compiled into the kernel -- 0: the one-FMA linear form, 1: RELU without a residual (multi-step
+// fast form), 2: any other, chosen at run time.  BUF: input rows through bounds-checked buffer loads (tensors below
+// 2 GiB, padding at most 1); otherwise pointer loads.  The two common forms of the MobileNet family get kernels that
+// hold nothing else: a launch of a few microseconds should not have to fetch eight epilogues' worth of code.
+template <int S, int R, int EPI, bool BUF>
 __global__ __launch_bounds__(256) void dw3x3_kernel(Dw3Args a) {
+    // Every kernel argument is requested in one batch of scalar loads: left alone the compiler fetches them where they
+    // are first used, behind the early exit and the item decoding -- three dependent round trips to the argument
+    // segment before the first vector load of a kernel whose whole life is a few microseconds.
+    asm volatile("" ::"s"(a.src), "s"(a.flt), "s"(a.bias), "s"(a.z), "s"(a.dst), "s"(a.CG), "s"(a.IH), "s"(a.IW), "s"(a.OH),
+                 "s"(a.OW), "s"(a.QW), "s"(a.OHS), "s"(a.ph), "s"(a.pw), "s"(a.items), "s"(a.src_bytes), "s"(a.src_sn),
+                 "s"(a.dst_sn), "s"(a.z_sn), "s"(a.has_bias));
+    asm volatile("" ::"s"(a.div_qw.m), "s"(a.div_qw.s1), "s"(a.div_qw.s2), "s"(a.div_ohs.m), "s"(a.div_ohs.s1),
+                 "s"(a.div_ohs.s2), "s"(a.div_cg.m), "s"(a.div_cg.s1), "s"(a.div_cg.s2), "s"(a.epi.fast), "s"(a.epi.lin),
+                 "s"(a.epi.has_z), "s"(a.epi.nonline), "s"(a.epi.lin_c), "s"(a.epi.lin_d), "s"(a.epi.lin_lo));
     const uint32_t item = blockIdx.x * 256u + threadIdx.x;
     if (item >= a.items) return;
     // item = ((n * CG + cg) * OHS + strip) * QW + quad
@@ -230,23 +250,19 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(Dw3Args a) {
     const uint32_t n = fdiv(i2, a.div_cg), cg = i2 - n * a.CG;
     const int oh0 = (int)strip * R, ow0 = (int)q * 4;
 
-    // filter rows per channel: wlo = {w(fh,0), w(fh,1), w(fh,2), 0}, whi = the same one byte up
-    uint32_t wlo[3][4], whi[3][4];
+    // The filter and the bias of this thread's channel quad are requested here and used only after the input rows
+    // have been requested too (below): one round trip to memory for everything the thread reads, not two.
+    uint32_t wraw[9];
     {
         const uint32_t* wp = reinterpret_cast<const uint32_t*>(a.flt) + cg * 9;
 #pragma unroll
-        for (int fh = 0; fh < 3; ++fh) {
-            const uint32_t w0 = wp[fh * 3], w1 = wp[fh * 3 + 1], w2 = wp[fh * 3 + 2];
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const uint32_t t = perm(w1, w0, 0x0c0c0000u | ((4u + c) << 8) | (uint32_t)c);
-                wlo[fh][c] = perm(w2, t, 0x0c000100u | ((4u + c) << 16));
-                whi[fh][c] = wlo[fh][c] << 8;
-            }
-        }
+        for (int i = 0; i < 9; ++i) wraw[i] = wp[i];
     }
-    v4i bias4 = {0, 0, 0, 0};
-    if (a.has_bias) bias4 = *reinterpret_cast<const v4i*>(a.bias + cg * 4);
+    // (a bounds-checked load: without a bias the buffer has no bytes and every lane reads zeros -- no branch whose join
+    // would make the compiler wait for the load on the spot)
+    const __amdgpu_buffer_rsrc_t rs_bias =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t*>(a.bias), 0, a.has_bias ? a.CG * 16 : 0, 0x00020000);
+    const v4i bias4 = __builtin_amdgcn_raw_buffer_load_b128(rs_bias, (int)cg * 16, 0, 0);
     int acc[R][4][4];
 
     const uint32_t* sp = reinterpret_cast<const uint32_t*>(a.src + n * a.src_sn) + (int64_t)cg * a.IH * a.IW;
@@ -255,7 +271,7 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(Dw3Args a) {
     // window columns: L = c0, block T = c0+1 .. c0+4, then (S = 1) Rt = c0+5 or (S = 2) block U = c0+5 .. c0+8
     uint32_t L[ROWS], Rt[ROWS], pt[ROWS][4], pu[ROWS][4];
     const bool interior = c0 + 1 >= 0 && c0 + (S == 1 ? 4 : 8) < a.IW;
-    if (a.src_bytes && a.pw <= 1) {
+    if (BUF) {
         // Bounds-checked buffer loads with 32-bit offsets, the same straight-line code for every thread.  A row outside
         // the image, or a side column outside the row, becomes the out-of-range offset and reads zeros: nothing to
         // clamp.  The 4-pixel blocks always start inside the row (pw <= 1); where one runs past the end of the row
@@ -340,6 +356,19 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(Dw3Args a) {
         }
     }
 
+    // filter rows per channel: wlo = {w(fh,0), w(fh,1), w(fh,2), 0}, whi = the same one byte up
+    uint32_t wlo[3][4], whi[3][4];
+#pragma unroll
+    for (int fh = 0; fh < 3; ++fh) {
+        const uint32_t w0 = wraw[fh * 3], w1 = wraw[fh * 3 + 1], w2 = wraw[fh * 3 + 2];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t t = perm(w1, w0, 0x0c0c0000u | ((4u + c) << 8) | (uint32_t)c);
+            wlo[fh][c] = perm(w2, t, 0x0c000100u | ((4u + c) << 16));
+            whi[fh][c] = wlo[fh][c] << 8;
+        }
+    }
+
 #pragma unroll
     for (int ir = 0; ir < ROWS; ++ir) {
         uint32_t T[4], U[4] = {0u, 0u, 0u, 0u};
@@ -364,18 +393,28 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(Dw3Args a) {
                 const int fh = ir - r * S;
                 if (fh < 0 || fh > 2) continue;
                 const int lo = (int)wlo[fh][c], hi = (int)whi[fh][c];
-                // the first filter row of an output row starts from the bias
-                const int p0 = fh ? acc[r][0][c] : bias4[c], p1 = fh ? acc[r][1][c] : bias4[c];
-                const int p2 = fh ? acc[r][2][c] : bias4[c], p3 = fh ? acc[r][3][c] : bias4[c];
-                acc[r][0][c] = __builtin_amdgcn_sdot4((int)e0, lo, p0, false);
-                acc[r][1][c] = __builtin_amdgcn_sdot4((int)e1, S == 1 ? lo : hi, p1, false);
-                acc[r][2][c] = __builtin_amdgcn_sdot4((int)e2, S == 1 ? hi : lo, p2, false);
-                acc[r][3][c] = __builtin_amdgcn_sdot4((int)e3, hi, p3, false);
+                if (fh == 0) {
+                    // the first filter row of an output row starts from the bias: the three-operand form of the dot
+                    // product reads it in place (the compiler's accumulate-in-place form costs a copy per accumulator)
+                    acc[r][0][c] = dot4_from(e0, lo, bias4[c]);
+                    acc[r][1][c] = dot4_from(e1, S == 1 ? lo : hi, bias4[c]);
+                    acc[r][2][c] = dot4_from(e2, S == 1 ? hi : lo, bias4[c]);
+                    acc[r][3][c] = dot4_from(e3, hi, bias4[c]);
+                    continue;
+                }
+                acc[r][0][c] = __builtin_amdgcn_sdot4((int)e0, lo, acc[r][0][c], false);
+                acc[r][1][c] = __builtin_amdgcn_sdot4((int)e1, S == 1 ? lo : hi, acc[r][1][c], false);
+                acc[r][2][c] = __builtin_amdgcn_sdot4((int)e2, S == 1 ? hi : lo, acc[r][2][c], false);
+                acc[r][3][c] = __builtin_amdgcn_sdot4((int)e3, hi, acc[r][3][c], false);
             }
         }
     }
 
-    if (!a.epi.fast) {
+    if (EPI == 0) {
+        dw3_store<R, NL_LIN, false, true>(a, acc, n, cg, oh0, ow0);
+    } else if (EPI == 1) {
+        dw3_store<R, NL_RELU, false, true>(a, acc, n, cg, oh0, ow0);
+    } else if (!a.epi.fast) {
         dw3_store<R, 0, false, false>(a, acc, n, cg, oh0, ow0);
     } else if (a.epi.lin) {
         dw3_store<R, NL_LIN, false, true>(a, acc, n, cg, oh0, ow0);
@@ -391,6 +430,20 @@ __global__ __launch_bounds__(256) void dw3x3_kernel(Dw3Args a) {
             case NL_H_SWISH: dw3_store<R, NL_H_SWISH, false, true>(a, acc, n, cg, oh0, ow0); break;
             default: dw3_store<R, NL_IDENTITY, false, true>(a, acc, n, cg, oh0, ow0); break;
         }
+    }
+}
+
+template <int S, int R>
+void launch_dw3(hipStream_t st, dim3 grid, const Dw3Args& b) {
+    const bool buf = b.src_bytes != 0 && b.pw <= 1;
+    const int epi = !b.epi.fast ? 2 : b.epi.lin ? 0 : (!b.epi.has_z && b.epi.nonline == NL_RELU) ? 1 : 2;
+    const dim3 block(256);
+    if (buf) {
+        if (epi == 0) hipLaunchKernelGGL((dw3x3_kernel<S, R, 0, true>), grid, block, 0, st, b);
+        else if (epi == 1) hipLaunchKernelGGL((dw3x3_kernel<S, R, 1, true>), grid, block, 0, st, b);
+        else hipLaunchKernelGGL((dw3x3_kernel<S, R, 2, true>), grid, block, 0, st, b);
+    } else {
+        hipLaunchKernelGGL((dw3x3_kernel<S, R, 2, false>), grid, block, 0, st, b);
     }
 }
 
@@ -433,15 +486,15 @@ int launch_conv_depthwise(hipStream_t st, const ConvProblem& p, const int8_t* sr
             const int64_t src_total = (int64_t)(d.n - 1) * p.src_sn + (int64_t)d.ic * d.ih * d.iw;
             b.src_bytes = src_total < ((int64_t)1 << 31) ? (uint32_t)src_total : 0u;
             b.div_qw = make_fastdiv(b.QW); b.div_ohs = make_fastdiv(b.OHS); b.div_cg = make_fastdiv(b.CG);
-            dim3 grid((unsigned)((items + 255) / 256)), block(256);
+            const dim3 grid((unsigned)((items + 255) / 256));
             if (d.stride_h == 1 && R == 4)
-                hipLaunchKernelGGL((dw3x3_kernel<1, 4>), grid, block, 0, st, b);
+                launch_dw3<1, 4>(st, grid, b);
             else if (d.stride_h == 1)
-                hipLaunchKernelGGL((dw3x3_kernel<1, 2>), grid, block, 0, st, b);
+                launch_dw3<1, 2>(st, grid, b);
             else if (R == 2)
-                hipLaunchKernelGGL((dw3x3_kernel<2, 2>), grid, block, 0, st, b);
+                launch_dw3<2, 2>(st, grid, b);
             else
-                hipLaunchKernelGGL((dw3x3_kernel<2, 1>), grid, block, 0, st, b);
+                launch_dw3<2, 1>(st, grid, b);
             return (int)hipGetLastError();
         }
     }

@@ -35,9 +35,17 @@
 namespace mi355 {
 namespace {
 
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, bool PW>
+// KS > 1: the waves of a workgroup also split the reduction.  KS groups of WM x WN waves each multiply the whole output
+// tile over their own chunks of every stage (CPS = KCH / KS chunk steps per stage instead of KCH: a serial chain KS
+// times shorter, and with wave tiles of 64 x 64 four MFMAs per four fragment reads), the int32 partial sums meet in LDS
+// -- in the ring, which is idle by then -- and every wave requantises and stores its share of the blocks.  Integer
+// addition is exact in any order, nothing leaves the workgroup, the workspace stays 0.  Such a workgroup runs ONE tile
+// (the launch gives every tile its own): these are the tiles for long reductions over few tiles.
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, bool PW, int KS = 1>
 struct Igemm2 {
-    static constexpr int NW = WM * WN;  // waves per workgroup
+    static constexpr int WMN = WM * WN;      // waves of one reduction group
+    static constexpr int NW = WMN * KS;      // waves per workgroup
+    static constexpr int CPS = KCH / KS;     // chunk steps per stage of one wave
     static constexpr int THREADS = NW * 64;
     static constexpr int WTM = BM / WM, WTN = BN / WN;
     static constexpr int MT = WTM / 32, NT = WTN / 32;
@@ -53,13 +61,18 @@ struct Igemm2 {
     // The 8-wave tiles of 256 x 128 outputs and more read the residual in the epilogue, straight from global memory:
     // an LDS slot for it (BM * BN bytes) would cost them a workgroup per CU, and a tile of theirs runs long enough to
     // hide the fetch of one block behind the requantisation of the previous one.
-    static constexpr bool ZD = BM * BN >= 256 * 128;
+    static constexpr bool ZD = BM * BN >= 256 * 128 || KS > 1;  // (the split tiles keep their LDS for the ring)
+    // partial sums of the blocks a wave does not finish itself: (KS - 1) / KS of its MT x NT blocks of 4 KiB
+    static constexpr int OB = MT * NT / KS;  // blocks a wave finishes
+    static constexpr int RED_BYTES = KS > 1 ? NW * OB * (KS - 1) * 4096 : 0;
+    static_assert(KCH % KS == 0 && CPS % 2 == 0, "chunk steps per wave and stage: even (fragment double buffer)");
+    static_assert(KS == 1 || ((MT * NT) % KS == 0 && RED_BYTES <= NS * STG), "partial sums fit the idle ring");
     static_assert(NW == 4 || NW == 8, "4 or 8 waves");
     static_assert(MT >= 1 && NT >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "wave tile");
     static_assert((KCH * NBA) % NW == 0 && (KCH * NBB) % NW == 0, "copies divide over the waves");
     static_assert(NBA >= NW ? NBA % NW == 0 : NW % NBA == 0, "filter blocks vs waves");
     static_assert(NBB >= NW ? NBB % NW == 0 : NW % NBB == 0, "pixel blocks vs waves");
-    static_assert(KCH % 2 == 0, "fragment double buffer: the first chunk of a stage uses register set 0");
+
     static_assert(NS >= 3 && (NS - 1) * U < 64, "ring depth (one buffer read, one refilled, the rest in flight) vs the 6-bit vmcnt");
 
     // copy j of wave w is block j * NW + w of the stage in [chunk][row block] order
@@ -192,7 +205,7 @@ struct Igemm2 {
     // Copy j of wave w is block j * NW + w of the stage, at LDS address wave_addr + j * NW KiB.
     template <int N>
     __device__ static constexpr int step_of(int j) {  // chunk step in which copy j of N is issued
-        return N >= KCH ? j / (N / KCH) : j * (KCH / N);
+        return N >= CPS ? j / (N / CPS) : j * (CPS / N);
     }
     template <int N>
     __device__ static constexpr int nth_in_step(int j) {  // position of copy j among the copies of its step
@@ -206,9 +219,9 @@ struct Igemm2 {
         for (int j = 0; j < N; ++j) n += step_of<N>(j) == c ? 1 : 0;
         return n;
     }
-    static_assert(UA >= KCH ? UA % KCH == 0 : KCH % UA == 0, "filter copies vs chunk steps");
-    static_assert(UB >= KCH ? UB % KCH == 0 : KCH % UB == 0, "activation copies vs chunk steps");
-    static constexpr int CS_LAST = copies_in_step<UA>(KCH - 1) + copies_in_step<UB>(KCH - 1);
+    static_assert(UA >= CPS ? UA % CPS == 0 : CPS % UA == 0, "filter copies vs chunk steps");
+    static_assert(UB >= CPS ? UB % CPS == 0 : CPS % UB == 0, "activation copies vs chunk steps");
+    static constexpr int CS_LAST = copies_in_step<UA>(CPS - 1) + copies_in_step<UB>(CPS - 1);
 
     // KT: the reduction is not a whole number of stages, chunks past its end read zeros (the activations' zeros meet
     // whatever the filter copy returns there).
@@ -221,7 +234,7 @@ struct Igemm2 {
     template <bool KT>
     __device__ static __forceinline__ void issue_all(const IgemmArgs& a, const Loader& L, const KEntry (&nk)[UB], const v4i& rs_src,
                                                      const v4i& rs_flt, uint32_t wave_addr, int w) {
-        issue_all_steps<KT>(a, L, nk, rs_src, rs_flt, wave_addr, w, std::make_integer_sequence<int, KCH>{});
+        issue_all_steps<KT>(a, L, nk, rs_src, rs_flt, wave_addr, w, std::make_integer_sequence<int, CPS>{});
     }
     template <bool KT, int... C>
     __device__ static __forceinline__ void issue_all_steps(const IgemmArgs& a, const Loader& L, const KEntry (&nk)[UB],
@@ -270,7 +283,15 @@ struct Igemm2 {
         }
     }
 
-    __device__ static __forceinline__ void init_acc_lds(v16i (&acc)[MT][NT], const int* sBias, int wm, int lh) {
+    // kg: the wave's reduction group; the bias enters the sum once, through group 0
+    __device__ static __forceinline__ void init_acc_lds(v16i (&acc)[MT][NT], const int* sBias, int wm, int lh, int kg = 0) {
+        if (KS > 1 && kg != 0) {  // wave-uniform
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NT; ++j) acc[i][j] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             v16i init;
@@ -373,7 +394,8 @@ struct Igemm2 {
         const int t = threadIdx.x;
         const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
         const int l32 = lane & 31, lh = lane >> 5;
-        const int wm = wave / WN, wn = wave % WN;
+        const int kg = KS > 1 ? wave / WMN : 0, wmn = KS > 1 ? wave - kg * WMN : wave;  // reduction group, wave inside it
+        const int wm = wmn / WN, wn = wmn % WN;
 
         // this workgroup's tile sequence: workgroup b runs on XCD b % 8 (round-robin dispatch), and each XCD works on
         // one contiguous slab of the tile space, so that its L2 sees disjoint pixels and one set of filter rows
@@ -402,6 +424,7 @@ struct Igemm2 {
         // bytes: every lane writes 0.
         const v4i rs_bias = uniform_rsrc(a.bias, a.has_bias ? (uint32_t)a.OC * 4u : 0u);
         if (wave * 64 < BM) lds_copy64x4(lds0 + (uint32_t)(NS * STG + wave * 256), (cur.oc0 + t) * 4, rs_bias);
+        const v4i rs_flt = uniform_rsrc(a.flt, a.flt_bytes);
 
         if (!PW) {
             const int cap = (nst + 1) * KCH;  // one stage of padding entries, read when the loader stands at the end of a tile
@@ -421,7 +444,6 @@ struct Igemm2 {
         }
 
         const v4i rs_src = uniform_rsrc(a.src, a.src_bytes);
-        const v4i rs_flt = uniform_rsrc(a.flt, a.flt_bytes);
         const v4i rs_z = uniform_rsrc(a.z, a.epi.has_z ? a.z_bytes : 0u);
         const int dA = KCH * a.flt_kstride, dB = KCH * a.src_scb;  // k-offset steps of one stage
 
@@ -472,8 +494,9 @@ struct Igemm2 {
         __syncthreads();             // ... and everyone's
 
         const int fragpos = ((l32 >> 4) * 2 + lh) * 256 + (l32 & 15) * 16;
-        const int8_t* fragA = lds + fragpos + wm * MT * 1024;
-        const int8_t* fragB = lds + fragpos + A_BYTES + wn * NT * 1024;
+        // (a reduction group reads its own CPS chunks of every stage)
+        const int8_t* fragA = lds + fragpos + wm * MT * 1024 + kg * (CPS * NBA * 1024);
+        const int8_t* fragB = lds + fragpos + A_BYTES + wn * NT * 1024 + kg * (CPS * NBB * 1024);
         int rd_off = 0;               // byte offset of the stage being multiplied
         int wr_off = (NS - 1) * STG;  // ... of the buffer refilled during this stage: the one read before it
 
@@ -497,7 +520,7 @@ struct Igemm2 {
         auto chunk_step = [&](auto steady, auto cc) __attribute__((always_inline)) {
             constexpr bool STEADY = decltype(steady)::value;
             constexpr int c = decltype(cc)::value;
-            constexpr bool LAST = c + 1 == KCH;
+            constexpr bool LAST = c + 1 == CPS;
             if (LAST) {
                 wait_lgkmcnt0();
                 // copies younger than the next stage's: NS - 3 whole stages and the chunk steps of this stage so far
@@ -557,11 +580,11 @@ struct Igemm2 {
         };
         auto stage = [&](auto steady) __attribute__((always_inline)) {
             for_each_chunk([&](auto cc) __attribute__((always_inline)) { chunk_step(steady, cc); },
-                           std::make_integer_sequence<int, KCH>{});
+                           std::make_integer_sequence<int, CPS>{});
         };
 
         frags(0, fa[0], fb[0]);
-        init_acc_lds(acc, sBias, wm, lh);
+        init_acc_lds(acc, sBias, wm, lh, kg);
 
         // stages whose refill stays inside the tile: the loader runs NS - 1 stages ahead
         const int steady = nst > NS - 1 ? nst - (NS - 1) : 0;
@@ -589,6 +612,42 @@ struct Igemm2 {
             }
             for (int s = steady; s < nst; ++s) stage(std::false_type{});
             if (DUAL) acc[0][0] += alt;
+            if constexpr (KS > 1) {
+                // The partial sums of the KS reduction groups meet in the ring: every copy has landed (the loader's trailing
+                // copies are out-of-range zero fills, but they do write), everyone is done reading.  Block b of a wave tile
+                // is finished by group b % KS: a wave parks its sums of the other blocks, lane-linear 16-byte stores, and
+                // collects the other groups' sums of its own.
+                wait_vmcnt<0>();
+                __syncthreads();
+                int8_t* red = lds + lane * 16;
+                auto slot = [&](int owner, int ob, int src) __attribute__((always_inline)) {
+                    return ((((owner * WMN + wmn) * OB + ob) * (KS - 1)) + (src < owner ? src : src - 1)) * 4096;
+                };
+#pragma unroll
+                for (int b = 0; b < MT * NT; ++b) {
+                    if (b % KS == kg) continue;  // wave-uniform
+                    int8_t* p = red + slot(b % KS, b / KS, kg);
+                    const v16i& c = acc[b / NT][b % NT];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        *reinterpret_cast<v4i*>(p + q * 1024) = v4i{c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
+                }
+                __syncthreads();
+#pragma unroll
+                for (int b = 0; b < MT * NT; ++b) {
+                    if (b % KS != kg) continue;
+                    v16i& c = acc[b / NT][b % NT];
+                    for (int src = 0; src < KS; ++src) {
+                        if (src == kg) continue;
+                        const int8_t* p = red + slot(kg, b / KS, src);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const v4i v = *reinterpret_cast<const v4i*>(p + q * 1024);
+                            c[4 * q] += v[0]; c[4 * q + 1] += v[1]; c[4 * q + 2] += v[2]; c[4 * q + 3] += v[3];
+                        }
+                    }
+                }
+            }
             ZRegs<MT, NT> zr;
             if (zslots) {
                 // A residual slot is complete once a stage boundary has waited with at least (NS - 2) U - CS_LAST younger
@@ -601,6 +660,8 @@ struct Igemm2 {
             }
             if constexpr (GEN)
                 igemm_epilogue_general<POUT, MT, NT>(a, acc, cur.oc0 + wm * WTM, cur.pix0 + wn * WTN, l32, lh, cur.oc_end);
+            else if constexpr (KS > 1)  // the blocks this wave finishes
+                igemm_run_epilogue<POUT, MT, NT, false>(a, acc, cur.oc0 + wm * WTM, cur.pix0 + wn * WTN, l32, lh, nullptr, cur.oc_end, KS, kg);
             else if constexpr (ZD)
                 igemm_run_epilogue<POUT, MT, NT, false>(a, acc, cur.oc0 + wm * WTM, cur.pix0 + wn * WTN, l32, lh, nullptr, cur.oc_end);
             else
@@ -614,7 +675,7 @@ struct Igemm2 {
                     if (t < BM) sBias[t] = fetch_bias(a, nxt.oc0, t);
                     __syncthreads();
                 }
-                init_acc_lds(acc, sBias, wm, lh);
+                init_acc_lds(acc, sBias, wm, lh, kg);
             }
             cur = nxt;
         }
@@ -623,9 +684,9 @@ struct Igemm2 {
     }
 };
 
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, bool KT, bool GEN>
-__global__ __launch_bounds__(WM * WN * 64, MINW) void igemm2_kernel(IgemmArgs a) {
-    Igemm2<POUT, BM, BN, WM, WN, KCH, NS, PW>::template run<KT, GEN>(a);
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, bool KT, bool GEN, int KS = 1>
+__global__ __launch_bounds__(WM * WN * KS * 64, MINW) void igemm2_kernel(IgemmArgs a) {
+    Igemm2<POUT, BM, BN, WM, WN, KCH, NS, PW, KS>::template run<KT, GEN>(a);
 }
 
 constexpr int kLdsPerCu = 160 * 1024;
@@ -651,12 +712,16 @@ const Cfg2 kCfg2[] = {
         {"v2_256x256x64r3w8", 256, 256, 2},
         {"v2_128x128x64r4w8", 128, 128, 2},
         {"v2_64x128x64r5", 64, 128, 2},
+        {"v2_128x64x128r3k2", 128, 64, 4},
+        {"v2_128x64x256r3k4w8", 128, 64, 8},
+        {"v2_64x128x128r3k2", 64, 128, 4},
+        {"v2_128x128x128r3k2w8", 128, 128, 4},
 };
 constexpr int kNumCfg2 = sizeof(kCfg2) / sizeof(kCfg2[0]);
 
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, bool KT, bool GEN>
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool PW, bool KT, bool GEN, int KS = 1>
 int launch_k(hipStream_t st, IgemmArgs& a, int cu_count) {
-    using K = Igemm2<POUT, BM, BN, WM, WN, KCH, NS, PW>;
+    using K = Igemm2<POUT, BM, BN, WM, WN, KCH, NS, PW, KS>;
     a.tiles_m_pg = (a.ocpg + BM - 1) / BM;
     a.tiles_m = a.tiles_m_pg * a.groups;
     a.div_tiles_m = make_fastdiv((uint32_t)a.tiles_m);
@@ -680,7 +745,7 @@ int launch_k(hipStream_t st, IgemmArgs& a, int cu_count) {
     const int lds = fixed + a.zslots * K::ZSLOT;
     if (lds > kLdsPerCu) return kNoFit;  // ring + residual slot of this tile do not fit
     if (a.dry_run) return 0;             // the question was only whether this tile can run the problem
-    auto kern = igemm2_kernel<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW, KT, GEN>;
+    auto kern = igemm2_kernel<POUT, BM, BN, WM, WN, KCH, NS, MINW, PW, KT, GEN, KS>;
     // per-instantiation caches; atomics, because operators on different streams may launch from several threads
     static std::atomic<int> max_lds_set{0};
     if (lds > max_lds_set.load(std::memory_order_relaxed)) {
@@ -703,22 +768,33 @@ int launch_k(hipStream_t st, IgemmArgs& a, int cu_count) {
     }
     if (cu_count <= 0) cu_count = 256;
     int64_t grid = (int64_t)occ * cu_count;
+    if (KS > 1) grid = tiles;  // a workgroup that splits the reduction runs one tile (its ring doubles as the meeting place)
+    // a multiple of 8 (one contiguous slab of the tile space per XCD).  When every tile has a workgroup of its own the
+    // count is rounded UP -- a few workgroups find no tile and leave -- because rounding down would hand some workgroups
+    // a second tile and double the launch's duration; otherwise down, inside what the device holds at once.
     if (grid > tiles) grid = tiles;
-    if (grid >= 8) grid &= ~(int64_t)7;
+    if (grid >= 8) grid = grid == tiles ? (grid + 7) & ~(int64_t)7 : grid & ~(int64_t)7;
     a.div_step = make_fastdiv((uint32_t)((grid & 7) == 0 ? grid >> 3 : grid));  // the kernel's tile stride
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(K::THREADS), lds, st, a);
     return (int)hipGetLastError();
 }
 
-template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool GEN>
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, bool GEN, int KS = 1>
 int launch_gen(hipStream_t st, IgemmArgs& a, int cu) {
     const bool pw = a.T == 1 && a.ph == 0 && a.pw == 0;
     const bool kt = a.KC % KCH != 0;
     if (pw)
-        return kt ? launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, true, true, GEN>(st, a, cu)
-                  : launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, true, false, GEN>(st, a, cu);
+        return kt ? launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, true, true, GEN, KS>(st, a, cu)
+                  : launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, true, false, GEN, KS>(st, a, cu);
     // the k-unit table carries the end of the reduction (padding entries)
-    return launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, false, false, GEN>(st, a, cu);
+    return launch_k<POUT, BM, BN, WM, WN, KCH, NS, MINW, false, false, GEN, KS>(st, a, cu);
+}
+
+// a tile whose waves also split the reduction (fast epilogue only)
+template <int POUT, int BM, int BN, int WM, int WN, int KCH, int NS, int MINW, int KS>
+int launch_split(hipStream_t st, IgemmArgs& a, int cu) {
+    if (a.general) return kNoGen;
+    return launch_gen<POUT, BM, BN, WM, WN, KCH, NS, MINW, false, KS>(st, a, cu);
 }
 
 // GENOK: the tile is also instantiated with the general epilogue (two tiles are: every general problem runs on one of them)
@@ -750,6 +826,11 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
         case 11: return launch_one<POUT, 256, 256, 4, 2, 2, 3, 2>(st, a, cu);
         case 12: return launch_one<POUT, 128, 128, 2, 4, 2, 4, 4>(st, a, cu);
         case 13: return launch_one<POUT, 64, 128, 2, 2, 2, 5, 2>(st, a, cu);
+        // reduction split over the waves of the workgroup: wave tiles of 64 x 64
+        case 14: return launch_split<POUT, 128, 64, 2, 1, 4, 3, 2, 2>(st, a, cu);
+        case 15: return launch_split<POUT, 128, 64, 2, 1, 8, 3, 2, 4>(st, a, cu);
+        case 16: return launch_split<POUT, 64, 128, 1, 2, 4, 3, 2, 2>(st, a, cu);
+        case 17: return launch_split<POUT, 128, 128, 2, 2, 4, 3, 2, 2>(st, a, cu);
         default: return (int)hipErrorInvalidValue;
     }
 }

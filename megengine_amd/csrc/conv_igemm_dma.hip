@@ -482,8 +482,11 @@ int launch_pw(hipStream_t st, IgemmArgs& a, int cu_count) {
     }
     if (cu_count <= 0) cu_count = 256;
     int64_t grid = (int64_t)occ * cu_count;
+    // a multiple of 8 (one contiguous slab of the tile space per XCD).  When every tile has a workgroup of its own the
+    // count is rounded UP -- a few workgroups find no tile and leave -- because rounding down would hand some workgroups
+    // a second tile and double the launch's duration; otherwise down, inside what the device holds at once.
     if (grid > tiles) grid = tiles;
-    if (grid >= 8) grid &= ~(int64_t)7;
+    if (grid >= 8) grid = grid == tiles ? (grid + 7) & ~(int64_t)7 : grid & ~(int64_t)7;
     a.div_step = make_fastdiv((uint32_t)((grid & 7) == 0 ? grid >> 3 : grid));  // the kernel's tile stride
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(K::THREADS), lds, st, a);
     return (int)hipGetLastError();

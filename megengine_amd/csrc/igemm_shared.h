@@ -115,9 +115,11 @@ __device__ __forceinline__ void igemm_load_z(const IgemmArgs& a, ZRegs<MT, NT>& 
 }
 
 // ZPRE: the residual was fetched by igemm_load_z into *zr; otherwise it is loaded here, block by block
+// blk_mod > 1: only the blocks b = i * NT + j with b % blk_mod == blk_rem are written (a wave of a workgroup that
+// splits the reduction finishes its share of the blocks; wave-uniform)
 template <int POUT, int MT, int NT, int NL, bool HZ, bool ZPRE>
 __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], const ZRegs<MT, NT>* zr, int oc_w,
-                                               int pix_w, int l32, int lh, int oc_end) {
+                                               int pix_w, int l32, int lh, int oc_end, int blk_mod = 1, int blk_rem = 0) {
     const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(a.z, HZ ? a.z_bytes : 0);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
@@ -131,6 +133,7 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
         for (int i = 0; i < MT; ++i) {
             const int ocb = oc_w + i * 32;  // first channel of this 32-channel block
             if (ocb >= oc_end) continue;    // wave-uniform
+            if (blk_mod > 1 && (i * NT + j) % blk_mod != blk_rem) continue;
             const v16i& c = acc[i][j];
             if (POUT == 32) {
                 const int blk_off = (ocb >> 5) * a.dst_scb + lh * 16;
@@ -177,21 +180,22 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
 // group); negative = the layer's channel count.
 template <int POUT, int MT, int NT, bool ZPRE = false>
 __device__ __forceinline__ void igemm_run_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w, int l32,
-                                                   int lh, const ZRegs<MT, NT>* zr = nullptr, int oc_end = -1) {
+                                                   int lh, const ZRegs<MT, NT>* zr = nullptr, int oc_end = -1, int blk_mod = 1,
+                                                   int blk_rem = 0) {
     if (oc_end < 0) oc_end = a.OC;
     if (a.epi.lin) {
-        igemm_epilogue<POUT, MT, NT, NL_LIN, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end);
+        igemm_epilogue<POUT, MT, NT, NL_LIN, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem);
     } else if (a.epi.has_z) {
         switch (a.epi.nonline) {
-            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
-            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
-            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
+            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
+            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
+            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
         }
     } else {
         switch (a.epi.nonline) {
-            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
-            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
-            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end); break;
+            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
+            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
+            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
         }
     }
 }
