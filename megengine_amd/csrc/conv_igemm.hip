@@ -479,14 +479,16 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
 
 }  // namespace
 
-// tile_cfg numbering: register-staged tiles, LDS-direct tiles, second-generation tiles
-int igemm_num_cfgs() { return kNumCfgs + igemm_dma_num_cfgs() + igemm2_num_cfgs(); }
+// tile_cfg numbering: register-staged tiles, LDS-direct tiles, second-generation tiles, patch-staged tiles
+int igemm_num_cfgs() { return kNumCfgs + igemm_dma_num_cfgs() + igemm2_num_cfgs() + igemm3_num_cfgs(); }
+int igemm_first_v2_cfg() { return kNumCfgs + igemm_dma_num_cfgs(); }
+static int igemm_first_v3_cfg() { return igemm_first_v2_cfg() + igemm2_num_cfgs(); }
 const char* igemm_cfg_name(int cfg) {
     if (cfg >= 0 && cfg < kNumCfgs) return kCfgs[cfg].name;
-    if (cfg < kNumCfgs + igemm_dma_num_cfgs()) return igemm_dma_cfg_name(cfg - kNumCfgs);
-    return igemm2_cfg_name(cfg - kNumCfgs - igemm_dma_num_cfgs());
+    if (cfg < igemm_first_v2_cfg()) return igemm_dma_cfg_name(cfg - kNumCfgs);
+    if (cfg < igemm_first_v3_cfg()) return igemm2_cfg_name(cfg - igemm_first_v2_cfg());
+    return igemm3_cfg_name(cfg - igemm_first_v3_cfg());
 }
-int igemm_first_v2_cfg() { return kNumCfgs + igemm_dma_num_cfgs(); }
 
 static bool igemm_needs_general(const ConvProblem& p) {
     return p.d.dst_dtype != MI355_DT_QS8 || p.d.bias_mode == MI355_BIAS_FULL || !p.epi.fast;
@@ -681,6 +683,7 @@ static void igemm_fill_args(const ConvProblem& p, IgemmArgs& a) {
     a.epi = p.epi;
     a.flt_rstride = a.kbytes;
     a.flt_kstride = 32;
+    a.NB = d.n;
     a.groups = d.group;
     a.ocpg = p.ocpg;
     a.src_sg = (p.icpg / p.pin) * a.src_scb;
@@ -707,6 +710,12 @@ int igemm_resolve_cfg(const ConvProblem& p, int cfg) {
     const int first_v2 = igemm_first_v2_cfg();
     // group convolutions and the general epilogue exist on the second-generation tiles only
     if ((d.group != 1 || a.general) && cfg < first_v2) cfg = first_v2 + (p.ocpg <= 64 ? 3 : 0);
+    if (cfg >= igemm_first_v3_cfg()) {
+        // the patch-staged tiles: stride 1, a filter window, 32-packed, the fast epilogue; otherwise the second-generation
+        // tile of 128 x 128 (resolved below like any other request for it)
+        if (igemm3_can_run(a, p.pin, p.pout, cfg - igemm_first_v3_cfg())) return cfg;
+        cfg = first_v2;
+    }
     if (cfg >= first_v2) {
         if (p.pin == 32) {
             int v = cfg - first_v2;
@@ -771,6 +780,7 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
         a.flt_bytes = (uint32_t)igemm_preprocessed_bytes(p, cfg);
     }
     const int first_v2 = igemm_first_v2_cfg();
+    if (cfg >= igemm_first_v3_cfg()) return launch_igemm3(st, a, p.pin, p.pout, cfg - igemm_first_v3_cfg());
     if (cfg >= first_v2) return launch_igemm2(st, a, p.pout, cfg - first_v2, cu_count);
     if (cfg >= kNumCfgs) return launch_igemm_dma(st, a, p.pout, cfg - kNumCfgs, cu_count);
     if (p.pin == 32 && p.pout == 32) return launch_fmt<32, 32>(st, a, cfg, cu_count);

@@ -48,6 +48,10 @@ struct IgemmArgs {
     // reciprocal on the critical path from kernel entry to the first copy): by the number of channel tiles, by the
     // channel tiles of a group, and by the tile stride of a workgroup (set by the launch code, which knows the grid)
     FastDiv div_tiles_m, div_tiles_m_pg, div_step;
+    // patch-staged kernel (conv_igemm3.hip): batch size, padded row width and rows per padded image, patch pixels
+    // (a multiple of 64), patch copies per wave, channel blocks of the reduction
+    int NB, p_w, p_himg, pxp, pcw, cbs;
+    FastDiv div_pw, div_phimg;
     int dry_run;  // host only: the launch code stops before anything is launched and reports whether the tile fits
 };
 
@@ -272,6 +276,13 @@ int igemm_first_v2_cfg();  // tile_cfg of the first second-generation tile
 // pre-processed filter of the second-generation kernel: [k-chunk][channel padded to 32][32 bytes]
 size_t igemm2_preprocessed_bytes(int oc, int kbytes);
 int launch_igemm2_preprocess(hipStream_t st, const int8_t* flt, int8_t* out, int oc, int kbytes);
+
+// patch-staged kernel for 32-packed inputs, filters larger than 1x1 at stride 1 (conv_igemm3.hip): same filter layouts
+// (reference or pre-processed) as the second-generation kernel
+int igemm3_num_cfgs();
+const char* igemm3_cfg_name(int cfg);
+bool igemm3_can_run(const IgemmArgs& a, int pin, int pout, int cfg);
+int launch_igemm3(hipStream_t st, IgemmArgs& a, int pin, int pout, int cfg);
 
 // streaming kernel for 4-packed pointwise layers with few input or few output channels (conv_pw4.hip)
 bool pw4s_usable(const IgemmArgs& a);

@@ -380,9 +380,9 @@ def test_preprocessed_filter_equals_plain_filter(oracle):
                 a.tile_cfg = tile
                 pre = ops.conv_bias_preprocess(d, dev[1], a)
                 if pre is None:
-                    assert not (names[tile].startswith("v2_") and fmt in ("NCHW32", "NCHW32_NCHW4"))
+                    assert not (names[tile].startswith(("v2_", "v3_")) and fmt in ("NCHW32", "NCHW32_NCHW4"))
                     continue
-                assert names[tile].startswith("v2_")
+                assert names[tile].startswith(("v2_", "v3_"))  # the patch-staged tiles read the same filter form
                 say("case preprocessed", fmt, n, ic, ih, iw, oc, f, pad, stride, nl, z, names[tile])
                 plain = ops.conv_bias_exec(d, dev[0], dev[1], dev[2], dev[3], algo=a)
                 got = ops.conv_bias_exec_preprocessed(d, dev[0], pre, dev[2], dev[3], algo=a)
@@ -560,6 +560,44 @@ def test_every_tile_on_ragged_shapes(oracle, i):
     from megengine_amd import lib
     for tile in range(len(lib.tile_names())):
         check_case(oracle, d, seed=400 + i, algo=IGEMM, tile=tile, tag="ragged%d/%s" % (i, lib.tile_names()[tile]))
+
+
+# ---------------------------------------------------------------------------------------------
+# patch-staged tiles (32-packed, stride 1, filters larger than 1x1): the activations of a tile staged once per channel
+# block as a patch of padded input rows
+# ---------------------------------------------------------------------------------------------
+
+PATCH_CASES = [
+    # n, ic, ih, iw, oc, fh, fw, pad
+    (2, 64, 14, 14, 64, 3, 3, 1),          # a tile spans both images (196 pixels each)
+    (3, 32, 7, 7, 96, 3, 3, 1),            # one channel block: nothing to prefetch
+    (2, 96, 9, 11, 160, 3, 3, 1),          # odd width, three channel blocks, ragged channel tile
+    (1, 64, 20, 17, 64, 5, 5, 2),          # 5x5
+    (2, 32, 12, 12, 32, 3, 3, 0),          # no padding
+    (5, 64, 7, 7, 256, 3, 3, 1),           # five small images per tile
+    (2, 64, 16, 16, 128, 3, 5, (1, 2)),    # non-square filter
+    (1, 128, 30, 30, 96, 3, 3, (2, 1)),    # padding wider than the filter radius: output larger than input
+    (2, 64, 56, 56, 64, 3, 3, 1),          # rows longer than a wave's pixels
+    (4, 256, 14, 14, 256, 3, 3, 1),        # eight channel blocks: the patch slots recycle
+    (9, 32, 5, 5, 64, 3, 3, 1),            # tiny images, ragged last tile
+    (1, 32, 40, 33, 288, 5, 5, 2),         # 5x5, three channel tiles
+]
+
+
+@pytest.mark.parametrize("i", range(len(PATCH_CASES)))
+def test_patch_staged_tiles(oracle, i):
+    n, ic, ih, iw, oc, fh, fw, pad = PATCH_CASES[i]
+    names = lib.tile_names()
+    ran = 0
+    for nl, z in (("RELU", True), ("IDENTITY", False), ("H_SWISH", True)):
+        # a destination scale that keeps most outputs inside the int8 range
+        d = _abi.make_conv_desc("NCHW32", n, ic, ih, iw, oc, fh, fw, pad=pad, nonline=nl, has_z=z, scale_bias=2e-4,
+                                scale_z=0.05, scale_dst=0.05 * (ic * fh * fw / 64) ** 0.5)
+        for tile, name in enumerate(names):
+            if name.startswith("v3_") and check_case(oracle, d, seed=50 + i, algo=IGEMM, tile=tile,
+                                                      tag="patch%d/%s" % (i, name)) is not None:
+                ran += 1
+    assert ran >= 3, "no patch-staged tile took case %d" % i
 
 
 # ---------------------------------------------------------------------------------------------

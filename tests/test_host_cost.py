@@ -47,7 +47,7 @@ def test_steady_state_query_and_canonize_stay_cheap_over_many_scales():
     # every call walks the validation and both proof caches.  Best of a few repeats per call: the bound is on the
     # work, not on what else the host was doing.
     worst_q = worst_c = 0
-    for rep in range(2):
+    for rep in range(4):
         for d in descs:
             ref = C.byref(d)
             tq = _best_ns(lambda: L.mi355_convbias_s8_query(ref, _abi.ALGO_HEURISTIC_PREPROCESS, C.byref(algo), C.byref(ws)), 1)
