@@ -28,6 +28,8 @@
  *                                 (dnn/src/naive/type_cvt/opr_impl.cpp:24-56)
  *   mi355_requant_s8_s8_exec   <- ElemwiseMultiType binary quantized modes on two QuantizedS8 tensors
  *                                 (dnn/src/naive/elemwise_multi_type/opr_impl.h:88-116, opr_impl_4.cpp:11-60)
+ *   mi355_elemwise_q_exec      <- ElemwiseMultiType::on_quantized_mode, one to three inputs, every libm-free mode
+ *                                 (opr_impl_3.cpp:11-60, opr_impl_4.cpp:11-66, opr_impl_5.cpp:11-45)
  *   mi355_relayout_exec        <- RelayoutFormat::exec (dnn/include/megdnn/oprs/general.h:1353-1359),
  *                                 arithmetic of naive::RelayoutFormatImpl::exec
  *                                 (dnn/src/naive/relayout_format/opr_impl.cpp:486-773)
@@ -308,6 +310,40 @@ int mi355_requant_s32_s8_exec(void* stream, const mi355_requant_desc* d, const i
  * rescaling TypeCvt QuantizedS8 -> QuantizedS8.  The residual add of a network whose fuser left it outside ConvBias.
  * All three tensors need 16-byte alignment. */
 int mi355_requant_s8_s8_exec(void* stream, const mi355_requant_desc* d, const int8_t* src, const int8_t* z, int8_t* dst);
+
+/* ---- ElemwiseMultiType quantized modes in general: dst = quantize(mode(dequantize(a) [, dequantize(b) [, dequantize(c)]])) ----
+ * ElemwiseMultiType::on_quantized_mode for one, two and three inputs (dnn/src/naive/elemwise_multi_type/opr_impl_3.cpp:
+ * 11-60, opr_impl_4.cpp:11-66, opr_impl_5.cpp:11-45; the per-element drivers opr_impl.h:45-66, :88-116, :142-175):
+ * every input is dequantized with its own scale (float(x) * scale, dnn/include/megdnn/dtype.h:854,:897), the float
+ * kernel of the mode runs on the floats (dnn/src/common/elemwise/kern_defs.cuh:166-313), the result is quantized with
+ * dst's scale (dtype.h:845-853 for QuantizedS8; :887-896 for QuantizedS32, which saturates at 2147483520).  The inputs
+ * share one dtype (opr_impl_4.cpp:14-16), QuantizedS8 or QuantizedS32; dst is QuantizedS8 or QuantizedS32.
+ * `mode` carries the reference's Elemwise::Mode enumerator values (dnn/scripts/opr_param_defs.py:341-455).  Served are
+ * the modes whose float kernel is made of individually rounded IEEE operations, so that the result is defined bit for
+ * bit; the modes that call the C math library (ACOS ASIN COS EXP EXPM1 LOG LOG1P SIGMOID SIN TANH ERF* POW LOG_SUM_EXP
+ * FUSE_ADD_SIGMOID FUSE_ADD_TANH ATAN2 MOD) return MI355_ERR_UNSUPPORTED: their bits are a property of the host's libm.
+ * The comparison modes produce 1.0f / 0.0f before the quantization, as the reference's float kernels do.
+ * Contiguous tensors of `count` elements; QuantizedS8 tensors need 4-byte, QuantizedS32 tensors 16-byte alignment. */
+enum {
+    MI355_EW_RELU = 0, MI355_EW_ABS = 1, MI355_EW_CEIL = 4, MI355_EW_FLOOR = 8, MI355_EW_NEGATE = 11,
+    MI355_EW_ABS_GRAD = 15, MI355_EW_ADD = 16, MI355_EW_FLOOR_DIV = 17, MI355_EW_MAX = 18, MI355_EW_MIN = 19,
+    MI355_EW_MUL = 21, MI355_EW_SIGMOID_GRAD = 23, MI355_EW_SUB = 24, MI355_EW_SWITCH_GT0 = 25, MI355_EW_TANH_GRAD = 26,
+    MI355_EW_TRUE_DIV = 27, MI355_EW_LT = 29, MI355_EW_LEQ = 30, MI355_EW_EQ = 31, MI355_EW_COND_LEQ_MOV = 34,
+    MI355_EW_FUSE_MUL_ADD3 = 35, MI355_EW_FUSE_ADD_RELU = 37, MI355_EW_FAST_TANH = 40, MI355_EW_FAST_TANH_GRAD = 41,
+    MI355_EW_ROUND = 42, MI355_EW_H_SWISH = 49, MI355_EW_H_SWISH_GRAD = 50, MI355_EW_FUSE_ADD_H_SWISH = 51,
+    MI355_EW_COND_LT_MOV = 60
+};
+typedef struct mi355_elemwise_desc {
+    uint32_t mode;        /* MI355_EW_* */
+    uint32_t arity;       /* 1, 2 or 3: must be the mode's */
+    uint32_t src_dtype;   /* MI355_DT_QS8 or MI355_DT_QS32, shared by the inputs */
+    uint32_t dst_dtype;   /* MI355_DT_QS8 or MI355_DT_QS32 */
+    float scale_src[3];
+    float scale_dst;
+    uint64_t count;       /* elements */
+} mi355_elemwise_desc;
+int mi355_elemwise_q_exec(void* stream, const mi355_elemwise_desc* d, const void* src0, const void* src1, const void* src2,
+                          void* dst);
 
 /* TypeCvt between Float32 and QuantizedS8, the quantize / dequantize at the two ends of an int8 network
  * (dnn/src/naive/type_cvt/opr_impl.cpp:24-56): Float32 -> QuantizedS8 is DTypeParamImpl<dt_qint8>::quantize =

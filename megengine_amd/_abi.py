@@ -82,6 +82,35 @@ class RequantDesc(C.Structure):
     ]
 
 
+# param::Elemwise::Mode values of the quantized modes that mi355_elemwise_q_exec serves (dnn/scripts/opr_param_defs.py:341-455)
+EW_MODES = {
+    "RELU": 0, "ABS": 1, "CEIL": 4, "FLOOR": 8, "NEGATE": 11, "ABS_GRAD": 15, "ADD": 16, "FLOOR_DIV": 17, "MAX": 18,
+    "MIN": 19, "MUL": 21, "SIGMOID_GRAD": 23, "SUB": 24, "SWITCH_GT0": 25, "TANH_GRAD": 26, "TRUE_DIV": 27, "LT": 29,
+    "LEQ": 30, "EQ": 31, "COND_LEQ_MOV": 34, "FUSE_MUL_ADD3": 35, "FUSE_ADD_RELU": 37, "FAST_TANH": 40,
+    "FAST_TANH_GRAD": 41, "ROUND": 42, "H_SWISH": 49, "H_SWISH_GRAD": 50, "FUSE_ADD_H_SWISH": 51, "COND_LT_MOV": 60,
+}
+EW_ARITY = {m: 1 for m in ("RELU", "ABS", "CEIL", "FLOOR", "NEGATE", "ROUND", "FAST_TANH", "H_SWISH")}
+EW_ARITY.update({m: 3 for m in ("COND_LEQ_MOV", "COND_LT_MOV", "FUSE_MUL_ADD3")})
+EW_ARITY.update({m: 2 for m in EW_MODES if m not in EW_ARITY})
+
+
+class ElemwiseDesc(C.Structure):
+    _fields_ = [
+        ("mode", C.c_uint32), ("arity", C.c_uint32), ("src_dtype", C.c_uint32), ("dst_dtype", C.c_uint32),
+        ("scale_src", C.c_float * 3), ("scale_dst", C.c_float), ("count", C.c_uint64),
+    ]
+
+
+def make_elemwise_desc(mode, scales_src, scale_dst, count, src_dtype=None, dst_dtype=None):
+    """mode by name; scales_src holds one scale per input of the mode"""
+    d = ElemwiseDesc(mode=EW_MODES[mode], arity=EW_ARITY[mode], src_dtype=DT_QS8 if src_dtype is None else src_dtype,
+                     dst_dtype=DT_QS8 if dst_dtype is None else dst_dtype, scale_dst=scale_dst, count=count)
+    assert len(scales_src) == EW_ARITY[mode]
+    for i, s in enumerate(scales_src):
+        d.scale_src[i] = s
+    return d
+
+
 # param::Pooling::Mode
 POOL_MAX, POOL_AVERAGE, POOL_AVERAGE_COUNT_EXCLUDE_PADDING = 0, 1, 2
 POOL_NAMES = {"MAX": POOL_MAX, "AVERAGE": POOL_AVERAGE, "AVERAGE_COUNT_EXCLUDE_PADDING": POOL_AVERAGE_COUNT_EXCLUDE_PADDING}

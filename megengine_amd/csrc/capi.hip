@@ -755,6 +755,30 @@ int mi355_requant_s8_s8_exec(void* stream, const mi355_requant_desc* d, const in
     return MI355_OK;
 }
 
+int mi355_elemwise_q_exec(void* stream, const mi355_elemwise_desc* d, const void* src0, const void* src1, const void* src2,
+                          void* dst) {
+    if (!d) return fail(MI355_ERR_BAD_ARG, "null descriptor");
+    const int arity = elemwise_q_arity(d->mode);
+    if (arity == 0)
+        return fail(MI355_ERR_UNSUPPORTED, "elemwise mode %u is not served (no such mode, or its float kernel calls the C math library)",
+                    d->mode);
+    if ((int)d->arity != arity) return fail(MI355_ERR_BAD_ARG, "elemwise mode %u takes %d inputs, descriptor says %u", d->mode, arity, d->arity);
+    if ((d->src_dtype != MI355_DT_QS8 && d->src_dtype != MI355_DT_QS32) || (d->dst_dtype != MI355_DT_QS8 && d->dst_dtype != MI355_DT_QS32))
+        return fail(MI355_ERR_UNSUPPORTED, "quantized elemwise takes QuantizedS8 or QuantizedS32 tensors");
+    if (d->count == 0) return MI355_OK;
+    const void* srcs[3] = {src0, src1, src2};
+    const uintptr_t src_mask = d->src_dtype == MI355_DT_QS32 ? 15 : 3, dst_mask = d->dst_dtype == MI355_DT_QS32 ? 15 : 3;
+    for (int i = 0; i < arity; ++i) {
+        if (!srcs[i]) return fail(MI355_ERR_BAD_ARG, "input %d is null", i);
+        if (reinterpret_cast<uintptr_t>(srcs[i]) & src_mask) return fail(MI355_ERR_BAD_ARG, "input %d is misaligned", i);
+    }
+    if (!dst) return fail(MI355_ERR_BAD_ARG, "null tensor pointer");
+    if (reinterpret_cast<uintptr_t>(dst) & dst_mask) return fail(MI355_ERR_BAD_ARG, "dst is misaligned");
+    int rc = launch_elemwise_q(reinterpret_cast<hipStream_t>(stream), *d, src0, src1, src2, dst, cu_count());
+    if (rc) return fail(MI355_ERR_LAUNCH, "elemwise: %s", hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
+}
+
 int mi355_typecvt_f32_s8_exec(void* stream, uint64_t count, float scale_dst, const float* src, int8_t* dst) {
     if (count == 0) return MI355_OK;
     if (!src || !dst) return fail(MI355_ERR_BAD_ARG, "null tensor pointer");

@@ -72,6 +72,9 @@ int launch_requant8(hipStream_t st, const EpiParams& e, const int8_t* src, const
                     int cu_count);
 
 // plain streaming kernel: reads read_bytes from src and writes write_bytes to dst in 16-byte accesses (a measuring stick)
+int elemwise_q_arity(uint32_t mode);
+int launch_elemwise_q(hipStream_t st, const mi355_elemwise_desc& d, const void* s0, const void* s1, const void* s2, void* dst,
+                      int cu_count);
 int launch_stream_probe(hipStream_t st, const void* src, uint64_t read_bytes, void* dst, uint64_t write_bytes, int cu_count);
 int launch_cvt_f32_s8(hipStream_t st, float scale, const float* src, int8_t* dst, uint64_t count, int cu_count);
 int launch_cvt_s8_f32(hipStream_t st, float scale, const int8_t* src, float* dst, uint64_t count, int cu_count);

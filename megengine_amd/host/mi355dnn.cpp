@@ -617,18 +617,66 @@ static void requant_exec(Handle* h, uint32_t nonline, const TensorND& a, const T
 
 void ElemwiseMultiType::exec(const std::vector<TensorND>& src, const TensorND& dst) {
     using Mode = Param::Mode;
-    uint32_t nl = MI355_NL_IDENTITY;
-    size_t arity = 2;
+    // Q-mode -> the Elemwise::Mode whose float kernel it runs and its number of operands (the ON_QUANTIZED_MODE table,
+    // dnn/src/common/elemwise_multi_type/opr_impl_helper.cpp:6-11,:53-111)
+    struct Row { Mode q; uint32_t ew, arity; };
+    static const Row kRows[] = {
+            {Mode::QADD, MI355_EW_ADD, 2}, {Mode::QFUSE_ADD_RELU, MI355_EW_FUSE_ADD_RELU, 2}, {Mode::QMUL, MI355_EW_MUL, 2},
+            {Mode::QMIN, MI355_EW_MIN, 2}, {Mode::QMAX, MI355_EW_MAX, 2}, {Mode::QSUB, MI355_EW_SUB, 2},
+            {Mode::QTRUE_DIV, MI355_EW_TRUE_DIV, 2}, {Mode::QRELU, MI355_EW_RELU, 1}, {Mode::QABS, MI355_EW_ABS, 1},
+            {Mode::QFUSE_MUL_ADD3, MI355_EW_FUSE_MUL_ADD3, 3}, {Mode::QFAST_TANH, MI355_EW_FAST_TANH, 1},
+            {Mode::QNEGATE, MI355_EW_NEGATE, 1}, {Mode::QCEIL, MI355_EW_CEIL, 1}, {Mode::QFLOOR, MI355_EW_FLOOR, 1},
+            {Mode::QROUND, MI355_EW_ROUND, 1}, {Mode::QABS_GRAD, MI355_EW_ABS_GRAD, 2}, {Mode::QFLOOR_DIV, MI355_EW_FLOOR_DIV, 2},
+            {Mode::QSIGMOID_GRAD, MI355_EW_SIGMOID_GRAD, 2}, {Mode::QSWITCH_GT0, MI355_EW_SWITCH_GT0, 2},
+            {Mode::QTANH_GRAD, MI355_EW_TANH_GRAD, 2}, {Mode::QLT, MI355_EW_LT, 2}, {Mode::QLEQ, MI355_EW_LEQ, 2},
+            {Mode::QEQ, MI355_EW_EQ, 2}, {Mode::QFAST_TANH_GRAD, MI355_EW_FAST_TANH_GRAD, 2},
+            {Mode::QCOND_LEQ_MOV, MI355_EW_COND_LEQ_MOV, 3}, {Mode::QH_SWISH, MI355_EW_H_SWISH, 1},
+            {Mode::QFUSE_ADD_H_SWISH, MI355_EW_FUSE_ADD_H_SWISH, 2}, {Mode::QH_SWISH_GRAD, MI355_EW_H_SWISH_GRAD, 2},
+            {Mode::QCOND_LT_MOV, MI355_EW_COND_LT_MOV, 3},
+    };
+    const Row* row = nullptr;
+    for (const Row& r : kRows)
+        if (r.q == m_param.mode) row = &r;
+    if (!row) fail(MI355_ERR_UNSUPPORTED, "ElemwiseMultiType mode " + std::to_string((unsigned)m_param.mode) + " is not implemented");
+    HOST_ASSERT(src.size() == row->arity, MI355_ERR_BAD_ARG, "mode takes %u operands, got %zu", row->arity, src.size());
+    // the requantisation kernels (proved divide-free forms) take the modes of the ConvBias post-process on their
+    // operand types: first operand QuantizedS8 / QuantizedS32, second QuantizedS8, dst QuantizedS8
+    uint32_t nl = 0;
+    bool chain = true;
     switch (m_param.mode) {
-        case Mode::QADD: break;
-        case Mode::QFUSE_ADD_RELU: nl = MI355_NL_RELU; break;
-        case Mode::QFUSE_ADD_H_SWISH: nl = MI355_NL_H_SWISH; break;
-        case Mode::QRELU: nl = MI355_NL_RELU; arity = 1; break;
-        case Mode::QH_SWISH: nl = MI355_NL_H_SWISH; arity = 1; break;
-        default: fail(MI355_ERR_UNSUPPORTED, "ElemwiseMultiType mode " + std::to_string((unsigned)m_param.mode) + " is not implemented");
+        case Mode::QADD: nl = MI355_NL_IDENTITY; break;
+        case Mode::QFUSE_ADD_RELU: case Mode::QRELU: nl = MI355_NL_RELU; break;
+        case Mode::QFUSE_ADD_H_SWISH: case Mode::QH_SWISH: nl = MI355_NL_H_SWISH; break;
+        default: chain = false;
     }
-    HOST_ASSERT(src.size() == arity, MI355_ERR_BAD_ARG, "mode takes %zu operands, got %zu", arity, src.size());
-    requant_exec(m_handle, nl, src[0], arity == 2 ? &src[1] : nullptr, dst);
+    if (chain && dst.layout.dtype.enumv == DTypeEnum::QuantizedS8 &&
+        (row->arity == 1 || src[1].layout.dtype.enumv == DTypeEnum::QuantizedS8))
+        return requant_exec(m_handle, nl, src[0], row->arity == 2 ? &src[1] : nullptr, dst);
+    auto code = [](DTypeEnum e) -> uint32_t {
+        if (e == DTypeEnum::QuantizedS8) return MI355_DT_QS8;
+        if (e == DTypeEnum::QuantizedS32) return MI355_DT_QS32;
+        fail(MI355_ERR_UNSUPPORTED, "quantized elemwise takes QuantizedS8 or QuantizedS32 tensors");
+        return 0;
+    };
+    mi355_elemwise_desc d = mi355_elemwise_desc();
+    d.mode = row->ew;
+    d.arity = row->arity;
+    d.src_dtype = code(src[0].layout.dtype.enumv);
+    d.dst_dtype = code(dst.layout.dtype.enumv);
+    d.scale_dst = dst.layout.dtype.scale;
+    d.count = dst.layout.total_nr_elems();
+    HOST_ASSERT(dst.layout.is_contiguous() && dst.raw_ptr, MI355_ERR_BAD_ARG, "dst must be contiguous and non-null");
+    const void* p[3] = {nullptr, nullptr, nullptr};
+    for (uint32_t i = 0; i < row->arity; ++i) {
+        // the operands share one dtype (dnn/src/naive/elemwise_multi_type/opr_impl_4.cpp:14-16)
+        HOST_ASSERT(src[i].layout.dtype.enumv == src[0].layout.dtype.enumv, MI355_ERR_BAD_ARG, "operand %u has another dtype", i);
+        HOST_ASSERT(src[i].layout.eq_shape(dst.layout) && src[i].layout.is_contiguous(), MI355_ERR_SHAPE,
+                    "operands must be contiguous and of the dst shape %s", dst.layout.to_string().c_str());
+        HOST_ASSERT(src[i].raw_ptr, MI355_ERR_BAD_ARG, "null tensor pointer");
+        d.scale_src[i] = src[i].layout.dtype.scale;
+        p[i] = src[i].raw_ptr;
+    }
+    check_abi(mi355_elemwise_q_exec(m_handle->stream(), &d, p[0], p[1], p[2], dst.raw_ptr));
 }
 
 void TypeCvt::exec(const TensorND& src, const TensorND& dst) {

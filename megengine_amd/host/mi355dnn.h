@@ -279,20 +279,27 @@ private:
     Param m_param;
 };
 
-// The quantized modes of megdnn::ElemwiseMultiType (dnn/include/megdnn/oprs/nn_int.h:12) that sit around ConvBias in
-// an int8 network: dst = quantize(mode(dequantize(a) [, dequantize(b)])).  First operand QuantizedS8 or QuantizedS32,
-// second (binary modes) QuantizedS8, dst QuantizedS8; contiguous tensors of one shape.
+// The quantized modes of megdnn::ElemwiseMultiType (dnn/include/megdnn/oprs/nn_int.h:12): dst = quantize(mode(
+// dequantize(a) [, dequantize(b) [, dequantize(c)]])), operands QuantizedS8 or QuantizedS32 of one dtype, dst
+// QuantizedS8 or QuantizedS32, contiguous tensors of one shape.  The modes whose float kernel calls the C math library
+// (QEXP, QSIGMOID, QTANH, QPOW ...) are MI355_ERR_UNSUPPORTED: their bits belong to the host's libm.
 class ElemwiseMultiType : public OperatorBase {
 public:
     struct Param {
-        // values of param::ElemwiseMultiType::Mode (dnn/scripts/opr_param_defs.py:479-529)
-        enum class Mode : uint32_t { QADD = 6, QFUSE_ADD_RELU = 7, QRELU = 15, QH_SWISH = 51, QFUSE_ADD_H_SWISH = 52 };
+        // values of param::ElemwiseMultiType::Mode (dnn/scripts/opr_param_defs.py:479-540)
+        enum class Mode : uint32_t {
+            QADD = 6, QFUSE_ADD_RELU = 7, QMUL = 8, QMIN = 9, QMAX = 10, QSUB = 11, QTRUE_DIV = 12, QRELU = 15, QABS = 16,
+            QFUSE_MUL_ADD3 = 20, QFAST_TANH = 21, QNEGATE = 22, QCEIL = 25, QFLOOR = 28, QROUND = 32, QABS_GRAD = 37,
+            QFLOOR_DIV = 38, QSIGMOID_GRAD = 40, QSWITCH_GT0 = 41, QTANH_GRAD = 42, QLT = 43, QLEQ = 44, QEQ = 45,
+            QFAST_TANH_GRAD = 48, QCOND_LEQ_MOV = 50, QH_SWISH = 51, QFUSE_ADD_H_SWISH = 52, QH_SWISH_GRAD = 53,
+            QCOND_LT_MOV = 57
+        };
         Mode mode = Mode::QADD;
     };
     explicit ElemwiseMultiType(Handle* h) : OperatorBase(h) {}
     Param& param() { return m_param; }
     const Param& param() const { return m_param; }
-    // src: one tensor for QRELU / QH_SWISH, two for the QADD family
+    // src: as many tensors as the mode has operands
     void exec(const std::vector<TensorND>& src, const TensorND& dst);
 
 private:

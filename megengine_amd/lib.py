@@ -18,7 +18,8 @@ EXPORTS = [
     "mi355_convbias_deduce_out", "mi355_convbias_algo_count", "mi355_convbias_algo_name",
     "mi355_convbias_algo_usable", "mi355_convbias_s8_query", "mi355_convbias_s8_exec",
     "mi355_igemm_tile_count", "mi355_igemm_tile_name", "mi355_igemm_tile_usable", "mi355_epilogue_linear_form",
-    "mi355_relayout_deduce", "mi355_relayout_exec", "mi355_requant_s32_s8_exec", "mi355_requant_s8_s8_exec", "mi355_convbias_s8_profile",
+    "mi355_relayout_deduce", "mi355_relayout_exec", "mi355_requant_s32_s8_exec", "mi355_requant_s8_s8_exec", "mi355_elemwise_q_exec",
+    "mi355_convbias_s8_profile",
     "mi355_pooling_deduce_out", "mi355_pooling_s8_exec", "mi355_typecvt_f32_s8_exec", "mi355_typecvt_s8_f32_exec",
     "mi355_static_workspace_bytes", "mi355_convbias_s8_exec_static_workspace",
     "mi355_epilogue_quotient_form", "mi355_convbias_s8_preprocess_size", "mi355_convbias_s8_preprocess", "mi355_convbias_s8_exec_preprocessed",
@@ -82,6 +83,7 @@ def lib():
     L.mi355_relayout_exec.argtypes = [C.c_void_p, P(_abi.RelayoutDesc), C.c_void_p, C.c_void_p]
     L.mi355_requant_s32_s8_exec.argtypes = [C.c_void_p, P(_abi.RequantDesc), C.c_void_p, C.c_void_p, C.c_void_p]
     L.mi355_requant_s8_s8_exec.argtypes = [C.c_void_p, P(_abi.RequantDesc), C.c_void_p, C.c_void_p, C.c_void_p]
+    L.mi355_elemwise_q_exec.argtypes = [C.c_void_p, P(_abi.ElemwiseDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
     L.mi355_pooling_deduce_out.argtypes = [P(_abi.PoolingDesc), P(C.c_uint32), P(C.c_uint32)]
     L.mi355_pooling_s8_exec.argtypes = [C.c_void_p, P(_abi.PoolingDesc), C.c_void_p, C.c_void_p]
     L.mi355_typecvt_f32_s8_exec.argtypes = [C.c_void_p, C.c_uint64, C.c_float, C.c_void_p, C.c_void_p]

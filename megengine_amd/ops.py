@@ -164,6 +164,23 @@ def requant_exec(src, scale_src, scale_dst, nonline="IDENTITY", z=None, scale_z=
     return dst
 
 
+def elemwise_q_exec(mode, srcs, scales_src, scale_dst, dst_dtype=None, dst=None):
+    """ElemwiseMultiType quantized mode `mode` (name of the Elemwise::Mode, e.g. "FUSE_MUL_ADD3") on one to three int8 or
+    int32 tensors of one shape with their scales; dst is QuantizedS8 unless dst_dtype says torch.int32."""
+    if len(srcs) != _abi.EW_ARITY[mode]:
+        raise RuntimeError("%s takes %d inputs" % (mode, _abi.EW_ARITY[mode]))
+    if any(s.dtype != srcs[0].dtype or s.shape != srcs[0].shape for s in srcs) or srcs[0].dtype not in (torch.int8, torch.int32):
+        raise RuntimeError("elemwise_q_exec takes int8 or int32 tensors of one dtype and shape")
+    ddt = torch.int8 if dst_dtype is None else dst_dtype
+    if dst is None:
+        dst = torch.empty(srcs[0].shape, dtype=ddt, device=srcs[0].device)
+    code = {torch.int8: _abi.DT_QS8, torch.int32: _abi.DT_QS32}
+    d = _abi.make_elemwise_desc(mode, scales_src, scale_dst, srcs[0].numel(), code[srcs[0].dtype], code[dst.dtype])
+    p = [_ptr(s) for s in srcs] + [None] * (3 - len(srcs))
+    check(lib().mi355_elemwise_q_exec(_stream(), C.byref(d), p[0], p[1], p[2], _ptr(dst)))
+    return dst
+
+
 def pooling_deduce_layout(d):
     """Output shape of megdnn::PoolingForward for the descriptor (dnn/src/common/pooling.cpp:7-125)."""
     oh, ow = C.c_uint32(), C.c_uint32()

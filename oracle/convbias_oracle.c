@@ -116,6 +116,80 @@ int oracle_requant_s8_s8(const mi355_requant_desc* d, const int8_t* src, const i
     return MI355_OK;
 }
 
+/* The float kernels of the quantized elemwise modes that use no libm function, transcribed expression by expression
+ * from dnn/src/common/elemwise/kern_defs.cuh (unary :166-208, binary :229-295, ternary :311-313; fast_tanh :44-46,
+ * fuse_add_hswish :52-55, fast_tanh_grad :57-61).  min / max there are std::min / std::max: max(a, b) = a < b ? b : a.
+ * x * y + z is a multiply and an add (this file is built with -ffp-contract=off), what an x86-64 build of the
+ * reference without FMA code generation evaluates.  Returns 0 for a mode outside the table (*ok = 0). */
+static float omax(float a, float b) { return a < b ? b : a; }
+static float omin(float a, float b) { return b < a ? b : a; }
+static float oracle_elemwise_float(uint32_t mode, float x, float y, float z, int* ok) {
+    *ok = 1;
+    switch (mode) {
+        case MI355_EW_RELU: return x <= 0.f ? 0.f : x;                                    /* :176 */
+        case MI355_EW_ABS: return fabsf(x);                                               /* :182 */
+        case MI355_EW_CEIL: return ceilf(x);                                              /* :187 */
+        case MI355_EW_FLOOR: return floorf(x);                                            /* :191 */
+        case MI355_EW_NEGATE: return -x;                                                  /* :166 */
+        case MI355_EW_ROUND: return roundf(x);                                            /* :198 */
+        case MI355_EW_FAST_TANH: return x * (27.f + x * x) / (27.f + 9.f * x * x);        /* :44-46 */
+        case MI355_EW_H_SWISH: return x * omin(omax(x + 3, 0.f), 6.f) * (1.f / 6.f);      /* :203 */
+        case MI355_EW_ABS_GRAD: return x > 0.f ? y : -y;                                  /* :230 */
+        case MI355_EW_ADD: return x + y;                                                  /* :234 */
+        case MI355_EW_FLOOR_DIV: return floorf(x / y);                                    /* :259 */
+        case MI355_EW_MAX: return x > y ? x : y;                                          /* :235 */
+        case MI355_EW_MIN: return x < y ? x : y;                                          /* :236 */
+        case MI355_EW_MUL: return x * y;                                                  /* :237 */
+        case MI355_EW_SIGMOID_GRAD: return x * (1.f - x) * y;                             /* :242 */
+        case MI355_EW_SUB: return x - y;                                                  /* :243 */
+        case MI355_EW_SWITCH_GT0: return x > 0.f ? y : 0.f;                               /* :246 */
+        case MI355_EW_TANH_GRAD: return (1.f - x * x) * y;                                /* :250 */
+        case MI355_EW_TRUE_DIV: return x / y;                                             /* :280 */
+        case MI355_EW_LT: return (float)(x < y);                                          /* :251 */
+        case MI355_EW_LEQ: return (float)(x <= y);                                        /* :252 */
+        case MI355_EW_EQ: return (float)(x == y);                                         /* :253 */
+        case MI355_EW_FUSE_ADD_RELU: return (x + y) <= 0.f ? 0.f : (x + y);               /* :268 */
+        case MI355_EW_FAST_TANH_GRAD: {                                                   /* :57-61 */
+            float x_pow2 = x * x;
+            float deno = 3.f + x_pow2;
+            return ((-48.f * x_pow2) / deno + 27.f + x_pow2) / (deno * 9.f) * y;
+        }
+        case MI355_EW_H_SWISH_GRAD:                                                       /* :287-290 */
+            return x < -3.f ? 0.f : (x > 3.f ? y : (2.f * x + 3.f) / 6.f * y);
+        case MI355_EW_FUSE_ADD_H_SWISH: {                                                 /* :52-55 */
+            float t = x + y;
+            return t * omin(omax(t + 3, 0.f), 6.f) * (1.f / 6.f);
+        }
+        case MI355_EW_COND_LEQ_MOV: return x <= y ? z : 0.f;                              /* :311 */
+        case MI355_EW_COND_LT_MOV: return x < y ? z : 0.f;                                /* :312 */
+        case MI355_EW_FUSE_MUL_ADD3: return x * y + z;                                    /* :313 */
+        default: *ok = 0; return 0.f;
+    }
+}
+
+/* ElemwiseMultiType::on_quantized_mode, naive: dst = dst_param.quantize(KernImpl::apply(param0.dequantize(a), ...))
+ * (dnn/src/naive/elemwise_multi_type/opr_impl.h:45-66 one input, :88-116 two, :142-175 three); dequantize =
+ * float(x) * scale (dtype.h:854, :897).  Inputs share one dtype; src and dst are int8 or int32 arrays. */
+int oracle_elemwise_q(const mi355_elemwise_desc* d, const void* s0, const void* s1, const void* s2, void* dst) {
+    int ok;
+    (void)oracle_elemwise_float(d->mode, 0.f, 0.f, 0.f, &ok);
+    if (!ok) return MI355_ERR_UNSUPPORTED;
+    if (d->arity < 1 || d->arity > 3) return MI355_ERR_BAD_ARG;
+    const void* src[3] = {s0, s1, s2};
+    const int s32 = d->src_dtype == MI355_DT_QS32, d32 = d->dst_dtype == MI355_DT_QS32;
+    for (uint64_t i = 0; i < d->count; ++i) {
+        float v[3] = {0.f, 0.f, 0.f};
+        for (uint32_t k = 0; k < d->arity; ++k)
+            v[k] = (s32 ? (float)((const int32_t*)src[k])[i] : (float)((const int8_t*)src[k])[i]) * d->scale_src[k];
+        const float r = oracle_elemwise_float(d->mode, v[0], v[1], v[2], &ok);
+        if (d32)
+            ((int32_t*)dst)[i] = oracle_quantize_s32(r, d->scale_dst);
+        else
+            ((int8_t*)dst)[i] = oracle_quantize_s8(r, d->scale_dst);
+    }
+    return MI355_OK;
+}
+
 /* TypeCvt Float32 <-> QuantizedS8 over n elements (naive/type_cvt/opr_impl.cpp:24-56: quantize / dequantize of
  * dtype.h:845-854, the scalar functions above) */
 void oracle_typecvt_f32_s8(uint64_t n, float scale, const float* src, int8_t* dst) {

@@ -55,6 +55,8 @@ def lib():
         L.oracle_round_sweep.argtypes = [C.c_uint32, C.c_uint32, P(C.c_float)]
         L.oracle_pooling_s8.restype = C.c_int
         L.oracle_pooling_s8.argtypes = [P(_abi.PoolingDesc), C.c_void_p, C.c_void_p]
+        L.oracle_elemwise_q.restype = C.c_int
+        L.oracle_elemwise_q.argtypes = [P(_abi.ElemwiseDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.oracle_typecvt_f32_s8.restype = None
         L.oracle_typecvt_f32_s8.argtypes = [C.c_uint64, C.c_float, C.c_void_p, C.c_void_p]
         L.oracle_typecvt_s8_f32.restype = None
@@ -156,6 +158,19 @@ def requant(src, scale_src, scale_dst, nonline=0, z=None, scale_z=1.0):
     dst = np.empty(src.shape, np.int8)
     zc = None if z is None else np.ascontiguousarray(z, dtype=np.int8)
     st = lib().oracle_requant_s32_s8(C.byref(d), _ptr(src), _ptr(zc) if zc is not None else None, _ptr(dst))
+    if st:
+        raise OracleError(st)
+    return dst
+
+
+def elemwise_q(mode, srcs, scales_src, scale_dst, dst_dtype=np.int8):
+    """quantized elemwise mode (by Elemwise::Mode name) on one to three int8 or int32 arrays; returns dst_dtype"""
+    srcs = [np.ascontiguousarray(s) for s in srcs]
+    code = {np.dtype(np.int8): _abi.DT_QS8, np.dtype(np.int32): _abi.DT_QS32}
+    d = _abi.make_elemwise_desc(mode, scales_src, scale_dst, srcs[0].size, code[srcs[0].dtype], code[np.dtype(dst_dtype)])
+    dst = np.empty(srcs[0].shape, dst_dtype)
+    p = [_ptr(s) for s in srcs] + [None] * (3 - len(srcs))
+    st = lib().oracle_elemwise_q(C.byref(d), p[0], p[1], p[2], _ptr(dst))
     if st:
         raise OracleError(st)
     return dst

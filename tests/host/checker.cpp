@@ -399,6 +399,7 @@ static void run_cache_roundtrip() {
 // ------------------------------------------------------------------ elementwise requantisation (GPU)
 extern "C" int oracle_requant_s32_s8(const mi355_requant_desc* d, const int32_t* src, const int8_t* z, int8_t* dst);
 extern "C" int oracle_requant_s8_s8(const mi355_requant_desc* d, const int8_t* src, const int8_t* z, int8_t* dst);
+extern "C" int oracle_elemwise_q(const mi355_elemwise_desc* d, const void* s0, const void* s1, const void* s2, void* dst);
 
 static void run_elemwise_gpu(Handle* h) {
     printf("case: ElemwiseMultiType quantized modes and TypeCvt\n");
@@ -455,6 +456,47 @@ static void run_elemwise_gpu(Handle* h) {
         EXPECT(bad == 0, "TypeCvt: %zu bytes differ", bad);
         opr->param().mode = EM::QADD;
         EXPECT(throws([&] { opr->exec({TensorND(da.p, la)}, TensorND(dd.p, ld)); }, MI355_ERR_BAD_ARG), "QADD with one operand");
+    }
+    // the general entry point: modes outside the post-process chain, three operands, a QuantizedS32 destination
+    {
+        std::vector<int8_t> hc(n);
+        fill_s8(hc, 34, -128, 127);
+        DevBuf dc(n), dd32(n * 4);
+        HIP_OK(hipMemcpy(dc.p, hc.data(), n, hipMemcpyHostToDevice));
+        const float s_c = 0.9f;
+        TensorLayout lc(shp, dtype::QuantizedS8(s_c)), ld32(shp, dtype::QuantizedS32(0.004f));
+        struct G { EM mode; uint32_t ew, arity; const char* name; };
+        const G gm[] = {{EM::QMUL, MI355_EW_MUL, 2, "QMUL"}, {EM::QMAX, MI355_EW_MAX, 2, "QMAX"}, {EM::QTRUE_DIV, MI355_EW_TRUE_DIV, 2, "QTRUE_DIV"},
+                        {EM::QFUSE_MUL_ADD3, MI355_EW_FUSE_MUL_ADD3, 3, "QFUSE_MUL_ADD3"}, {EM::QCOND_LEQ_MOV, MI355_EW_COND_LEQ_MOV, 3, "QCOND_LEQ_MOV"},
+                        {EM::QABS, MI355_EW_ABS, 1, "QABS"}, {EM::QADD, MI355_EW_ADD, 2, "QADD"}};
+        std::vector<int32_t> expect32(n), got32(n);
+        for (int d32 = 0; d32 < 2; ++d32)
+            for (auto& m : gm) {
+                mi355_elemwise_desc d = mi355_elemwise_desc();
+                d.mode = m.ew; d.arity = m.arity; d.src_dtype = MI355_DT_QS8; d.dst_dtype = d32 ? MI355_DT_QS32 : MI355_DT_QS8;
+                d.scale_src[0] = s_a; d.scale_src[1] = s_b; d.scale_src[2] = s_c; d.scale_dst = d32 ? 0.004f : s_d; d.count = n;
+                void* want = d32 ? (void*)expect32.data() : (void*)expect.data();
+                EXPECT(oracle_elemwise_q(&d, ha.data(), hb.data(), hc.data(), want) == 0, "CPU checker refused %s", m.name);
+                opr->param().mode = m.mode;
+                std::vector<TensorND> src{TensorND(da.p, la)};
+                if (m.arity > 1) src.push_back(TensorND(db.p, lb));
+                if (m.arity > 2) src.push_back(TensorND(dc.p, lc));
+                if (m.mode == EM::QADD && !d32) continue;  // the chain's case, covered above
+                HIP_OK(hipMemset(d32 ? dd32.p : dd.p, 0x5a, d32 ? n * 4 : n));
+                opr->exec(src, d32 ? TensorND(dd32.p, ld32) : TensorND(dd.p, ld));
+                HIP_OK(hipStreamSynchronize((hipStream_t)h->stream()));
+                size_t bad = 0;
+                if (d32) {
+                    HIP_OK(hipMemcpy(got32.data(), dd32.p, n * 4, hipMemcpyDeviceToHost));
+                    for (size_t i = 0; i < n; ++i) bad += got32[i] != expect32[i];
+                } else {
+                    HIP_OK(hipMemcpy(got.data(), dd.p, n, hipMemcpyDeviceToHost));
+                    for (size_t i = 0; i < n; ++i) bad += got[i] != expect[i];
+                }
+                EXPECT(bad == 0, "%s (%s dst): %zu of %zu elements differ", m.name, d32 ? "s32" : "s8", bad, n);
+            }
+        opr->param().mode = (EM)18;  // QEXP: a libm mode
+        EXPECT(throws([&] { opr->exec({TensorND(da.p, la)}, TensorND(dd.p, ld)); }, MI355_ERR_UNSUPPORTED), "QEXP is refused");
     }
 }
 
