@@ -540,9 +540,14 @@ static int exec_impl(void* stream, const mi355_conv_desc* d, const mi355_algo* a
     // the tiled kernels use 16-byte vector accesses; misaligned tensors take the generic kernel
     if (id != ALGO_DIRECT && id != ALGO_NCHW_MFMA) {  // (the relayouts of plain NCHW tensors take any pointer)
         // (pack-32 tensors move as 16-byte vectors, pack-4 tensors as dwords)
-        const int sa = p.pin == 32 ? 16 : 4, da = p.pout == 32 ? 16 : 4;
-        bool al = aligned16(src) && aligned16(filter) && aligned16(dst) && (!bias || aligned16(bias)) &&
-                  (!z || aligned16(z)) && p.src_sn % sa == 0 && p.dst_sn % da == 0 && p.z_sn % da == 0;
+        // (a planar destination is written element by element: dst, z and a Float32 bias need their natural alignment only)
+        const int sa = p.pin == 32 ? 16 : 4, da = p.pout == 32 ? 16 : p.pout == 1 ? 1 : 4;
+        const bool planar = p.pout == 1 && id == ALGO_IGEMM_MFMA;
+        const uintptr_t el = d->dst_dtype == MI355_DT_F32 ? 3 : 0;
+        auto natural = [el](const void* q) { return (reinterpret_cast<uintptr_t>(q) & el) == 0; };
+        bool al = aligned16(src) && aligned16(filter) && (planar ? natural(dst) : aligned16(dst)) &&
+                  (!bias || (planar ? (reinterpret_cast<uintptr_t>(bias) & 3) == 0 : aligned16(bias))) &&
+                  (!z || (planar ? natural(z) : aligned16(z))) && p.src_sn % sa == 0 && p.dst_sn % da == 0 && p.z_sn % da == 0;
         if (!al) {
             // the generic kernel reads the reference filter layout only
             if (preprocessed || !by_heuristic)

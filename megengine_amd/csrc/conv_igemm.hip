@@ -362,7 +362,10 @@ struct IgemmKernel {
             // ---- bookkeeping
             if (last_stage) {
                 if (DUAL) acc[0][0] += alt;
-                igemm_run_epilogue<POUT, MT, NT>(a, acc, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh);
+                if (POUT == 1)
+                    igemm_epilogue_planar<MT, NT>(a, acc, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh);
+                else
+                    igemm_run_epilogue<POUT, MT, NT>(a, acc, c_oc0 + wm * WTM, c_pix0 + wn * WTN, l32, lh);
                 c_stage = 0;
                 c_tile += step;
                 if (a.tiles_m > 1) {
@@ -482,6 +485,15 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
 // tile_cfg numbering: register-staged tiles, LDS-direct tiles, second-generation tiles, patch-staged tiles
 int igemm_num_cfgs() { return kNumCfgs + igemm_dma_num_cfgs() + igemm2_num_cfgs() + igemm3_num_cfgs(); }
 int igemm_first_v2_cfg() { return kNumCfgs + igemm_dma_num_cfgs(); }
+// planar destination (NCHW4_NCHW): two of the register-staged tiles
+static int launch_planar(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
+    switch (cfg) {
+        case 0: return launch_one<4, 1, 128, 128, 2, 2, 2, 2>(st, a, cu);
+        case 3: return launch_one<4, 1, 64, 64, 2, 2, 4, 3>(st, a, cu);
+        default: return (int)hipErrorInvalidConfiguration;
+    }
+}
+
 static int igemm_first_v3_cfg() { return igemm_first_v2_cfg() + igemm2_num_cfgs(); }
 const char* igemm_cfg_name(int cfg) {
     if (cfg >= 0 && cfg < kNumCfgs) return kCfgs[cfg].name;
@@ -520,13 +532,17 @@ bool igemm_usable(const ConvProblem& p) {
     // group convolution: 32-packed tensors whose groups are whole channel blocks (second-generation tiles only), or
     // NCHW4 with whole blocks of 4 on both sides, one dense launch per group (igemm_group_view)
     if (d.group != 1 && !(p.pin == 32 && p.icpg % 32 == 0 && p.ocpg % 32 == 0) && !igemm_group_by_launch(p)) return false;
+    // planar destination (NCHW4_NCHW: QuantizedS8 or Float32 dst, any bias shape, any scales): dense, on two of the
+    // register-staged tiles, whose planar epilogue covers all of it
+    const bool planar = d.format == MI355_FMT_NCHW4_NCHW;
+    if (planar && (d.group != 1 || d.dst_dtype == MI355_DT_QS32)) return false;
     if (d.format != MI355_FMT_NCHW4 && d.format != MI355_FMT_NCHW32 && d.format != MI355_FMT_NCHW4_NCHW32 &&
-        d.format != MI355_FMT_NCHW32_NCHW4)
+        d.format != MI355_FMT_NCHW32_NCHW4 && !planar)
         return false;
     if (d.mode != MI355_MODE_CROSS_CORRELATION || d.dilate_h != 1 || d.dilate_w != 1) return false;
     // QuantizedS32 dst (without a residual), full-shape bias and scales outside the fast forms' envelope run the
     // second-generation tiles with their general epilogue: 32-packed inputs only
-    if (igemm_needs_general(p)) {
+    if (igemm_needs_general(p) && !planar) {
         if (p.pin != 32) return false;
         if (d.dst_dtype == MI355_DT_F32) return false;
     }
@@ -547,6 +563,11 @@ bool igemm_usable(const ConvProblem& p) {
 
 static int pick_cfg_by_shape(const ConvProblem& p, int cu_count, bool will_preprocess) {
     const mi355_conv_desc& d = p.d;
+    if (p.pout == 1) {
+        // planar destination: 128 x 128 tiles once they fill the device, else 64 x 64
+        const int64_t t128 = (int64_t)((d.oc + 127) / 128) * (((int64_t)d.n * p.oh * p.ow + 127) / 128);
+        return d.oc > 64 && t128 >= (cu_count > 0 ? cu_count : 256) ? 0 : 3;
+    }
     if (will_preprocess && p.pin == 32 && p.pout == 32 && d.group == 1 && !igemm_needs_general(p)) {
         // The caller re-tiles the filter for the chosen algorithm (weight pre-processing): the second-generation tiles
         // then copy whole kilobytes for both operands.  Every tile was forced on every ResNet-50 shape in turn and timed
@@ -687,7 +708,9 @@ static void igemm_fill_args(const ConvProblem& p, IgemmArgs& a) {
     a.groups = d.group;
     a.ocpg = p.ocpg;
     a.src_sg = (p.icpg / p.pin) * a.src_scb;
-    a.general = igemm_needs_general(p) ? 1 : 0;
+    a.general = igemm_needs_general(p) && p.pout != 1 ? 1 : 0;
+    a.dst_f32 = d.dst_dtype == MI355_DT_F32;
+    if (a.dst_f32) a.has_bias = 0;  // a Float32 bias is added by the planar epilogue, not to the int32 accumulators
     a.dst_s32 = d.dst_dtype == MI355_DT_QS32;
     a.bias_full = d.bias_mode == MI355_BIAS_FULL;
     if (a.dst_s32) a.epi.s_b = a.epi.s_d;  // the sum lives in dst and is dequantised with the dtype of dst
@@ -707,6 +730,7 @@ int igemm_resolve_cfg(const ConvProblem& p, int cfg) {
     IgemmArgs a;
     igemm_fill_args(p, a);
     if (a.M == 0 || a.OC == 0) return cfg;  // nothing is launched
+    if (p.pout == 1) return cfg == 3 ? 3 : 0;  // planar destination: two register-staged tiles
     const int first_v2 = igemm_first_v2_cfg();
     // group convolutions and the general epilogue exist on the second-generation tiles only
     if ((d.group != 1 || a.general) && cfg < first_v2) cfg = first_v2 + (p.ocpg <= 64 ? 3 : 0);
@@ -778,6 +802,10 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
         a.flt_rstride = 32;
         a.flt_kstride = ocp * 32;
         a.flt_bytes = (uint32_t)igemm_preprocessed_bytes(p, cfg);
+    }
+    if (p.pout == 1) {
+        if (p.d.bias_mode == MI355_BIAS_NONE) a.bias = nullptr;  // the planar epilogue tests the pointer
+        return launch_planar(st, a, cfg, cu_count);
     }
     const int first_v2 = igemm_first_v2_cfg();
     if (cfg >= igemm_first_v3_cfg()) return launch_igemm3(st, a, p.pin, p.pout, cfg - igemm_first_v3_cfg());

@@ -44,6 +44,8 @@ struct IgemmArgs {
     // general epilogue (second-generation kernel): QuantizedS32 dst, full-shape bias, or scales outside the fast
     // forms' envelope.  bias_full: a.bias has the shape of dst (contiguous) and has_bias is 0.
     int general, dst_s32, bias_full;
+    // planar destination (format NCHW4_NCHW, register-staged kernel): dst_f32 = dst, bias and z are Float32 tensors
+    int dst_f32;
     // tile decoding of the LDS-direct kernels without run-time integer divisions (each costs ~30 scalar instructions and a
     // reciprocal on the critical path from kernel entry to the first copy): by the number of channel tiles, by the
     // channel tiles of a group, and by the tile stride of a workgroup (set by the launch code, which knows the grid)
@@ -254,6 +256,101 @@ __device__ __forceinline__ void igemm_epilogue_general(const IgemmArgs& a, v16i 
             }
         }
     }
+}
+
+// Epilogue of one wave tile for a planar destination (format NCHW4_NCHW: dst, z and a full-shape bias are NCHW tensors,
+// dnn/src/common/convolution.cpp:929-947).  Register quad q of a 32x32 block holds four consecutive channels of one pixel:
+// four stores OHW elements apart, each contiguous over the 32 lanes of a half wave.  QuantizedS8 dst: the requantisation
+// chain in whichever form the scales allow; Float32 dst: the exact sum dequantised once, then bias, z and activation in
+// float (forward_bias and handle_z_inp_and_activation_naive on float tensors, dnn/src/naive/conv_bias/opr_impl.cpp:21-98).
+enum { PLANAR_F32 = 0, PLANAR_S8_EXACT = 1, PLANAR_S8_FAST = 2 };
+template <int MT, int NT, int KIND, int NL, bool HZ>
+__device__ __forceinline__ void igemm_epilogue_planar_as(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w, int l32,
+                                                         int lh) {
+    const bool hz = KIND == PLANAR_S8_FAST ? HZ : a.epi.has_z != 0;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int m = pix_w + j * 32 + l32;
+        const bool pok = m < a.M;
+        const uint32_t mm = pok ? m : 0;
+        const uint32_t n = fdiv(mm, a.div_ohw), rem = mm - n * a.OHW;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int ocb = oc_w + i * 32;
+            const v16i& c = acc[i][j];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int oc4 = ocb + 8 * q + 4 * lh;
+                const int left = pok ? a.OC - oc4 : 0;              // channels of this quad that exist (<= 0: none)
+                const int64_t in_img = (int64_t)oc4 * a.OHW + rem;  // element of channel oc4 inside one image
+                const int64_t full = (int64_t)n * ((int64_t)a.OC * a.OHW) + in_img;
+                if (KIND == PLANAR_F32) {
+                    float* dp = reinterpret_cast<float*>(a.dst) + (int64_t)n * a.dst_sn + in_img;
+                    const float* zp = reinterpret_cast<const float*>(a.z) + (int64_t)n * a.z_sn + in_img;
+                    const float* fb = reinterpret_cast<const float*>(a.bias);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (r < left) {
+                            float v = (float)c[4 * q + r] * a.epi.s_b;
+                            if (a.bias_full)
+                                v = v + fb[full + (int64_t)r * a.OHW];
+                            else if (a.bias)
+                                v = v + fb[oc4 + r];
+                            if (hz) v = v + zp[(int64_t)r * a.OHW];
+                            if (a.epi.nonline == NL_RELU)
+                                v = v <= 0.f ? 0.f : v;
+                            else if (a.epi.nonline == NL_H_SWISH)
+                                v = v * fminf(fmaxf(v + 3.f, 0.f), 6.f) * (1.f / 6.f);
+                            dp[(int64_t)r * a.OHW] = v;
+                        }
+                    }
+                } else {
+                    int8_t* dp = a.dst + (int64_t)n * a.dst_sn + in_img;
+                    const int8_t* zp = a.z + (int64_t)n * a.z_sn + in_img;
+                    int v[4] = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
+                    uint32_t zw = 0;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (r < left) {
+                            if (a.bias_full) v[r] += a.bias[full + (int64_t)r * a.OHW];
+                            if (hz) zw |= (uint32_t)(uint8_t)zp[(int64_t)r * a.OHW] << (8 * r);
+                        }
+                    }
+                    const uint32_t o = KIND == PLANAR_S8_EXACT ? requant4_exact(v[0], v[1], v[2], v[3], zw, a.epi)
+                                                               : requant4_fast<NL, HZ>(v[0], v[1], v[2], v[3], zw, a.epi);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (r < left) dp[(int64_t)r * a.OHW] = (int8_t)(o >> (8 * r));
+                }
+            }
+        }
+    }
+}
+
+template <int MT, int NT>
+__device__ __forceinline__ void igemm_epilogue_planar(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w, int l32,
+                                                      int lh) {
+#define MI355_PLANAR(KIND, NL, HZ) igemm_epilogue_planar_as<MT, NT, KIND, NL, HZ>(a, acc, oc_w, pix_w, l32, lh)
+    if (a.dst_f32) {
+        MI355_PLANAR(PLANAR_F32, NL_IDENTITY, false);
+    } else if (!a.epi.fast) {
+        MI355_PLANAR(PLANAR_S8_EXACT, NL_IDENTITY, false);
+    } else if (a.epi.lin) {
+        MI355_PLANAR(PLANAR_S8_FAST, NL_LIN, false);
+    } else if (a.epi.has_z) {
+        switch (a.epi.nonline) {
+            case NL_RELU: MI355_PLANAR(PLANAR_S8_FAST, NL_RELU, true); break;
+            case NL_H_SWISH: MI355_PLANAR(PLANAR_S8_FAST, NL_H_SWISH, true); break;
+            default: MI355_PLANAR(PLANAR_S8_FAST, NL_IDENTITY, true); break;
+        }
+    } else {
+        switch (a.epi.nonline) {
+            case NL_RELU: MI355_PLANAR(PLANAR_S8_FAST, NL_RELU, false); break;
+            case NL_H_SWISH: MI355_PLANAR(PLANAR_S8_FAST, NL_H_SWISH, false); break;
+            default: MI355_PLANAR(PLANAR_S8_FAST, NL_IDENTITY, false); break;
+        }
+    }
+#undef MI355_PLANAR
 }
 
 // LDS-direct variant (conv_igemm_dma.hip): global -> LDS copies without a register stage

@@ -86,6 +86,52 @@ def test_nchw4_nchw(oracle, i):
                tag="nchw4_nchw s32")
 
 
+NCHW4_NCHW_MFMA_CASES = [
+    dict(fmt="NCHW4_NCHW", n=3, ic=32, ih=20, iw=20, oc=150, fh=3, pad=1),           # several tiles both ways, ragged channels
+    dict(fmt="NCHW4_NCHW", n=2, ic=16, ih=23, iw=20, oc=37, fh=3, pad=1),            # oc % 4 != 0: a quad that ends early
+    dict(fmt="NCHW4_NCHW", n=2, ic=64, ih=12, iw=16, oc=24, fh=1),                    # pointwise fast path
+    dict(fmt="NCHW4_NCHW", n=1, ic=8, ih=31, iw=9, oc=1000, fh=5, pad=2, stride=2),   # a classifier-like tail: many channels
+]
+
+
+@pytest.mark.parametrize("i", range(len(NCHW4_NCHW_MFMA_CASES)))
+def test_nchw4_nchw_on_the_mfma_kernel(oracle, i):
+    """The planar epilogue of the register-staged tiles: QuantizedS8 dst bit-exact in every requantisation form, with
+    channel, full-shape and no bias; Float32 dst exact where float arithmetic is exact and to the reference checker's
+    tolerance elsewhere.  The heuristic takes the MFMA algorithm for dense problems of this format."""
+    c = NCHW4_NCHW_MFMA_CASES[i]
+    names = lib.tile_names()
+    d = mk(c, nonline="RELU", **S)
+    assert ops.conv_bias_query(d)[0].id == IGEMM
+    usable = [t for t in range(len(names)) if lib.tile_usable(d, t)]
+    assert [names[t] for t in usable] == ["128x128x64", "64x64x128"]
+    for tile in usable:
+        for nl in ("IDENTITY", "RELU", "H_SWISH"):
+            for has_z in (False, True):
+                tag = "nchw4_nchw mfma %s" % names[tile]
+                check_case(oracle, mk(c, nonline=nl, has_z=has_z, **S), seed=140 + i, algo=IGEMM, tile=tile, tag=tag)
+                check_case(oracle, mk(c, nonline=nl, has_z=has_z, dst_dtype=_abi.DT_F32, scale_bias=0.0173, scale_z=0.0041),
+                           seed=160 + i, algo=IGEMM, tile=tile, tag=tag + " f32")
+        # scales outside the divide-free forms (the literal chain), a full-shape bias, no bias
+        check_case(oracle, mk(c, nonline="H_SWISH", has_z=True, scale_bias=3.1e-7, scale_z=1e-6, scale_dst=2.9e-6), seed=170 + i,
+                   algo=IGEMM, tile=tile, tag="nchw4_nchw mfma literal chain")
+        check_case(oracle, mk(c, nonline="RELU", has_z=True, bias_mode=_abi.BIAS_FULL, **S), seed=171 + i, algo=IGEMM, tile=tile,
+                   tag="nchw4_nchw mfma full bias")
+        check_case(oracle, mk(c, nonline="IDENTITY", bias_mode=_abi.BIAS_NONE, **S), seed=172 + i, algo=IGEMM, tile=tile,
+                   tag="nchw4_nchw mfma no bias")
+        check_case(oracle, mk(c, nonline="RELU", has_z=True, bias_mode=_abi.BIAS_FULL, dst_dtype=_abi.DT_F32, scale_bias=0.0173,
+                              scale_z=0.0041), seed=173 + i, algo=IGEMM, tile=tile, tag="nchw4_nchw mfma f32 full bias")
+        # exact: unit scales, so every float product and partial sum is a small integer
+        d = mk(c, nonline="RELU", has_z=True, dst_dtype=_abi.DT_F32, scale_bias=1.0, scale_z=0.5)
+        src, flt, bias, z = util.make_tensors(d, seed=180 + i, src_range=(-8, 8), flt_range=(-8, 8))
+        want = oracle.conv_bias(d, src, flt, bias, z)
+        got = run_gpu(d, src, flt, bias, z, algo=IGEMM, tile=tile)
+        assert np.array_equal(got, want)
+    # what stays on the generic kernel: groups and a QuantizedS32 destination
+    assert ops.conv_bias_query(mk(NCHW4_NCHW_CASES[3], **S))[0].id == DIRECT
+    assert ops.conv_bias_query(mk(c, dst_dtype=_abi.DT_QS32, scale_bias=2e-4, scale_dst=2e-4))[0].id == DIRECT
+
+
 def test_direct_s32_dst_and_full_bias(oracle, kats):
     # the reference KAT itself, on the GPU (QuantizedS32 dst and z)
     k = kats["conv_bias_quantized8x8x32"]
