@@ -30,6 +30,17 @@ def test_host_classes_cpu():
     _run("--cpu", allow_build=True)
 
 
+def test_abi_calls_from_many_threads():
+    """tests/host/abi_stress.cpp: eight threads ask the host-side calls of the C ABI (deduce, query, usability, proofs) about
+    1500 random descriptors, valid and invalid; every answer equals the one computed first.  The same driver runs under
+    AddressSanitizer / UndefinedBehaviorSanitizer / ThreadSanitizer with `make -C tests/host sanitize` and `... tsan`."""
+    _binary(allow_build=True)
+    exe = os.path.join(ROOT, "tests", "host", "abi_stress")
+    r = subprocess.run([exe, "8", "1500"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    print(r.stdout)
+    assert r.returncode == 0 and "ALL OK" in r.stdout, r.stdout[-4000:]
+
+
 @pytest.mark.gpu
 def test_host_classes_gpu():
     """exec of every listed algorithm through the C++ classes, bit-exact against the CPU checker"""
