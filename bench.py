@@ -440,6 +440,17 @@ def run_extras(torch, np, _abi, lib, ops, workloads, side_iters=50):
         t_in = time_launches(torch, lambda: ops.relayout_exec(d_in, x_nchw, p["src"]), iters=n10)
         t_out = time_launches(torch, lambda: ops.relayout_exec(d_out, p["dst"], y_nchw), iters=n10)
         rl_bytes_in, rl_bytes_out = 2 * x_nchw.numel(), 2 * y_nchw.numel()
+        # the same launch (same instruction stream, same addresses) with every operand byte zero: what the kernel's
+        # schedule reaches when the matrix units switch no bits.  The difference from "us" is the part of the time that
+        # the power limit of the device, not the schedule, decides.
+        for t_ in (p["src"], p["flt"], p["bias"], p["z"], p.get("pre")):
+            if t_ is not None:
+                t_.zero_()
+        conv()
+        torch.cuda.synchronize()
+        t_zero = min(time_launches(torch, conv, iters=n10), time_launches(torch, conv, iters=n10))
+        rows[0]["us_zero_operands"] = round(t_zero * 1e6, 2)
+        rows[0]["tops_zero_operands"] = round(l.ops / t_zero / 1e12, 1)
         # (these tensors are 67-134 MB each and stream through both caches: every launch is a cold one)
         c4.append(dict(conv=rows[0], total_us=round(t_full * 1e6, 1),
                        relayout_in_gbs=round(rl_bytes_in / t_in / 1e9, 1),

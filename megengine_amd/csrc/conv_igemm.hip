@@ -573,6 +573,7 @@ static int pick_cfg_by_shape(const ConvProblem& p, int cu_count, bool will_prepr
         // then copy whole kilobytes for both operands.  Every tile was forced on every ResNet-50 shape in turn and timed
         // as whole-stack replays of one captured graph, against the unchanged stack in the same process.
         enum { V128x128x64r4 = 0, V64x128x128r3 = 3, V64x128x64r4 = 4, V64x64x128r4 = 8, V128x256x64w8 = 10, V256x256x64w8 = 11 };
+        enum { V3_128x128x256r3 = 6 };
         const int v2 = igemm_first_v2_cfg();
         const int cu = cu_count > 0 ? cu_count : 256;
         const int64_t M = (int64_t)d.n * p.oh * p.ow;
@@ -593,6 +594,11 @@ static int pick_cfg_by_shape(const ConvProblem& p, int cu_count, bool will_prepr
             // small tile with the deepest ring
             if (pw) return v2 + (kb >= 2048 && t128 < cu ? V64x64x128r4 : V64x128x128r3);
             if (kb >= 4608) return v2 + V64x64x128r4;
+            // 3x3 over 256 channels at stride 1 with one 128 x 128 tile for most CUs: the patch-staged tile, whose stage of
+            // eight k-chunks halves both the bytes through the CU's copy path and the stage boundaries (-1.4 us per
+            // launch against the tile below on 256 -> 256 at 14 x 14, batch 64; falls back when the patch does not fit)
+            if (d.fh == 3 && d.fw == 3 && d.stride_h == 1 && d.stride_w == 1 && kb >= 2304 && 2 * t128 >= cu)
+                return igemm_first_v3_cfg() + V3_128x128x256r3;
             if (d.stride_h == 1 && d.stride_w == 1) return v2 + V64x128x128r3;
             // few tiles, strided 3x3 over at most 256 channels: the first-generation tiles below
         }

@@ -45,14 +45,14 @@ struct Igemm3 {
     static constexpr int STG = KCH * NBA * 1024;   // filter bytes of one stage
     static constexpr int UA = KCH * NBA / NW;      // filter copies per wave per stage
     static constexpr int RA = NBA >= NW ? NBA / NW : 1;
-    static constexpr int U = UA;                   // copies per wave per stage that the explicit waits count
+    static constexpr int U = UA + PCS;             // copies per wave per stage at most: filter copies and patch-copy slots
     static constexpr int PCW_MAX = 4;              // patch copies per wave and patch, at most
     static constexpr int BIAS_OFF = NS * STG, PATCH_OFF = BIAS_OFF + BM * 4;
     static_assert(NW == 4 || NW == 8, "4 or 8 waves");
     static_assert(MT >= 1 && NT >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "wave tile");
     static_assert((KCH * NBA) % NW == 0 && (NBA >= NW ? NBA % NW == 0 : NW % NBA == 0), "filter copies divide over the waves");
     static_assert(KCH % 2 == 0, "fragment double buffer: the first chunk of a stage uses register set 0");
-    static_assert(NS >= 3 && (NS - 1) * (U + PCS) + PCW_MAX < 64, "ring depth vs the 6-bit vmcnt");
+    static_assert(NS >= 3 && (NS - 1) * U + PCW_MAX < 64, "ring depth vs the 6-bit vmcnt");
 
     __device__ static __forceinline__ int copy_chunk(int j, int w) { return NBA >= NW ? j / RA : j * (NW / NBA) + w / NBA; }
     __device__ static __forceinline__ int copy_bi(int j) { return NBA >= NW ? j % RA : 0; }
@@ -74,7 +74,24 @@ struct Igemm3 {
     }
     static_assert(UA >= KCH ? UA % KCH == 0 : KCH % UA == 0, "filter copies vs chunk steps");
     static_assert(PCS >= 1 && PCS <= KCH && KCH % PCS == 0, "patch copies vs chunk steps");
-    static constexpr int CS_LAST = copies_in_step<UA>(KCH - 1);
+    static constexpr int CA_LAST = copies_in_step<UA>(KCH - 1);
+    // Patch copies are issued before the filter copies of their chunk step, and no patch-copy slot lies behind the last step
+    // that has a filter copy: every patch copy issued with a stage is older than that stage's last filter copy.
+    static_assert(copies_in_step<PCS>(KCH - 1) == 0 && step_of<PCS>(PCS - 1) <= step_of<UA>(UA - 1), "patch slots vs filter copies");
+    static_assert(NS <= 4, "the waits look two issued stages back");
+
+    // s_waitcnt vmcnt(B + extra) for a wave-uniform extra in 0 .. MAXE (the count is an immediate of the instruction)
+    template <int B, int MAXE>
+    __device__ static __forceinline__ void wait_vmcnt_plus(int extra) {
+        if constexpr (MAXE == 0) {
+            wait_vmcnt<B>();
+        } else {
+            if (extra >= MAXE)
+                wait_vmcnt<B + MAXE>();
+            else
+                wait_vmcnt_plus<B, MAXE - 1>(extra);
+        }
+    }
 
     // M0 = wave-uniform LDS address, offset = per-lane base + wave-uniform term (the add sits between the write of M0 and
     // the copy, which needs one wait state after it)
@@ -137,9 +154,9 @@ struct Igemm3 {
         // patch copies of this wave: copy id = k NW + wave covers 64 patch pixels of one 16-byte plane
         const int cpp = a.pxp >> 6;  // copies per plane
         const int npct = 2 * cpp;    // ... per patch; a.pcw = copies per wave = ceil(npct / NW) <= PCW_MAX
-        int poff[PCW_MAX];
-#pragma unroll
-        for (int k = 0; k < PCW_MAX; ++k) {
+        // (four scalars, not an array: a selection among array elements by the run-time copy index would be folded into an
+        // indexed load from scratch memory, and a scratch load in the loop waits for every copy in flight)
+        auto patch_offset = [&](int k) __attribute__((always_inline)) -> int {
             const int id = k * NW + wave;
             const int plane = id >= cpp ? 1 : 0;
             const int u = (id - plane * cpp) * 64 + lane;  // patch pixel
@@ -149,8 +166,10 @@ struct Igemm3 {
             const uint32_t n = fdiv(R, a.div_phimg);
             const int ih = (int)(R - n * (uint32_t)PHI) - a.ph, iw = pcol - a.pw;
             const bool ok = id < npct && (int)n < a.NB && (unsigned)ih < (unsigned)a.IH && (unsigned)iw < (unsigned)a.IW;
-            poff[k] = ok ? (int)n * a.src_sn + (ih * a.IW + iw) * 32 + plane * 16 : SENT;
-        }
+            return ok ? (int)n * a.src_sn + (ih * a.IW + iw) * 32 + plane * 16 : SENT;
+        };
+        static_assert(PCW_MAX == 4, "four patch-copy offsets per lane");
+        const int poff0 = patch_offset(0), poff1 = patch_offset(1), poff2 = patch_offset(2), poff3 = patch_offset(3);
 
         // filter copies: byte offset of (row, half) of this lane, chunk added per copy
         const int rib = 16 * (lane >> 5) + (lane & 15), half = (lane >> 4) & 1;
@@ -186,15 +205,21 @@ struct Igemm3 {
         const int pcw = a.pcw, cbs = a.cbs;
         const uint32_t wave_k = (uint32_t)(wave * 1024);
 
+        int pc_cur = 0, pc_prev = 0;  // patch copies this wave issued with the stage being issued / with the one before
         auto patch_copy = [&]() __attribute__((always_inline)) {
-            // The next copy of the patch being fetched, if it has one left for this wave (wave-uniform).  The explicit
-            // waits count filter copies only: vector-memory operations complete in order, so a wait that allows fewer
-            // operations in flight than were issued behind the stage it waits for is stricter, never too weak.
+            // The next copy of the patch being fetched, if this wave has one left (wave-uniform).  The explicit waits count
+            // the copies that may stay in flight exactly: the filter copies of the stages behind the awaited one, a
+            // compile-time number, plus the patch copies issued with those stages, counted here.  (A wait that ignored the
+            // patch copies would wait for copies issued a moment ago; a copy with every lane out of range in each empty
+            // slot, to make the number constant, costs more than the real copies.)
             if (p_slot < pcw && p_cb < cbs && p_slot * NW + wave < npct) {
-                int off = poff[0];
-#pragma unroll
-                for (int k = 1; k < PCW_MAX; ++k) off = p_slot == k ? poff[k] : off;
+#ifdef V3_ABLATE_CONTIG
+                const int off = lane * 16 + p_slot * 1024;
+#else
+                const int off = p_slot == 0 ? poff0 : p_slot == 1 ? poff1 : p_slot == 2 ? poff2 : poff3;
+#endif
                 copy_at(p_dst + (uint32_t)(p_slot * NW * 1024) + wave_k, p_src, off, rs_src);
+                ++pc_cur;
             }
             ++p_slot;
         };
@@ -218,26 +243,31 @@ struct Igemm3 {
         auto loader_advance = [&]() __attribute__((always_inline)) {
             l_kc0 += KCH;
             l_kA += dA;
+            pc_prev = pc_cur;
+            pc_cur = 0;
         };
 
         __syncthreads();  // table ready
 
         // prologue: the first patch whole, then stages 0 .. NS - 2
+        {
+            const int pk[PCW_MAX] = {poff0, poff1, poff2, poff3};
 #pragma unroll
-        for (int k = 0; k < PCW_MAX; ++k) {
-            const int id = k * NW + wave;
-            if (k < pcw && id < npct) copy_at(lds0 + (uint32_t)(PATCH_OFF + id * 1024), 0, poff[k], rs_src);
+            for (int k = 0; k < PCW_MAX; ++k) {
+                const int id = k * NW + wave;
+                if (k < pcw && id < npct) copy_at(lds0 + (uint32_t)(PATCH_OFF + id * 1024), 0, pk[k], rs_src);
+            }
         }
 #pragma unroll
         for (int s = 0; s < NS - 1; ++s) {
             patch_switch();
-            for_each([&](auto jj) __attribute__((always_inline)) { filter_copy(jj, lds0 + (uint32_t)(s * STG)); },
-                     std::make_integer_sequence<int, UA>{});
 #pragma unroll
             for (int i = 0; i < PCS; ++i) patch_copy();
+            for_each([&](auto jj) __attribute__((always_inline)) { filter_copy(jj, lds0 + (uint32_t)(s * STG)); },
+                     std::make_integer_sequence<int, UA>{});
             loader_advance();
         }
-        wait_vmcnt<(NS - 2) * U>();  // stage 0, the first patch, the bias
+        wait_vmcnt<(NS - 2) * UA>();  // stage 0, the first patch, the bias (and, stricter than needed, the patch copies behind them)
         __syncthreads();
 
         const int fragpos = ((l32 >> 4) * 2 + lh) * 256 + (l32 & 15) * 16;
@@ -280,7 +310,7 @@ struct Igemm3 {
             constexpr bool LAST = c + 1 == KCH;
             if (LAST) {
                 wait_lgkmcnt0();
-                wait_vmcnt<(NS - 2) * U - CS_LAST>();
+                wait_vmcnt_plus<(NS - 2) * UA - CA_LAST, (NS - 2) * PCS>(pc_cur + (NS >= 4 ? pc_prev : 0));
                 __syncthreads();
             }
             constexpr int CA = copies_in_step<UA>(c), CP = copies_in_step<PCS>(c);
@@ -301,13 +331,13 @@ struct Igemm3 {
                     fb[cn & 1][k - MT] = *reinterpret_cast<const v4i*>(lds + vB[k - MT] + bo);
                 } else if constexpr (c == 0 && k == PC) {
                     patch_switch();  // before the first copy of the stage
-                } else if constexpr (k < K0 + CA) {
+                } else if constexpr (k < K0 + CP) {
+                    patch_copy();
+                } else if constexpr (k < K0 + CP + CA) {
                     for_each([&](auto jj) __attribute__((always_inline)) {
                         constexpr int j = decltype(jj)::value;
-                        if constexpr (step_of<UA>(j) == c && nth_in_step<UA>(j) == k - K0) filter_copy(jj, lds0 + (uint32_t)wr_off);
+                        if constexpr (step_of<UA>(j) == c && nth_in_step<UA>(j) == k - K0 - CP) filter_copy(jj, lds0 + (uint32_t)wr_off);
                     }, std::make_integer_sequence<int, UA>{});
-                } else if constexpr (k < K0 + CA + CP) {
-                    patch_copy();
                 } else if constexpr (LAST && k == K0 + CA + CP) {
                     loader_advance();
                     wr_off = rd_off;
@@ -359,6 +389,9 @@ const Cfg3 kCfg3[] = {
         {"v3_128x256x64r4w8", 128, 256, 2},
         {"v3_256x256x64r3w8", 256, 256, 2},
         {"v3_128x128x128r3", 128, 128, 4},
+        {"v3_64x128x256r3", 64, 128, 8},
+        {"v3_128x128x256r3", 128, 128, 8},
+        {"v3_64x64x256r3", 64, 64, 8},
 };
 constexpr int kNumCfg3 = sizeof(kCfg3) / sizeof(kCfg3[0]);
 
@@ -428,6 +461,9 @@ int launch_cfg(hipStream_t st, IgemmArgs& a, int cfg) {
         case 2: return launch_k<128, 256, 2, 4, 2, 4, 3, 1, 4>(st, a);
         case 3: return launch_k<256, 256, 4, 2, 2, 3, 3, 1, 2>(st, a);
         case 4: return launch_k<128, 128, 2, 2, 4, 3, 4, 2, 2>(st, a);
+        case 5: return launch_k<64, 128, 2, 2, 8, 3, 5, 2, 2>(st, a);
+        case 6: return launch_k<128, 128, 2, 2, 8, 3, 5, 2, 2>(st, a);
+        case 7: return launch_k<64, 64, 2, 2, 8, 3, 5, 2, 2>(st, a);
         default: return -1;
     }
 }

@@ -370,6 +370,14 @@ def test_heuristic_picks(oracle):
                                ((160, 7, 960), "dma4_128x64x128"), ((96, 14, 576), "128x128x64")):
         a, _ = ops.conv_bias_query(_abi.make_conv_desc("NCHW4", 64, ic, hw, hw, oc, 1))
         assert a.id == IGEMM and names[a.tile_cfg] == want, (ic, hw, oc, names[a.tile_cfg])
+    # 32-packed layers of ResNet-50 at batch 64 for a caller that pre-processes the filter: second-generation tiles, and
+    # the patch-staged tile for the 3x3 layers over 256 channels
+    S8 = dict(scale_bias=2e-4, scale_z=0.05, scale_dst=0.05, nonline="RELU")
+    for (ic, hw, oc, f), want in (((256, 14, 256, 3), "v3_128x128x256r3"), ((1024, 14, 256, 1), "v2_64x128x128r3"),
+                                  ((64, 56, 64, 3), "v2_64x128x64r4"), ((512, 7, 512, 3), "v2_64x64x128r4")):
+        a, _ = ops.conv_bias_query(_abi.make_conv_desc("NCHW32", 64, ic, hw, hw, oc, f, pad=f // 2, **S8),
+                                   _abi.ALGO_HEURISTIC_PREPROCESS)
+        assert a.id == IGEMM and names[a.tile_cfg] == want, (ic, hw, oc, f, names[a.tile_cfg])
 
 
 def test_general_epilogue_on_the_mfma_kernel(oracle):
