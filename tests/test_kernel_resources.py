@@ -75,3 +75,16 @@ def test_general_epilogue_lives_in_its_own_instantiations(resources):
     gen = kernels(resources, r"igemm2_kernel<(32|4), [^>]*, true, 1>")
     tiles = {re.search(r"igemm2_kernel<(?:32|4), (\d+, \d+), ", k).group(1) for k in gen}
     assert tiles == {"128, 128", "64, 128"}, tiles
+
+
+def test_patch_staged_kernels_use_no_scratch(resources):
+    """igemm3_kernel: a selection among per-lane values by a run-time index was once folded into an indexed load from
+    scratch memory, and a scratch load in a loop that keeps LDS-direct copies in flight is followed by vmcnt(0): it
+    empties the ring.  (The kernels keep such values in scalars selected by compares.)"""
+    for name, r in kernels(resources, r"igemm3_kernel<").items():
+        assert r["scratch"] == 0, (name, r)
+
+
+def test_second_generation_kernels_use_no_scratch_in_the_tiles_the_heuristic_takes(resources):
+    for name, r in kernels(resources, r"igemm2_kernel<(32|4), (128, 128, 2, 2, 2, 4|64, 128, 2, 2, 4, 3|64, 128, 2, 2, 2, 4|64, 64, 2, 2, 4, 4), \d, (true|false), (true|false), false, 1>").items():
+        assert r["scratch"] == 0, (name, r)
