@@ -231,6 +231,17 @@ __global__ __launch_bounds__(C4_THREADS, 3) void c4_kernel(C4Args a) {
             }
         }
 
+        // The next tile's patch goes into LDS BEFORE this tile's stores are issued: the wait for its loads then counts no
+        // store (vector-memory operations are counted together and retire in order; behind the epilogue the same wait
+        // stood for fifteen of this tile's sixteen stores, i.e. every tile paid the latency of its own stores).
+        if (has_next) {
+            if (tn.mt != tl.mt) {
+                __syncthreads();  // every wave is done with the old weights
+                c4_load_weights(a, tn.mt, sW, wrow_dw, sBias, t);
+            }
+            c4_store_patch<S>(sP[buf ^ 1], t, preg);
+            __syncthreads();
+        }
         if (a.epi.lin) {
             c4_epilogue<NL_LIN, false>(a, acc, zr, doff, rs_dst);
         } else if (a.epi.has_z) {
@@ -247,12 +258,6 @@ __global__ __launch_bounds__(C4_THREADS, 3) void c4_kernel(C4Args a) {
             }
         }
         if (!has_next) break;
-        if (tn.mt != tl.mt) {
-            __syncthreads();  // every wave is done with the old weights
-            c4_load_weights(a, tn.mt, sW, wrow_dw, sBias, t);
-        }
-        c4_store_patch<S>(sP[buf ^ 1], t, preg);
-        __syncthreads();
         buf ^= 1;
         tile = next;
         tl = tn;
