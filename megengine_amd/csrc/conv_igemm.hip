@@ -572,7 +572,7 @@ static int pick_cfg_by_shape(const ConvProblem& p, int cu_count, bool will_prepr
         // The caller re-tiles the filter for the chosen algorithm (weight pre-processing): the second-generation tiles
         // then copy whole kilobytes for both operands.  Every tile was forced on every ResNet-50 shape in turn and timed
         // as whole-stack replays of one captured graph, against the unchanged stack in the same process.
-        enum { V128x128x64r4 = 0, V64x128x128r3 = 3, V64x128x64r4 = 4, V64x64x128r4 = 8, V128x256x64w8 = 10, V256x256x64w8 = 11 };
+        enum { V128x128x64r4 = 0, V128x128x128r3 = 2, V64x128x128r3 = 3, V64x128x64r4 = 4, V64x64x128r3 = 7, V64x64x128r4 = 8, V128x256x64w8 = 10, V256x256x64w8 = 11 };
         enum { V3_128x128x256r3 = 6 };
         const int v2 = igemm_first_v2_cfg();
         const int cu = cu_count > 0 ? cu_count : 256;
@@ -590,16 +590,23 @@ static int pick_cfg_by_shape(const ConvProblem& p, int cu_count, bool will_prepr
             // costs no LDS
             if (d.oc <= 64) return v2 + V64x128x64r4;
             if (t128 >= cu) return v2 + V128x128x64r4;
-            // pointwise: more pixels than channels per tile; with fewer tiles than CUs and a very long reduction the
-            // small tile with the deepest ring
-            if (pw) return v2 + (kb >= 2048 && t128 < cu ? V64x64x128r4 : V64x128x128r3);
-            if (kb >= 4608) return v2 + V64x64x128r4;
+            // a handful of tiles (small batches): the smallest tile puts the most CUs to work (3x3 256->256 at 14x14,
+            // batch 1 and 8: 7.4 / 7.6 us against 8.9 / 9.1 on 64 x 128 tiles)
+            const int64_t t64 = (int64_t)((d.oc + 63) / 64) * ((M + 127) / 128);
+            if (2 * t64 < cu) return v2 + V64x64x128r3;
+            const bool s1 = d.stride_h == 1 && d.stride_w == 1;
             // 3x3 over 256 channels at stride 1 with one 128 x 128 tile for most CUs: the patch-staged tile, whose stage of
             // eight k-chunks halves both the bytes through the CU's copy path and the stage boundaries (-1.4 us per
             // launch against the tile below on 256 -> 256 at 14 x 14, batch 64; falls back when the patch does not fit)
-            if (d.fh == 3 && d.fw == 3 && d.stride_h == 1 && d.stride_w == 1 && kb >= 2304 && 2 * t128 >= cu)
-                return igemm_first_v3_cfg() + V3_128x128x256r3;
-            if (d.stride_h == 1 && d.stride_w == 1) return v2 + V64x128x128r3;
+            if (d.fh == 3 && d.fw == 3 && s1 && kb >= 2304 && kb < 4608 && 2 * t128 >= cu) return igemm_first_v3_cfg() + V3_128x128x256r3;
+            // long reductions with a 128 x 128 tile for more than half of the CUs: that tile, with half the operand bytes per
+            // MAC of the 64 x 64 one (2048 -> 512 at 7 x 7, batch 128: 8.9 against 12.6 us; 3x3 512 -> 512: 17 against 24.6)
+            if (kb >= 2048 && 2 * t128 > cu && (pw || s1 || kb >= 4608)) return v2 + V128x128x128r3;
+            // pointwise: more pixels than channels per tile; with few tiles and a very long reduction the small tile with
+            // the deepest ring
+            if (pw) return v2 + (kb >= 2048 ? V64x64x128r4 : V64x128x128r3);
+            if (kb >= 4608) return v2 + V64x64x128r4;
+            if (s1) return v2 + V64x128x128r3;
             // few tiles, strided 3x3 over at most 256 channels: the first-generation tiles below
         }
     }
