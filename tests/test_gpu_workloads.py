@@ -260,5 +260,18 @@ def test_config4_chain_at_batch_128(oracle, case):
     torch.cuda.synchronize()
     assert torch.equal(dst32, ref)
     assert torch.equal(dst_plain, ref)
+    # the patch-staged tiles at full size (stride-1 cases; every usable one, with the pre-processed filter)
+    names = lib.tile_names()
+    staged = [t for t, nm in enumerate(names) if nm.startswith("v3_") and lib.tile_usable(d, t)]
+    assert (len(staged) >= 2) == (l.stride == 1), (l.name, [names[t] for t in staged])
+    for t in staged:
+        say("patch-staged tile", names[t])
+        a3, _ = ops.conv_bias_query(d, IGEMM)
+        a3.tile_cfg = t
+        pre3 = ops.conv_bias_preprocess(d, flt, a3)
+        out3 = ops.conv_bias_exec_preprocessed(d, src32, pre3, bias, z, algo=a3)
+        torch.cuda.synchronize()
+        assert torch.equal(out3, ref), names[t]
+        del out3, pre3
     del x_nchw, src32, dst32, dst_plain, y_nchw, ref, z
     torch.cuda.empty_cache()
