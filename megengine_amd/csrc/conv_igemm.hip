@@ -514,8 +514,13 @@ static bool igemm_needs_general(const ConvProblem& p) {
 constexpr uint32_t kMaxGroupLaunches = 1024;
 static bool igemm_group_by_launch(const ConvProblem& p) {
     const mi355_conv_desc& d = p.d;
-    return d.format == MI355_FMT_NCHW4 && d.group > 1 && d.group <= kMaxGroupLaunches && !p.dw4 && p.icpg % 4 == 0 &&
-           p.ocpg % 4 == 0 && !igemm_needs_general(p);
+    if (!(d.group > 1 && d.group <= kMaxGroupLaunches && !p.dw4 && p.icpg % 4 == 0)) return false;
+    if (d.format == MI355_FMT_NCHW4) return p.ocpg % 4 == 0 && !igemm_needs_general(p);
+    // planar destination: a group's output channels are a contiguous run of planes of every image (any ocpg); a
+    // full-shape bias is indexed by the whole tensor's channel count, which a group's view does not have
+    // (every group's piece of the filter starts 16-byte aligned)
+    return d.format == MI355_FMT_NCHW4_NCHW && d.dst_dtype != MI355_DT_QS32 && d.bias_mode != MI355_BIAS_FULL &&
+           ((uint64_t)p.ocpg * p.icpg * d.fh * d.fw) % 16 == 0;
 }
 static ConvProblem igemm_group_view(const ConvProblem& p) {
     ConvProblem q = p;
@@ -535,7 +540,7 @@ bool igemm_usable(const ConvProblem& p) {
     // planar destination (NCHW4_NCHW: QuantizedS8 or Float32 dst, any bias shape, any scales): dense, on two of the
     // register-staged tiles, whose planar epilogue covers all of it
     const bool planar = d.format == MI355_FMT_NCHW4_NCHW;
-    if (planar && (d.group != 1 || d.dst_dtype == MI355_DT_QS32)) return false;
+    if (planar && ((d.group != 1 && !igemm_group_by_launch(p)) || d.dst_dtype == MI355_DT_QS32)) return false;
     if (d.format != MI355_FMT_NCHW4 && d.format != MI355_FMT_NCHW32 && d.format != MI355_FMT_NCHW4_NCHW32 &&
         d.format != MI355_FMT_NCHW32_NCHW4 && !planar)
         return false;
@@ -795,10 +800,11 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
         const mi355_conv_desc& d = p.d;
         const int64_t src_g = (int64_t)p.icpg * d.ih * d.iw, dst_g = (int64_t)p.ocpg * p.oh * p.ow;
         const int64_t flt_g = (int64_t)p.ocpg * p.icpg * d.fh * d.fw;
+        const int64_t eb = d.dst_dtype == MI355_DT_F32 ? 4 : 1;  // bytes per element of dst and z (bias: 4 either way)
         for (uint32_t g = 0; g < d.group; ++g) {
             const int rc = launch_conv_igemm(st, q, cfg, cu_count, src + g * src_g, flt + g * flt_g,
-                                             bias ? bias + (int64_t)g * p.ocpg : nullptr, z ? z + g * dst_g : nullptr,
-                                             dst + g * dst_g, false);
+                                             bias ? bias + (int64_t)g * p.ocpg : nullptr, z ? z + g * dst_g * eb : nullptr,
+                                             dst + g * dst_g * eb, false);
             if (rc) return rc;
         }
         return 0;

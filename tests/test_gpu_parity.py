@@ -127,9 +127,30 @@ def test_nchw4_nchw_on_the_mfma_kernel(oracle, i):
         want = oracle.conv_bias(d, src, flt, bias, z)
         got = run_gpu(d, src, flt, bias, z, algo=IGEMM, tile=tile)
         assert np.array_equal(got, want)
-    # what stays on the generic kernel: groups and a QuantizedS32 destination
+    # what stays on the generic kernel: a QuantizedS32 destination, groups whose filter pieces are not 16-byte aligned
     assert ops.conv_bias_query(mk(NCHW4_NCHW_CASES[3], **S))[0].id == DIRECT
     assert ops.conv_bias_query(mk(c, dst_dtype=_abi.DT_QS32, scale_bias=2e-4, scale_dst=2e-4))[0].id == DIRECT
+
+
+NCHW4_NCHW_GROUP_CASES = [
+    dict(fmt="NCHW4_NCHW", n=2, ic=32, ih=12, iw=12, oc=24, fh=3, group=2, pad=1),     # ocpg = 12
+    dict(fmt="NCHW4_NCHW", n=3, ic=64, ih=9, iw=11, oc=40, fh=3, group=4, pad=1),      # icpg = 16, ocpg = 10: ragged quads
+    dict(fmt="NCHW4_NCHW", n=2, ic=48, ih=8, iw=8, oc=96, fh=1, group=3),               # pointwise groups
+]
+
+
+@pytest.mark.parametrize("i", range(len(NCHW4_NCHW_GROUP_CASES)))
+def test_nchw4_nchw_groups_one_dense_launch_per_group(oracle, i):
+    c = NCHW4_NCHW_GROUP_CASES[i]
+    assert ops.conv_bias_query(mk(c, nonline="RELU", **S))[0].id == IGEMM
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        for has_z in (False, True):
+            check_case(oracle, mk(c, nonline=nl, has_z=has_z, **S), seed=240 + i, algo=IGEMM, tag="nchw4_nchw group")
+            check_case(oracle, mk(c, nonline=nl, has_z=has_z, dst_dtype=_abi.DT_F32, scale_bias=0.0173, scale_z=0.0041),
+                       seed=250 + i, algo=IGEMM, tag="nchw4_nchw group f32")
+    check_case(oracle, mk(c, nonline="RELU", bias_mode=_abi.BIAS_NONE, **S), seed=260 + i, algo=IGEMM, tag="nchw4_nchw group no bias")
+    # a full-shape bias with groups stays on the generic kernel
+    assert ops.conv_bias_query(mk(c, bias_mode=_abi.BIAS_FULL, **S))[0].id == DIRECT
 
 
 def test_direct_s32_dst_and_full_bias(oracle, kats):
