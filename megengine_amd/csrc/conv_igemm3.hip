@@ -112,6 +112,16 @@ struct Igemm3 {
     }
 
     __device__ static __forceinline__ void run(const IgemmArgs& a) {
+        // every kernel argument the path to the first copy reads, requested in one batch of scalar loads (left alone the
+        // compiler fetches them where they are first used: several dependent round trips to the argument segment)
+        asm volatile("" ::"s"(a.src), "s"(a.flt), "s"(a.bias), "s"(a.src_bytes), "s"(a.flt_bytes), "s"(a.M), "s"(a.OC),
+                     "s"(a.tiles), "s"(a.tiles_m), "s"(a.nstages), "s"(a.KC), "s"(a.T), "s"(a.FW), "s"(a.src_sn), "s"(a.src_scb),
+                     "s"(a.flt_rstride), "s"(a.flt_kstride), "s"(a.OHW), "s"(a.OW), "s"(a.IW), "s"(a.IH), "s"(a.ph), "s"(a.pw),
+                     "s"(a.has_bias), "s"(a.NB), "s"(a.p_w), "s"(a.p_himg), "s"(a.pxp), "s"(a.pcw), "s"(a.cbs));
+        asm volatile("" ::"s"(a.div_ohw.m), "s"(a.div_ohw.s1), "s"(a.div_ohw.s2), "s"(a.div_ow.m), "s"(a.div_ow.s1),
+                     "s"(a.div_ow.s2), "s"(a.div_tiles_m.m), "s"(a.div_tiles_m.s1), "s"(a.div_tiles_m.s2), "s"(a.div_t.m),
+                     "s"(a.div_t.s1), "s"(a.div_t.s2), "s"(a.div_fw.m), "s"(a.div_fw.s1), "s"(a.div_fw.s2), "s"(a.div_pw.m),
+                     "s"(a.div_pw.s1), "s"(a.div_pw.s2), "s"(a.div_phimg.m), "s"(a.div_phimg.s1), "s"(a.div_phimg.s2));
         extern __shared__ __attribute__((aligned(16))) int8_t lds[];
         const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)lds);
         const int t = threadIdx.x;
@@ -169,7 +179,9 @@ struct Igemm3 {
             return ok ? (int)n * a.src_sn + (ih * a.IW + iw) * 32 + plane * 16 : SENT;
         };
         static_assert(PCW_MAX == 4, "four patch-copy offsets per lane");
-        const int poff0 = patch_offset(0), poff1 = patch_offset(1), poff2 = patch_offset(2), poff3 = patch_offset(3);
+        // (only the copies this launch has: the count is uniform over the launch)
+        const int poff0 = patch_offset(0), poff1 = a.pcw > 1 ? patch_offset(1) : SENT, poff2 = a.pcw > 2 ? patch_offset(2) : SENT,
+                  poff3 = a.pcw > 3 ? patch_offset(3) : SENT;
 
         // filter copies: byte offset of (row, half) of this lane, chunk added per copy
         const int rib = 16 * (lane >> 5) + (lane & 15), half = (lane >> 4) & 1;
