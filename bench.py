@@ -46,6 +46,9 @@ def main():
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch one plain 256 MiB streaming kernel (counter calibration for profilers)")
     ap.add_argument("--layers-out", default=None, help="write the per-layer table to this JSON file")
+    ap.add_argument("--batch-sweep", action="store_true",
+                    help="time ten representative ResNet-50 layers alone at batch 4..128 with their batch-64 tile, print the "
+                         "table (JSON on stdout, text on stderr) and exit: where a layer's time goes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU (the path shards by batch with no exchange); "
@@ -65,6 +68,11 @@ def main():
     log("device: %s %s, %d CUs, %.0f MHz" % (info.name.decode(), info.arch.decode(), info.compute_units,
                                              info.clock_khz / 1e3))
     torch.manual_seed(1234)
+    if args.batch_sweep:
+        side = torch.cuda.Stream()
+        torch.cuda.set_stream(side)
+        print(json.dumps(dict(batch_sweep=run_batch_sweep(torch, _abi, lib, ops, workloads))), flush=True)
+        return
     if args.extras_only:
         side = torch.cuda.Stream()
         torch.cuda.set_stream(side)
@@ -460,6 +468,41 @@ def run_extras(torch, np, _abi, lib, ops, workloads, side_iters=50):
         torch.cuda.empty_cache()
     res["config4_large_hswish"] = c4
     return res
+
+
+def run_batch_sweep(torch, _abi, lib, ops, workloads):
+    """One layer at a time, repeated as replays of a captured graph (operands warm), at batch 4 .. 128 with the tile the
+    stack uses at batch 64 forced at every size: the intercept is what a launch of that shape costs before any tile
+    count matters, the slope what a tile costs once the device is full."""
+    names = lib.tile_names()
+    igemm = lib.algo_names().index("MI355_IGEMM_MFMA_I8")
+    want = ["s1b0c1", "s1b0c2", "s1b0c3", "s2b1c2", "s3b1c1", "s3b1c2", "s3b1c3", "s4b1c1", "s4b1c2", "s4b1c3", "stem"]
+    ref = {l.name: l for l in workloads.resnet50(64)}
+    rows = []
+    for name in want:
+        l0 = ref[name]
+        plan0 = workloads.build_stack([l0], 4)
+        workloads.choose_algorithms(plan0)
+        a0 = plan0[0]["algo"]
+        del plan0
+        row = dict(layer=name, algo=lib.algo_names()[a0.id], tile=names[a0.tile_cfg] if a0.id == igemm else None, us={})
+        for n in (4, 8, 16, 32, 64, 128):
+            l = workloads.Layer(l0.name, l0.fmt, n, l0.ic, l0.ih, l0.iw, l0.oc, l0.f, stride=l0.stride, pad=l0.pad,
+                                group=l0.group, nonline=l0.nonline, z=("input:z" if l0.z else None))
+            plan = workloads.build_stack([l], 4)
+            p = plan[0]
+            a, _ = ops.conv_bias_query(p["desc"], _abi.ALGO_HEURISTIC_PREPROCESS)
+            if a0.id == igemm and lib.tile_usable(p["desc"], a0.tile_cfg):
+                a.tile_cfg = a0.tile_cfg
+            pre = ops.conv_bias_preprocess(p["desc"], p["flt"], a) if a.id == igemm else None
+            call = ops.conv_bias_bind(p["desc"], p["src"], p["flt"], p["bias"], p["z"], p["dst"], a, preprocessed=pre)
+            call()
+            torch.cuda.synchronize()
+            row["us"][str(n)] = round(min(time_launches(torch, call, iters=30) for _ in range(2)) * 1e6, 2)
+            del plan, p
+        log("%-7s %-28s " % (name, row["tile"] or row["algo"]) + " ".join("n%-3d %6.2f" % (int(k), v) for k, v in row["us"].items()))
+        rows.append(row)
+    return rows
 
 
 def cpu_baseline(np, plan):
