@@ -3,27 +3,26 @@
 //
 // With 4 channels a filter row is FW * 4 contiguous bytes in the filter AND in the image, so the
 // reduction is re-blocked as one 32-byte k-chunk per filter row: 8 taps x 4 channels, taps >= FW
-// carrying zero weights.  A workgroup
-//   * keeps the zero-padded weights of 64 output channels in LDS (written once per channel tile),
-//   * stages the input patch of an 8 x 16 output-pixel tile in LDS once (double buffered; the next
-//     tile's patch is fetched into registers while this tile is multiplied), and
+// carrying zero weights.  A workgroup (4 waves, a persistent loop over 64-channel x 8 x 16-pixel tiles)
+//   * keeps the zero-padded weights of its 64 output channels in REGISTERS, as the A fragments of all filter rows
+//     (16 bytes per lane, row and 32-channel block; loaded once per channel tile),
+//   * copies the input patch of each tile from global memory straight into LDS (no register stage), three tiles
+//     ahead of the one being multiplied, into a ring of four patch slots, and
 //   * reads every MFMA B-fragment straight from the patch: lane (pixel, half) needs taps
 //     4*half .. 4*half+3 of filter row fh = 16 contiguous patch bytes.
 // The im2col matrix is never formed and each input byte is fetched from global memory about 1.5
-// times (patch halo) instead of FH * FW / stride^2 times.
+// times (patch halo) instead of FH * FW / stride^2 times.  One barrier per tile.
 //
 // v_mfma_i32_32x32x32_i8: A = 32 output channels, B = 32 pixels (2 output rows x 16 columns of the
 // tile), accumulator layout as in conv_igemm.hip; epilogue per lane: 4 consecutive channels of one
 // pixel = one dword of the NCHW4 output.
 #include <atomic>
 
-#include "common.h"
+#include "lds_copy.h"
 
 namespace mi355 {
 namespace {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int C4_THREADS = 256;
@@ -39,7 +38,7 @@ struct C4Args {
     int8_t* dst;
     int N, IH, IW, OH, OW, OC, FH, FW, ph, pw;
     int src_sn, dst_sn, z_sn;  // batch strides in bytes
-    uint32_t dst_bytes, dst_bytes_z;  // extents of dst and z for the buffer descriptors
+    uint32_t src_bytes, dst_bytes, dst_bytes_z;  // extents for the buffer descriptors
     int has_bias;
     int tiles_w, tiles_h, tiles_m, tiles;  // tile = ((mt * N + n) * tiles_h + th) * tiles_w + tw
     FastDiv div_tw, div_th, div_n;
@@ -51,8 +50,9 @@ struct C4Geom {
     // patch row pitch in dwords (>= 15 * S + 8); S * PWD = 32 mod 64 puts the two pixel rows of a wave's block on
     // disjoint LDS banks
     static constexpr int PWD = S == 2 ? 48 : 32;
-    static constexpr int MAXROWS = (C4_TH - 1) * S + C4_MAXF;        // patch rows for the tallest filter
-    static constexpr int PREG = (MAXROWS * PWD + C4_THREADS - 1) / C4_THREADS;  // patch dwords per thread
+    static constexpr int MAXROWS = (C4_TH - 1) * S + C4_MAXF;                      // patch rows for the tallest filter
+    static constexpr int SLOT_DW = MAXROWS * PWD + 64;  // a ring slot, in dwords
+    static constexpr int NSLOT = 4;
 };
 
 struct C4Tile {
@@ -68,126 +68,181 @@ __device__ __forceinline__ C4Tile c4_decode(const C4Args& a, int tile) {
     return r;
 }
 
-template <int S>
-__device__ __forceinline__ void c4_fetch_patch(const C4Args& a, const C4Tile& tl, int rows, int t,
-                                               uint32_t (&reg)[C4Geom<S>::PREG]) {
-    using G = C4Geom<S>;
-    const uint32_t* sp = reinterpret_cast<const uint32_t*>(a.src + (int64_t)tl.n * a.src_sn);
-    const int gy0 = tl.oh0 * S - a.ph, gx0 = tl.ow0 * S - a.pw;
-#pragma unroll
-    for (int j = 0; j < G::PREG; ++j) {
-        const int idx = t + C4_THREADS * j;
-        const int row = idx / G::PWD, col = idx - row * G::PWD;
-        const int gy = gy0 + row, gx = gx0 + col;
-        const bool ok = row < rows && (unsigned)gy < (unsigned)a.IH && (unsigned)gx < (unsigned)a.IW;
-        reg[j] = ok ? sp[gy * a.IW + gx] : 0u;
+// s_waitcnt vmcnt(n) for a wave-uniform n in 0 .. 63 (the count is an immediate of the instruction)
+__device__ __forceinline__ void c4_wait_vmcnt(int n) {
+    switch (n) {
+#define C4_W1(k) case k: wait_vmcnt<k>(); break;
+#define C4_W8(k) C4_W1(k) C4_W1(k + 1) C4_W1(k + 2) C4_W1(k + 3) C4_W1(k + 4) C4_W1(k + 5) C4_W1(k + 6) C4_W1(k + 7)
+        C4_W8(0) C4_W8(8) C4_W8(16) C4_W8(24) C4_W8(32) C4_W8(40) C4_W8(48) C4_W8(56)
+#undef C4_W8
+#undef C4_W1
+        default: wait_vmcnt<63>(); break;
     }
 }
 
-template <int S>
-__device__ __forceinline__ void c4_store_patch(uint32_t* sP, int t, const uint32_t (&reg)[C4Geom<S>::PREG]) {
-    using G = C4Geom<S>;
-#pragma unroll
-    for (int j = 0; j < G::PREG; ++j) {
-        const int idx = t + C4_THREADS * j;
-        if (idx < G::MAXROWS * G::PWD) sP[idx] = reg[j];
-    }
+// Output addressing: the 8 dwords a lane stores (and the 8 residual dwords it loads) share ONE per-lane offset
+// -- its pixel and lane half -- and differ by wave-uniform plane offsets, which go into the scalar offset of the
+// buffer instruction.  C4Out holds the lane part (SENT when the pixel is outside the tensor: such an access is
+// dropped / returns 0) and what the scalar parts are made of.
+struct C4Out {
+    int voff;    // (oh * OW + ow) * 4 + lh * plane4, or SENT
+    int plane4;  // bytes of one 4-channel plane
+    int oc0;     // first channel of the tile
+    bool full;   // all 64 channels of the tile exist
+};
+
+// scalar offset of quad (i, q): batch stride * n + plane of channel oc0 + 32 * i + 8 * q (the lane half adds 4 channels)
+__device__ __forceinline__ int c4_soff(const C4Out& o, int nbase, int i, int q) {
+    return nbase + ((o.oc0 + 32 * i + 8 * q) >> 2) * o.plane4;
 }
 
-// weights of channel tile mt, re-blocked to 8 taps per filter row (zeros past FW and past OC), and its bias
-__device__ __forceinline__ void c4_load_weights(const C4Args& a, int mt, uint32_t* sW, int wrow_dw, int* sBias, int t) {
-    const uint32_t* fp = reinterpret_cast<const uint32_t*>(a.flt);
-    const int per_oc = a.FH * 8;
-    for (int idx = t; idx < C4_BM * per_oc; idx += C4_THREADS) {
-        const int oc = idx / per_oc, rem = idx - oc * per_oc;
-        const int fh = rem >> 3, tap = rem & 7;
-        const int goc = mt * C4_BM + oc;
-        uint32_t v = 0u;
-        if (goc < a.OC && tap < a.FW) v = fp[(goc * a.FH + fh) * a.FW + tap];
-        sW[oc * wrow_dw + fh * 8 + tap] = v;
-    }
-    if (t < C4_BM) {
-        const int goc = mt * C4_BM + t;
-        sBias[t] = (a.has_bias && goc < a.OC) ? a.bias[goc] : 0;
-    }
+// per-lane offset of quad (i, q) in a channel tile that reaches past OC
+__device__ __forceinline__ int c4_voff(const C4Out& o, int OC, int lh, int i, int q) {
+    return (o.full || o.oc0 + 32 * i + 8 * q + 4 * lh < OC) ? o.voff : SENT;
 }
 
-// dst / z byte offsets of this lane's 8 output dwords (SENT where the pixel or the channel quad is outside the tensor:
-// a buffer access at that offset is dropped / returns 0, so neither loads nor stores need a branch)
-__device__ __forceinline__ void c4_offsets(const C4Args& a, const C4Tile& tl, int oh, int ow, int lh, int sn, int (&off)[2][4]) {
-    const bool pok = oh < a.OH && ow < a.OW;
-    const int plane4 = a.OH * a.OW * 4;
-    const int base = tl.n * sn + (oh * a.OW + ow) * 4;
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int oc4 = tl.mt * C4_BM + i * 32 + 8 * q + 4 * lh;
-            off[i][q] = (pok && oc4 < a.OC) ? base + (oc4 >> 2) * plane4 : (int)0x80000000;
-        }
-}
+constexpr int C4_VMCNT0 = 0x0f70;  // s_waitcnt vmcnt(0) with the other counters at their maxima
+constexpr int C4_STORES = 8;  // vector-memory stores of one epilogue, per wave
 
 template <int NL, bool HZ>
 __device__ __forceinline__ void c4_epilogue(const C4Args& a, const v16i (&acc)[2], const uint32_t (&zr)[2][4],
-                                            const int (&off)[2][4], __amdgpu_buffer_rsrc_t rs_dst) {
+                                            const C4Out& out, int nbase, int lh, __amdgpu_buffer_rsrc_t rs_dst) {
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const v16i& c = acc[i];
             const uint32_t o = requant4_fast<NL, HZ>(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], zr[i][q], a.epi);
-            __builtin_amdgcn_raw_buffer_store_b32(o, rs_dst, off[i][q], 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(o, rs_dst, c4_voff(out, a.OC, lh, i, q), c4_soff(out, nbase, i, q), 0);
         }
 }
 
-template <int S>
-__global__ __launch_bounds__(C4_THREADS, 3) void c4_kernel(C4Args a) {
+// HZ: the launch has a residual (its registers exist only in that instantiation); FHT: the number of filter rows when it
+// is 3 or 7 (no branches between the MFMAs), 0 = any number up to 8
+template <int S, bool HZ, int FHT>
+__global__ __launch_bounds__(C4_THREADS, FHT ? 3 : 2) void c4_kernel(C4Args a) {
     using G = C4Geom<S>;
+    __shared__ __attribute__((aligned(16))) uint32_t sP[G::NSLOT * G::SLOT_DW];
     __shared__ __attribute__((aligned(16))) uint32_t sW[C4_BM * (C4_MAXF * 8 + 4)];
-    __shared__ __attribute__((aligned(16))) uint32_t sP[2][G::MAXROWS * G::PWD];
-    __shared__ int sBias[C4_BM];
+    __shared__ __attribute__((aligned(16))) int sBias[C4_BM];
 
     const int t = threadIdx.x;
-    const int lane = t & 63, w = t >> 6;
+    const int lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
     const int r = l32 >> 4, c = l32 & 15;  // pixel of this lane inside the wave's 2 x 16 block
-    const int wrow_dw = a.FH * 8 + 4;      // 16 bytes of padding per weight row: conflict-free 128-bit reads
-    const int rows = (C4_TH - 1) * S + a.FH;
+    const int FH = FHT ? FHT : a.FH;
+    const int rows = (C4_TH - 1) * S + FH;
 
-    const __amdgpu_buffer_rsrc_t rs_dst = __builtin_amdgcn_make_buffer_rsrc(a.dst, 0, a.dst_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rs_z =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.z), 0, a.epi.has_z ? a.dst_bytes_z : 0, 0x00020000);
+    const int first = blockIdx.x, step = gridDim.x;
+    if (first >= a.tiles) return;
+    const int count = (a.tiles - 1 - first) / step + 1;  // tiles of this workgroup
 
-    int tile = blockIdx.x;
-    if (tile >= a.tiles) return;
-    C4Tile tl = c4_decode(a, tile);
-    uint32_t preg[G::PREG];
-    c4_fetch_patch<S>(a, tl, rows, t, preg);
-    c4_load_weights(a, tl.mt, sW, wrow_dw, sBias, t);
-    c4_store_patch<S>(sP[0], t, preg);
-    __syncthreads();
+    const uint32_t lds_p = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)sP);
+    const v4i rs_src = uniform_rsrc(a.src, a.src_bytes);
+    const __amdgpu_buffer_rsrc_t rs_dst = make_rsrc(a.dst, a.dst_bytes);
+    const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(a.z, HZ ? a.dst_bytes_z : 0);
 
-    int buf = 0;
-    while (true) {
-        const int next = tile + gridDim.x;
-        const bool has_next = next < a.tiles;
-        C4Tile tn = tl;
-        if (has_next) {
-            tn = c4_decode(a, next);
-            c4_fetch_patch<S>(a, tn, rows, t, preg);  // in flight during the MFMAs and the epilogue
+    // The patch of tile k (k-th of this workgroup) goes to ring slot k & 3, one patch row per copy: lane l < PWD holds
+    // column l (the other lanes are masked off and write nothing), wave w copies rows w, w + 4, ...  The row part of the
+    // address is wave-uniform and travels in the scalar offset; columns outside the image and rows outside the image are
+    // zero-filled by the copy itself (out-of-range lane offset).  Returns the number of copies this wave issued.
+    const int ncopy = w < rows ? (rows - w + 3) >> 2 : 0;
+    auto copy_patch = [&](int k) __attribute__((always_inline)) -> int {
+        const C4Tile tt = c4_decode(a, first + k * step);
+        const int gy0 = tt.oh0 * S - a.ph, gx = tt.ow0 * S - a.pw + lane;
+        const int vcol = (unsigned)gx < (unsigned)a.IW ? gx * 4 : SENT;
+        const int base = tt.n * a.src_sn;
+        const uint32_t dst = lds_p + (uint32_t)((k & (G::NSLOT - 1)) * G::SLOT_DW * 4);
+        if (lane < G::PWD) {
+            for (int row = w; row < rows; row += 4) {
+                const int gy = gy0 + row;
+                const bool ok = (unsigned)gy < (unsigned)a.IH;
+                lds_copy_row64x4(dst + (uint32_t)(row * G::PWD * 4), ok ? vcol : SENT, ok ? base + gy * a.IW * 4 : 0, rs_src);
+            }
         }
+        return ncopy;
+    };
+
+    // A fragments of every filter row: lane (l32, lh) holds taps 4 * lh .. 4 * lh + 3 of channel i * 32 + l32, zeros for
+    // taps >= FW and channels >= OC.  The filter is read once per channel tile with consecutive threads on consecutive
+    // dwords, re-blocked in LDS to 8 taps per row (16 bytes of padding per channel: conflict-free 128-bit reads), and
+    // from there each lane takes its fragments.
+    v4i wr[C4_MAXF][2];
+    const int wrow_dw = FH * 8 + 4;
+    auto stage_weights = [&](int mt) __attribute__((always_inline)) {
+        const uint32_t* fp = reinterpret_cast<const uint32_t*>(a.flt);
+        const int per_oc = FH * 8, total = C4_BM * per_oc;
+        // thread indices through an opaque copy: nothing of this rarely run block is kept in registers across the tile loop
+        int tid = t;
+        asm volatile("" : "+v"(tid));
+        constexpr int HALF = C4_BM * C4_MAXF * 8 / C4_THREADS / 2;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            uint32_t v[HALF];
+#pragma unroll
+            for (int j = 0; j < HALF; ++j) {  // a batch of loads before the first LDS write
+                const int idx = tid + C4_THREADS * (h * HALF + j);
+                const int oc = idx / per_oc, rem = idx - oc * per_oc;
+                const int fh = rem >> 3, tap = rem & 7;
+                const int goc = mt * C4_BM + oc;
+                v[j] = (idx < total && goc < a.OC && tap < a.FW) ? fp[(goc * FH + fh) * a.FW + tap] : 0u;
+            }
+#pragma unroll
+            for (int j = 0; j < HALF; ++j) {
+                const int idx = tid + C4_THREADS * (h * HALF + j);
+                const int oc = idx / per_oc, rem = idx - oc * per_oc;
+                if (idx < total) sW[oc * wrow_dw + rem] = v[j];
+            }
+        }
+    };
+    auto read_weights = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int fh = 0; fh < C4_MAXF; ++fh) {
+            if (fh < FH) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i) wr[fh][i] = *reinterpret_cast<const v4i*>(sW + (i * 32 + l32) * wrow_dw + fh * 8 + lh * 4);
+            }
+        }
+    };
+    auto load_bias = [&](int mt) __attribute__((always_inline)) {
+        if (t < C4_BM) {
+            const int goc = mt * C4_BM + t;
+            sBias[t] = (a.has_bias && goc < a.OC) ? a.bias[goc] : 0;
+        }
+    };
+
+    // Vector-memory operations complete in order, so "the patch of tile k has landed" is "at most as many operations
+    // outstanding as were issued after its copies".  issued = operations issued so far that are counted (the copies and
+    // the epilogue's stores; loads the compiler issues are left out, which only makes a wait stricter); mk1 / mk2 / mk3 =
+    // that count right after the copies of the next / second-next / third-next tile.
+    int issued = copy_patch(0);
+    int mk1 = issued, mk2 = issued, mk3 = issued;
+    if (count > 1) { issued += copy_patch(1); mk1 = issued; }
+    if (count > 2) { issued += copy_patch(2); mk2 = issued; }
+    C4Tile tl = c4_decode(a, first);
+    stage_weights(tl.mt);
+    load_bias(tl.mt);
+    __builtin_amdgcn_s_waitcnt(C4_VMCNT0);  // the first patches have landed (this wave's copies; the barrier covers the rest)
+    __syncthreads();
+    read_weights();
+
+    for (int k = 0; k < count; ++k) {
+        if (k + 3 < count) { issued += copy_patch(k + 3); mk3 = issued; }
         const int oh = tl.oh0 + 2 * w + r, ow = tl.ow0 + c;
+        C4Out out;
+        out.plane4 = a.OH * a.OW * 4;
+        out.voff = (oh < a.OH && ow < a.OW) ? (oh * a.OW + ow) * 4 + lh * out.plane4 : SENT;
+        out.oc0 = tl.mt * C4_BM;
+        out.full = out.oc0 + C4_BM <= a.OC;
         // residual of this lane's pixel, requested before the MFMAs
-        int doff[2][4];
-        c4_offsets(a, tl, oh, ow, lh, a.dst_sn, doff);
         uint32_t zr[2][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
-        if (a.epi.has_z) {
-            int zoff[2][4];
-            c4_offsets(a, tl, oh, ow, lh, a.z_sn, zoff);
+        if constexpr (HZ) {
+            const int zbase = tl.n * a.z_sn;
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) zr[i][q] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_z, zoff[i][q], 0, 0);
+                for (int q = 0; q < 4; ++q)
+                    zr[i][q] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_z, c4_voff(out, a.OC, lh, i, q), c4_soff(out, zbase, i, q), 0);
         }
 
         v16i acc[2];
@@ -198,68 +253,64 @@ __global__ __launch_bounds__(C4_THREADS, 3) void c4_kernel(C4Args a) {
                 const v4i b = *reinterpret_cast<const v4i*>(sBias + i * 32 + 8 * q + 4 * lh);
                 acc[i][4 * q + 0] = b[0]; acc[i][4 * q + 1] = b[1]; acc[i][4 * q + 2] = b[2]; acc[i][4 * q + 3] = b[3];
             }
-        const uint32_t* pb = sP[buf] + ((2 * w + r) * S) * G::PWD + c * S + 4 * lh;
-        const uint32_t* wa = sW + l32 * wrow_dw + lh * 4;
-        // filter rows two at a time: the fragment reads of the next row are in flight while this row multiplies
-        struct Frag {
-            v4i b, a0, a1;
-        };
-        auto frags = [&](int fh, Frag& f) __attribute__((always_inline)) {
+        const uint32_t* pb = sP + (k & (G::NSLOT - 1)) * G::SLOT_DW + ((2 * w + r) * S) * G::PWD + c * S + 4 * lh;
+        auto frag_b = [&](int fh) __attribute__((always_inline)) -> v4i {
             const uint32_t* p = pb + fh * G::PWD;
+            v4i b;
             if (S == 2) {  // c * 2 + 4 * lh is even: 8-byte aligned
                 const u32x2 lo = *reinterpret_cast<const u32x2*>(p), hi = *reinterpret_cast<const u32x2*>(p + 2);
-                f.b[0] = (int)lo[0]; f.b[1] = (int)lo[1]; f.b[2] = (int)hi[0]; f.b[3] = (int)hi[1];
+                b[0] = (int)lo[0]; b[1] = (int)lo[1]; b[2] = (int)hi[0]; b[3] = (int)hi[1];
             } else {
-                f.b[0] = (int)p[0]; f.b[1] = (int)p[1]; f.b[2] = (int)p[2]; f.b[3] = (int)p[3];
+                b[0] = (int)p[0]; b[1] = (int)p[1]; b[2] = (int)p[2]; b[3] = (int)p[3];
             }
-            f.a0 = *reinterpret_cast<const v4i*>(wa + fh * 8);
-            f.a1 = *reinterpret_cast<const v4i*>(wa + 32 * wrow_dw + fh * 8);
+            return b;
         };
-        auto mfmas = [&](const Frag& f) __attribute__((always_inline)) {
-            acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a0, f.b, acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a1, f.b, acc[1], 0, 0, 0);
-        };
-        Frag f0, f1;
-        frags(0, f0);
-        for (int fh = 0; fh < a.FH; fh += 2) {
-            const bool odd = fh + 1 < a.FH;
-            if (odd) frags(fh + 1, f1);
-            mfmas(f0);
-            if (odd) {
-                if (fh + 2 < a.FH) frags(fh + 2, f0);
-                mfmas(f1);
+        // the B fragment of the next filter row is in flight while this row multiplies
+        v4i fb[2];
+        fb[0] = frag_b(0);
+#pragma unroll
+        for (int fh = 0; fh < C4_MAXF; ++fh) {
+            if (fh < FH) {
+                if (fh + 1 < C4_MAXF && fh + 1 < FH) fb[(fh + 1) & 1] = frag_b(fh + 1);
+                acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wr[fh][0], fb[fh & 1], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wr[fh][1], fb[fh & 1], acc[1], 0, 0, 0);
             }
         }
 
-        // The next tile's patch goes into LDS BEFORE this tile's stores are issued: the wait for its loads then counts no
-        // store (vector-memory operations are counted together and retire in order; behind the epilogue the same wait
-        // stood for fifteen of this tile's sixteen stores, i.e. every tile paid the latency of its own stores).
-        if (has_next) {
-            if (tn.mt != tl.mt) {
-                __syncthreads();  // every wave is done with the old weights
-                c4_load_weights(a, tn.mt, sW, wrow_dw, sBias, t);
-            }
-            c4_store_patch<S>(sP[buf ^ 1], t, preg);
+        // One barrier per tile, before the epilogue: the next tile's patch has landed (this wave's part; the barrier
+        // covers the other waves') and every wave is done with this tile's slot, which the copies issued at the top of
+        // the next iteration overwrite.
+        C4Tile tn = tl;
+        if (k + 1 < count) {
+            tn = c4_decode(a, first + (k + 1) * step);
+            const int after = issued - mk1;
+            c4_wait_vmcnt(after > 63 ? 63 : after);
             __syncthreads();
-        }
-        if (a.epi.lin) {
-            c4_epilogue<NL_LIN, false>(a, acc, zr, doff, rs_dst);
-        } else if (a.epi.has_z) {
-            switch (a.epi.nonline) {
-                case NL_RELU: c4_epilogue<NL_RELU, true>(a, acc, zr, doff, rs_dst); break;
-                case NL_H_SWISH: c4_epilogue<NL_H_SWISH, true>(a, acc, zr, doff, rs_dst); break;
-                default: c4_epilogue<NL_IDENTITY, true>(a, acc, zr, doff, rs_dst); break;
+            if (tn.mt != tl.mt) {  // every wave has read the old bias; the old weights are dead
+                stage_weights(tn.mt);
+                load_bias(tn.mt);
+                __syncthreads();
+                read_weights();
             }
+        }
+        const int dbase = tl.n * a.dst_sn;
+        if constexpr (HZ) {
+            switch (a.epi.nonline) {
+                case NL_RELU: c4_epilogue<NL_RELU, true>(a, acc, zr, out, dbase, lh, rs_dst); break;
+                case NL_H_SWISH: c4_epilogue<NL_H_SWISH, true>(a, acc, zr, out, dbase, lh, rs_dst); break;
+                default: c4_epilogue<NL_IDENTITY, true>(a, acc, zr, out, dbase, lh, rs_dst); break;
+            }
+        } else if (a.epi.lin) {
+            c4_epilogue<NL_LIN, false>(a, acc, zr, out, dbase, lh, rs_dst);
         } else {
             switch (a.epi.nonline) {
-                case NL_RELU: c4_epilogue<NL_RELU, false>(a, acc, zr, doff, rs_dst); break;
-                case NL_H_SWISH: c4_epilogue<NL_H_SWISH, false>(a, acc, zr, doff, rs_dst); break;
-                default: c4_epilogue<NL_IDENTITY, false>(a, acc, zr, doff, rs_dst); break;
+                case NL_RELU: c4_epilogue<NL_RELU, false>(a, acc, zr, out, dbase, lh, rs_dst); break;
+                case NL_H_SWISH: c4_epilogue<NL_H_SWISH, false>(a, acc, zr, out, dbase, lh, rs_dst); break;
+                default: c4_epilogue<NL_IDENTITY, false>(a, acc, zr, out, dbase, lh, rs_dst); break;
             }
         }
-        if (!has_next) break;
-        buf ^= 1;
-        tile = next;
+        issued += C4_STORES;
+        mk1 = mk2; mk2 = mk3;
         tl = tn;
     }
 }
@@ -292,6 +343,7 @@ int launch_conv_c4(hipStream_t st, const ConvProblem& p, int cu_count, const int
     a.ph = d.pad_h; a.pw = d.pad_w;
     a.src_sn = (int)p.src_sn; a.dst_sn = (int)p.dst_sn; a.z_sn = (int)p.z_sn;
     a.has_bias = d.bias_mode == MI355_BIAS_BROADCAST_CHANNEL;
+    a.src_bytes = (uint32_t)((int64_t)(d.n - 1) * p.src_sn + (int64_t)4 * d.ih * d.iw);
     a.dst_bytes = (uint32_t)((int64_t)(d.n - 1) * p.dst_sn + (int64_t)d.oc * p.oh * p.ow);
     a.dst_bytes_z = d.has_z ? (uint32_t)((int64_t)(d.n - 1) * p.z_sn + (int64_t)d.oc * p.oh * p.ow) : 0;
     a.tiles_w = (p.ow + C4_TW - 1) / C4_TW;
@@ -304,12 +356,16 @@ int launch_conv_c4(hipStream_t st, const ConvProblem& p, int cu_count, const int
     if (cu_count <= 0) cu_count = 256;
     // persistent grid: exactly as many workgroups as are resident at once (a workgroup that had to wait for a
     // slot would start its whole share of tiles late)
-    static std::atomic<int> occ[2];  // zero-initialised; several threads may launch
-    const int si = d.stride_h == 2 ? 1 : 0;
+    using Kern = void (*)(C4Args);
+    static const Kern kerns[12] = {
+            c4_kernel<1, false, 0>, c4_kernel<1, false, 3>, c4_kernel<1, false, 7>, c4_kernel<1, true, 0>,
+            c4_kernel<1, true, 3>,  c4_kernel<1, true, 7>,  c4_kernel<2, false, 0>, c4_kernel<2, false, 3>,
+            c4_kernel<2, false, 7>, c4_kernel<2, true, 0>,  c4_kernel<2, true, 3>,  c4_kernel<2, true, 7>};
+    static std::atomic<int> occ[12];  // zero-initialised; several threads may launch
+    const int si = (d.stride_h == 2 ? 6 : 0) + (d.has_z ? 3 : 0) + (d.fh == 3 ? 1 : d.fh == 7 ? 2 : 0);
     if (!occ[si].load(std::memory_order_relaxed)) {
         int o = 0;
-        hipError_t e = si ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&o, reinterpret_cast<const void*>(c4_kernel<2>), C4_THREADS, 0)
-                          : hipOccupancyMaxActiveBlocksPerMultiprocessor(&o, reinterpret_cast<const void*>(c4_kernel<1>), C4_THREADS, 0);
+        hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&o, reinterpret_cast<const void*>(kerns[si]), C4_THREADS, 0);
         if (e != hipSuccess || o < 1) {
             (void)hipGetLastError();
             o = 1;
@@ -318,10 +374,7 @@ int launch_conv_c4(hipStream_t st, const ConvProblem& p, int cu_count, const int
     }
     int64_t grid = (int64_t)occ[si].load(std::memory_order_relaxed) * cu_count;
     if (grid > a.tiles) grid = a.tiles;
-    if (si)
-        hipLaunchKernelGGL((c4_kernel<2>), dim3((unsigned)grid), dim3(C4_THREADS), 0, st, a);
-    else
-        hipLaunchKernelGGL((c4_kernel<1>), dim3((unsigned)grid), dim3(C4_THREADS), 0, st, a);
+    hipLaunchKernelGGL(kerns[si], dim3((unsigned)grid), dim3(C4_THREADS), 0, st, a);
     return (int)hipGetLastError();
 }
 

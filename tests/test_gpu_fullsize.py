@@ -50,6 +50,11 @@ FULL_CASES = [
     ("r50_3x3s2", "NCHW32", 64, 256, 28, 256, 3, 2, 1, "RELU", False),
     ("r50_ds", "NCHW32", 64, 256, 56, 512, 1, 2, 0, "IDENTITY", False),
     ("stem", "NCHW4", 16, 4, 224, 64, 7, 2, 3, "RELU", False),             # config 2 stem (batch 16)
+    # first-layer kernel, eight tiles per workgroup (its ring of patch slots wraps twice), with a residual; and three
+    # channel tiles of a 3x3 stem, so that a workgroup reloads its weights between tiles
+    ("stem_bs64_z", "NCHW4", 64, 4, 224, 64, 7, 2, 3, "RELU", True),
+    ("stem3x3_oc160", "NCHW4", 24, 4, 112, 160, 3, 1, 1, "H_SWISH", True),
+    ("stem5x5s2_oc96", "NCHW4", 32, 4, 160, 96, 5, 2, 2, "IDENTITY", False),
     ("mbv2_expand", "NCHW4", 64, 24, 56, 144, 1, 1, 0, "RELU", False),     # config 3
     ("mbv2_project", "NCHW4", 64, 144, 56, 24, 1, 1, 0, "IDENTITY", True),
     # three / six channel tiles: successive tiles of a workgroup change channel tile, so the bias copy is rewritten
