@@ -46,6 +46,8 @@ def main():
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch one plain 256 MiB streaming kernel (counter calibration for profilers)")
     ap.add_argument("--layers-out", default=None, help="write the per-layer table to this JSON file")
+    ap.add_argument("--sweep-layers", default=None,
+                    help="comma-separated ResNet-50 layer names for --batch-sweep, or 'all' (default: ten representative ones)")
     ap.add_argument("--batch-sweep", action="store_true",
                     help="time ten representative ResNet-50 layers alone at batch 4..128 with their batch-64 tile, print the "
                          "table (JSON on stdout, text on stderr) and exit: where a layer's time goes")
@@ -71,7 +73,7 @@ def main():
     if args.batch_sweep:
         side = torch.cuda.Stream()
         torch.cuda.set_stream(side)
-        print(json.dumps(dict(batch_sweep=run_batch_sweep(torch, _abi, lib, ops, workloads))), flush=True)
+        print(json.dumps(dict(batch_sweep=run_batch_sweep(torch, _abi, lib, ops, workloads, args.sweep_layers))), flush=True)
         return
     if args.extras_only:
         side = torch.cuda.Stream()
@@ -470,7 +472,7 @@ def run_extras(torch, np, _abi, lib, ops, workloads, side_iters=50):
     return res
 
 
-def run_batch_sweep(torch, _abi, lib, ops, workloads):
+def run_batch_sweep(torch, _abi, lib, ops, workloads, layers=None):
     """One layer at a time, repeated as replays of a captured graph (operands warm), at batch 4 .. 128 with the tile the
     stack uses at batch 64 forced at every size: the intercept is what a launch of that shape costs before any tile
     count matters, the slope what a tile costs once the device is full."""
@@ -478,6 +480,10 @@ def run_batch_sweep(torch, _abi, lib, ops, workloads):
     igemm = lib.algo_names().index("MI355_IGEMM_MFMA_I8")
     want = ["s1b0c1", "s1b0c2", "s1b0c3", "s2b1c2", "s3b1c1", "s3b1c2", "s3b1c3", "s4b1c1", "s4b1c2", "s4b1c3", "stem"]
     ref = {l.name: l for l in workloads.resnet50(64)}
+    if layers == "all":
+        want = list(ref)
+    elif layers:
+        want = layers.split(",")
     rows = []
     for name in want:
         l0 = ref[name]
