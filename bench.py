@@ -43,6 +43,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only")
     ap.add_argument("--no-preprocess", action="store_true", help="exec with the filters in the reference layout only")
+    ap.add_argument("--no-memory-plan", action="store_true",
+                    help="one buffer per layer output instead of the static activation-memory plan")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch one plain 256 MiB streaming kernel (counter calibration for profilers)")
     ap.add_argument("--layers-out", default=None, help="write the per-layer table to this JSON file")
@@ -85,6 +87,9 @@ def main():
     batch = 64
     layers = workloads.resnet50(batch)
     plan = workloads.build_stack(layers, 7)
+    # activation memory laid out once by liveness, as the graph runtime above the operator does before it runs a
+    # computing sequence (--no-memory-plan: one buffer per layer output)
+    mem = None if args.no_memory_plan else workloads.plan_memory(plan)
     # algorithm choice and weight pre-processing happen once, before the timed region (exec_preprocess is the
     # reference's own hook for hoisting filter re-tiling out of exec)
     workloads.choose_algorithms(plan, weight_preprocess=not args.no_preprocess)
@@ -145,6 +150,33 @@ def main():
     log("eager %.4f ms/step, graph %s ms/step (%s)" % (eager_ms, graph_ms, graph_note))
     ms_per_step = graph_ms if graph_ms is not None else eager_ms
     launch_mode = "hipGraph replay" if graph_ms is not None else "eager"
+
+    # ---- the same stack with one buffer per layer output (what the memory plan is worth), fewer replays
+    unplanned_ms = None
+    if mem is not None and graph_ms is not None:
+        try:
+            plan2 = workloads.choose_algorithms(workloads.build_stack(layers, 7), weight_preprocess=not args.no_preprocess)
+            calls2 = workloads.bind_plan(plan2)
+            for c in calls2:
+                c()
+            torch.cuda.synchronize()
+            g2 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g2, stream=side):
+                for c in calls2:
+                    c()
+            reps2 = max(20, args.steps // 4)
+            for _ in range(3):
+                g2.replay()
+            torch.cuda.synchronize()
+            e0.record(stream)
+            for _ in range(reps2):
+                g2.replay()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            unplanned_ms = e0.elapsed_time(e1) / reps2
+            del g2, calls2, plan2
+        except Exception as e:  # a comparison figure must not lose the headline
+            log("one-buffer-per-layer stack: %r" % (e,))
     img_s = batch * 1000.0 / ms_per_step
     tot_ops = sum(l.ops for l in layers)
     tot_bytes = sum(l.bytes for l in layers)
@@ -214,9 +246,14 @@ def main():
                            workload="BASELINE configs[2]: ResNet-50 v1.5 int8 conv stack, batch 64, 224x224, "
                                     "NCHW4 stem + NCHW32, fused residual z + RELU, random per-tensor scales",
                            batch=batch, layers=nl, launch=launch_mode, graph=graph_note,
+                           activation_memory=("one buffer per layer output, %.0f MB" % (sum(p["dst"].numel() for p in plan) / 1e6)
+                                              if mem is None else
+                                              "static plan by liveness: %.0f MB for the %.0f MB of layer outputs"
+                                              % (mem["planned"] / 1e6, mem["one_buffer_per_layer"] / 1e6)),
                            weight_preprocess="%d of %d filters pre-processed once through exec_preprocess, outside the timed "
                                              "region" % (sum(p.get("pre") is not None for p in plan), nl)),
                eager_ms_per_step=round(eager_ms, 4),
+               ms_per_step_one_buffer_per_layer=None if unplanned_ms is None else round(unplanned_ms, 4),
                tops=round(tot_ops / (ms_per_step * 1e-3) / 1e12, 1),
                pct_int8_peak=round(100 * tot_ops / (ms_per_step * 1e-3) / INT8_PEAK_OPS, 2),
                roofline=roofline)
@@ -233,7 +270,7 @@ def main():
         out["other_configs"] = extras
 
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(np, plan)
+        out["cpu_baseline"] = cpu_baseline(np, plan, workloads.snapshot_run(plan, calls, min(batch, 16)))
 
     if args.layers_out:
         with open(args.layers_out, "w") as f:
@@ -511,11 +548,12 @@ def run_batch_sweep(torch, _abi, lib, ops, workloads, layers=None):
     return rows
 
 
-def cpu_baseline(np, plan):
+def cpu_baseline(np, plan, snaps):
     """The CPU parity checker (a port of the reference's naive ConvBias, OpenMP over output rows) on a bounded sample
     of the SAME workload: the first b images of the very tensors the GPU plan ran on (same weights, biases, residuals
     and scales, layer by layer), b chosen so that the whole leg is 10-30 s of CPU work on this host; scaled to images
-    per second.  Its outputs are compared with the first b images of the GPU's outputs."""
+    per second.  Its outputs are compared with the first b images of the GPU's outputs.  snaps = per layer the host
+    copies (source, residual, output) of the first images, taken right after the layer's launch."""
     import copy
 
     from oracle import oracle
@@ -527,15 +565,15 @@ def cpu_baseline(np, plan):
 
     def run(batch, budget):
         t_tot, macs, done, bad = 0.0, 0, 0, 0
-        for p in plan:
+        for p, (h_src, h_z, h_dst) in zip(plan, snaps):
             d = copy.copy(p["desc"])
             d.n = batch
-            host = [None if t is None else t[:batch].cpu().numpy() for t in (p["src"], p["z"])]
+            host = [None if t is None else np.ascontiguousarray(t[:batch]) for t in (h_src, h_z)]
             flt, bias = p["flt"].cpu().numpy(), p["bias"].cpu().numpy()
             t0 = time.perf_counter()
             out = oracle.conv_bias(d, host[0], flt, bias, host[1])
             t_tot += time.perf_counter() - t0
-            bad += int((out != p["dst"][:batch].cpu().numpy()).sum())
+            bad += int((out != h_dst[:batch]).sum())
             macs += p["layer"].ops // 2 // p["layer"].n * batch
             done += 1
             if t_tot > budget:
@@ -544,7 +582,7 @@ def cpu_baseline(np, plan):
 
     t1, m1, _, _ = run(1, 10.0)                 # probe: one image
     est = t1 * total_macs / max(m1, 1)
-    batch = int(max(1, min(plan[0]["layer"].n, round(15.0 / max(est, 1e-3)))))
+    batch = int(max(1, min(len(snaps[0][0]), round(15.0 / max(est, 1e-3)))))
     t_tot, macs, done, bad = run(batch, 30.0)
     img_s = (macs / total_macs) / t_tot if t_tot > 0 else 0.0
     return dict(value=round(img_s, 3), unit="img/s", cores=cores, kind="port",

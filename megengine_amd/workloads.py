@@ -156,6 +156,70 @@ def build_stack(layers, seed):
     return plan
 
 
+def first_fit_offsets(tensors, granule=4096):
+    """Offsets for tensors given as (bytes, index of the writing step, index of the last reading step), in writing
+    order: each goes to the lowest granule-aligned offset where it overlaps no tensor that is live at its writing step
+    (written earlier and read at that step or later).  Returns (offsets, arena bytes)."""
+    live, offsets, top = [], [], 0
+    for size, i, last_read in tensors:
+        live = [r for r in live if r[2] >= i]
+        size = (size + granule - 1) // granule * granule
+        off = 0
+        for o, sz, _ in sorted(live):
+            if off + size <= o:
+                break
+            off = max(off, o + sz)
+        live.append((off, size, max(last_read, i)))
+        offsets.append(off)
+        top = max(top, off + size)
+    return offsets, top
+
+
+def plan_memory(plan):
+    """Static activation-memory plan for a layer list of build_stack, as a graph runtime lays out the variables of a
+    computing sequence before it runs (the reference: StaticMemAlloc, src/core/impl/graph/var_node_mem_mgr/
+    static_mem_alloc.h:18-40, intervals = first write to last read): every layer output becomes a range of ONE arena
+    that no LIVE tensor occupies -- live = written and still to be read, as a source or a residual, by this layer or a
+    later one -- at the lowest address where it fits (address-ordered first fit, 4 KiB granules), instead of a buffer
+    of its own.  Graph inputs (seeded tensors) keep theirs.  A layer never writes memory it reads.  Rewires src / z / dst
+    of the plan in place; returns the bytes of activation memory before and after."""
+    import torch
+
+    last = {}
+    for i, p in enumerate(plan):
+        for t in (p["src"], p["z"]):
+            if t is not None:
+                last[t.data_ptr()] = i
+    # an output nobody reads is dead after its own layer
+    offsets, top = first_fit_offsets([(p["dst"].numel(), i, last.get(p["dst"].data_ptr(), i)) for i, p in enumerate(plan)])
+    before = sum(p["dst"].numel() for p in plan)
+    arena = torch.empty(top, dtype=plan[0]["dst"].dtype, device=plan[0]["dst"].device)
+    remap = {}    # data_ptr of the original output -> its range of the arena
+    for p, off in zip(plan, offsets):
+        for k in ("src", "z"):
+            t = p[k]
+            if t is not None and t.data_ptr() in remap:
+                p[k] = remap[t.data_ptr()].view(t.shape)
+        old = p["dst"]
+        remap[old.data_ptr()] = arena[off:off + old.numel()]
+        p["dst"] = remap[old.data_ptr()].view(old.shape)
+    return dict(one_buffer_per_layer=before, planned=top)
+
+
+def snapshot_run(plan, calls, images):
+    """Runs the launches of a plan once, in order, and copies the first `images` images of every layer's source,
+    residual and output to the host right after its launch: with planned activation memory a buffer holds a layer's
+    output only until its last reader has run."""
+    import torch
+
+    snaps = []
+    for p, c in zip(plan, calls):
+        c()
+        torch.cuda.synchronize()
+        snaps.append(tuple(None if t is None else t[:images].cpu().numpy() for t in (p["src"], p["z"], p["dst"])))
+    return snaps
+
+
 def run_calibrated(plan, seed, weight_preprocess=True):
     """Runs a plan of build_stack layer by layer with scales and biases re-drawn so that most outputs are LIVE values,
     strictly inside the int8 range, instead of the clamped bytes that per-tensor scales drawn at random give after a

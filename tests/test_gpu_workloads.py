@@ -97,6 +97,33 @@ def test_config2_resnet50_stack_on_live_values(oracle, resnet_live_plan, part):
         check_layer(oracle, plan[i], seed=5000 + i)
 
 
+def test_static_memory_plan_changes_no_output():
+    """The benchmark lays the activations of the stack out by liveness (workloads.plan_memory).  The planned stack
+    must produce, layer by layer, the bytes of the stack with one buffer per output; no layer may write a buffer it
+    reads; and a buffer may only be reused after its last reader."""
+    def build():
+        torch.manual_seed(77)
+        return workloads.choose_algorithms(workloads.build_stack(workloads.resnet50(4), 7))
+    ref = build()
+    for c in workloads.bind_plan(ref):
+        c()
+    torch.cuda.synchronize()
+    plan = build()
+    mem = workloads.plan_memory(plan)
+    assert mem["planned"] < 0.35 * mem["one_buffer_per_layer"]
+    for p in plan:
+        w = p["dst"].data_ptr()
+        assert w != p["src"].data_ptr() and (p["z"] is None or w != p["z"].data_ptr()), p["layer"].name
+    snaps = workloads.snapshot_run(plan, workloads.bind_plan(plan), 4)
+    for p, r, (h_src, h_z, h_dst) in zip(plan, ref, snaps):
+        assert np.array_equal(h_src, r["src"].cpu().numpy()), "source of " + p["layer"].name
+        assert r["z"] is None or np.array_equal(h_z, r["z"].cpu().numpy()), "residual of " + p["layer"].name
+        assert np.array_equal(h_dst, r["dst"].cpu().numpy()), "output of " + p["layer"].name
+    # and a second step over the same buffers (what a replayed graph does) ends on the same bytes
+    snaps2 = workloads.snapshot_run(plan, workloads.bind_plan(plan), 4)
+    assert all(np.array_equal(a[2], b[2]) for a, b in zip(snaps, snaps2))
+
+
 def test_config2_uses_preprocessed_filters(resnet_plan):
     n = sum(p.get("pre") is not None for p in resnet_plan)
     say(n, "of 53 layers run with a pre-processed filter")
