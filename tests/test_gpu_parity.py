@@ -709,6 +709,32 @@ def test_first_layer_kernel(oracle, i):
     check_case(oracle, d, seed=600 + i, tag="c4-%d-strided" % i)
 
 
+def test_first_layer_kernel_on_random_shapes(oracle):
+    """Thirty seeded random first-layer problems: every filter height and width up to 8, both strides, paddings up to
+    the filter size, odd image sizes, channel counts that end inside a channel tile, every activation, with and without
+    a residual -- against the checker, with scales that keep most outputs inside the int8 range."""
+    rng = np.random.RandomState(2024)
+    ran = 0
+    for i in range(30):
+        n = int(rng.randint(1, 4))
+        fh, fw = int(rng.randint(1, 9)), int(rng.randint(1, 9))
+        stride = int(rng.choice([1, 2]))
+        pad_h, pad_w = int(rng.randint(0, fh + 1)), int(rng.randint(0, fw + 1))
+        ih, iw = int(rng.randint(max(fh - 2 * pad_h, 1), 45)), int(rng.randint(max(fw - 2 * pad_w, 1), 45))
+        oc = 4 * int(rng.randint(1, 50))
+        nl = ["IDENTITY", "RELU", "H_SWISH"][int(rng.randint(0, 3))]
+        has_z = bool(rng.randint(0, 2))
+        k = 4 * fh * fw
+        d = _abi.make_conv_desc("NCHW4", n, 4, ih, iw, oc, fh, fw, stride=stride, pad=(pad_h, pad_w), nonline=nl, has_z=has_z,
+                                scale_bias=2e-4, scale_z=0.02, scale_dst=float(np.float32(2e-4 * 73.9 * 73.3 * k ** 0.5 / 25.0)))
+        a, _ = ops.conv_bias_query(d)
+        if a.id != C4:
+            continue
+        check_case(oracle, d, seed=900 + i, tag="c4-random-%d" % i)
+        ran += 1
+    assert ran >= 25
+
+
 def test_profile_entry_point(oracle):
     """the timed trial run of a fast-run chooser: times one algorithm, leaves the right result in dst"""
     d = _abi.make_conv_desc("NCHW32", 8, 128, 14, 14, 128, 3, pad=1, nonline="RELU", **S)
