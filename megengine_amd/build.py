@@ -18,7 +18,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmi355_convbias.so")
-SOURCES = ["capi.hip", "conv_direct.hip", "conv_igemm.hip", "conv_igemm_dma.hip", "conv_igemm2.hip", "conv_igemm3.hip", "conv_pw4.hip", "conv_c4.hip", "conv_dw.hip", "conv_nchw.hip", "relayout.hip", "requant.hip", "elemwise_q.hip", "pooling.hip"]
+SOURCES = ["capi.hip", "conv_direct.hip", "conv_igemm.hip", "conv_igemm_dma.hip", "conv_igemm2.hip", "conv_igemm3.hip", "conv_igemm4.hip", "conv_pw4.hip", "conv_c4.hip", "conv_dw.hip", "conv_nchw.hip", "relayout.hip", "requant.hip", "elemwise_q.hip", "pooling.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt", "-fno-fast-math",

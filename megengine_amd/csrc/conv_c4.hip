@@ -102,7 +102,6 @@ __device__ __forceinline__ int c4_voff(const C4Out& o, int OC, int lh, int i, in
 }
 
 constexpr int C4_VMCNT0 = 0x0f70;  // s_waitcnt vmcnt(0) with the other counters at their maxima
-constexpr int C4_STORES = 8;  // vector-memory stores of one epilogue, per wave
 
 template <int NL, bool HZ>
 __device__ __forceinline__ void c4_epilogue(const C4Args& a, const v16i (&acc)[2], const uint32_t (&zr)[2][4],
@@ -211,10 +210,11 @@ __global__ __launch_bounds__(C4_THREADS, FHT ? 3 : 2) void c4_kernel(C4Args a) {
         }
     };
 
-    // Vector-memory operations complete in order, so "the patch of tile k has landed" is "at most as many operations
-    // outstanding as were issued after its copies".  issued = operations issued so far that are counted (the copies and
-    // the epilogue's stores; loads the compiler issues are left out, which only makes a wait stricter); mk1 / mk2 / mk3 =
-    // that count right after the copies of the next / second-next / third-next tile.
+    // Vector-memory loads complete in order, so "the patch of tile k has landed" is "at most as many operations outstanding
+    // as COPIES were issued after its copies": were one of its copies outstanding, so would be every younger copy.  Only
+    // the copies are counted (issued = copies issued so far; mk1 / mk2 / mk3 = that count right after the copies of the
+    // next / second-next / third-next tile): loads and stores the compiler issues in between only make the wait
+    // stricter, whatever the order in which stores complete relative to loads.
     int issued = copy_patch(0);
     int mk1 = issued, mk2 = issued, mk3 = issued;
     if (count > 1) { issued += copy_patch(1); mk1 = issued; }
@@ -309,7 +309,6 @@ __global__ __launch_bounds__(C4_THREADS, FHT ? 3 : 2) void c4_kernel(C4Args a) {
                 default: c4_epilogue<NL_IDENTITY, false>(a, acc, zr, out, dbase, lh, rs_dst); break;
             }
         }
-        issued += C4_STORES;
         mk1 = mk2; mk2 = mk3;
         tl = tn;
     }

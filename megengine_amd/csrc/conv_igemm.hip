@@ -482,8 +482,9 @@ int launch_fmt(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
 
 }  // namespace
 
-// tile_cfg numbering: register-staged tiles, LDS-direct tiles, second-generation tiles, patch-staged tiles
-int igemm_num_cfgs() { return kNumCfgs + igemm_dma_num_cfgs() + igemm2_num_cfgs() + igemm3_num_cfgs(); }
+// tile_cfg numbering: register-staged tiles, LDS-direct tiles, second-generation tiles, patch-staged tiles, weight-resident
+// tiles
+int igemm_num_cfgs() { return kNumCfgs + igemm_dma_num_cfgs() + igemm2_num_cfgs() + igemm3_num_cfgs() + igemm4_num_cfgs(); }
 int igemm_first_v2_cfg() { return kNumCfgs + igemm_dma_num_cfgs(); }
 // planar destination (NCHW4_NCHW): two of the register-staged tiles
 static int launch_planar(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
@@ -495,11 +496,13 @@ static int launch_planar(hipStream_t st, IgemmArgs& a, int cfg, int cu) {
 }
 
 static int igemm_first_v3_cfg() { return igemm_first_v2_cfg() + igemm2_num_cfgs(); }
+static int igemm_first_v4_cfg() { return igemm_first_v3_cfg() + igemm3_num_cfgs(); }
 const char* igemm_cfg_name(int cfg) {
     if (cfg >= 0 && cfg < kNumCfgs) return kCfgs[cfg].name;
     if (cfg < igemm_first_v2_cfg()) return igemm_dma_cfg_name(cfg - kNumCfgs);
     if (cfg < igemm_first_v3_cfg()) return igemm2_cfg_name(cfg - igemm_first_v2_cfg());
-    return igemm3_cfg_name(cfg - igemm_first_v3_cfg());
+    if (cfg < igemm_first_v4_cfg()) return igemm3_cfg_name(cfg - igemm_first_v3_cfg());
+    return igemm4_cfg_name(cfg - igemm_first_v4_cfg());
 }
 
 static bool igemm_needs_general(const ConvProblem& p) {
@@ -572,6 +575,15 @@ static int pick_cfg_by_shape(const ConvProblem& p, int cu_count, bool will_prepr
         // planar destination: 128 x 128 tiles once they fill the device, else 64 x 64
         const int64_t t128 = (int64_t)((d.oc + 127) / 128) * (((int64_t)d.n * p.oh * p.ow + 127) / 128);
         return d.oc > 64 && t128 >= (cu_count > 0 ? cu_count : 256) ? 0 : 3;
+    }
+    if (p.pin == 32 && p.pout == 32 && d.group == 1 && !igemm_needs_general(p) && d.fh == 3 && d.fw == 3 &&
+        d.stride_h == 1 && d.stride_w == 1 && d.pad_h == 1 && d.pad_w == 1 && (d.ic == 32 || d.ic == 64)) {
+        // 3x3 over 32 or 64 channels with five and more 64 x 128 tiles for each of the two workgroups of a CU: the
+        // weight-resident tile, whose workgroups load the filter once (64 -> 64 at 56 x 56, batch 128: 24.4 against 26.7 us
+        // on the second-generation tile; at batch 64, three tiles per workgroup, its longer prologue loses: 15.7 against 14.8)
+        const int64_t t = (int64_t)((d.oc + 63) / 64) * d.n * ((p.oh * p.ow + 127) / 128);
+        const int v4 = igemm_first_v4_cfg();
+        if (t >= 10 * (int64_t)(cu_count > 0 ? cu_count : 256) && igemm_resolve_cfg(p, v4) == v4) return v4;
     }
     if (will_preprocess && p.pin == 32 && p.pout == 32 && d.group == 1 && !igemm_needs_general(p)) {
         // The caller re-tiles the filter for the chosen algorithm (weight pre-processing): the second-generation tiles
@@ -677,7 +689,8 @@ static int pick_cfg_by_shape(const ConvProblem& p, int cu_count, bool will_prepr
 }
 
 size_t igemm_preprocessed_bytes(const ConvProblem& p, int cfg) {
-    if (p.pin != 32 || cfg < igemm_first_v2_cfg() || cfg >= igemm_num_cfgs()) return 0;
+    // the weight-resident tiles read the reference layout (once per workgroup: nothing to gain from re-tiling)
+    if (p.pin != 32 || cfg < igemm_first_v2_cfg() || cfg >= igemm_first_v4_cfg()) return 0;
     return igemm2_preprocessed_bytes((int)p.d.oc, (int)(p.icpg * p.d.fh * p.d.fw));
 }
 
@@ -752,6 +765,11 @@ int igemm_resolve_cfg(const ConvProblem& p, int cfg) {
     const int first_v2 = igemm_first_v2_cfg();
     // group convolutions and the general epilogue exist on the second-generation tiles only
     if ((d.group != 1 || a.general) && cfg < first_v2) cfg = first_v2 + (p.ocpg <= 64 ? 3 : 0);
+    if (cfg >= igemm_first_v4_cfg()) {
+        // the weight-resident tiles: 3x3 / stride 1 / pad 1 over 32 or 64 channels; otherwise as above
+        if (igemm4_can_run(a, p.pin, p.pout, cfg - igemm_first_v4_cfg())) return cfg;
+        cfg = first_v2;
+    }
     if (cfg >= igemm_first_v3_cfg()) {
         // the patch-staged tiles: stride 1, a filter window, 32-packed, the fast epilogue; otherwise the second-generation
         // tile of 128 x 128 (resolved below like any other request for it)
@@ -827,6 +845,7 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
         return launch_planar(st, a, cfg, cu_count);
     }
     const int first_v2 = igemm_first_v2_cfg();
+    if (cfg >= igemm_first_v4_cfg()) return launch_igemm4(st, a, p.pin, p.pout, cfg - igemm_first_v4_cfg(), cu_count);
     if (cfg >= igemm_first_v3_cfg()) return launch_igemm3(st, a, p.pin, p.pout, cfg - igemm_first_v3_cfg());
     if (cfg >= first_v2) return launch_igemm2(st, a, p.pout, cfg - first_v2, cu_count);
     if (cfg >= kNumCfgs) return launch_igemm_dma(st, a, p.pout, cfg - kNumCfgs, cu_count);

@@ -93,12 +93,14 @@ struct ZRegs {
 
 // Fetches the whole wave tile's residual at once, so that a caller can issue it ahead of the epilogue
 template <int POUT, int MT, int NT>
-__device__ __forceinline__ void igemm_load_z(const IgemmArgs& a, ZRegs<MT, NT>& zr, int oc_w, int pix_w, int l32, int lh) {
+__device__ __forceinline__ void igemm_load_z(const IgemmArgs& a, ZRegs<MT, NT>& zr, int oc_w, int pix_w, int l32, int lh,
+                                             int m_end = -1) {
     const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(a.z, a.z_bytes);
+    if (m_end < 0) m_end = a.M;
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
         const int m = pix_w + j * 32 + l32;
-        const bool pok = m < a.M;
+        const bool pok = m < m_end;
         const uint32_t mm = pok ? m : 0;
         const uint32_t n = fdiv(mm, a.div_ohw), rem = mm - n * a.OHW;
         const int z_pix = (int)n * a.z_sn + (int)rem * POUT;
@@ -123,14 +125,18 @@ __device__ __forceinline__ void igemm_load_z(const IgemmArgs& a, ZRegs<MT, NT>& 
 // ZPRE: the residual was fetched by igemm_load_z into *zr; otherwise it is loaded here, block by block
 // blk_mod > 1: only the blocks b = i * NT + j with b % blk_mod == blk_rem are written (a wave of a workgroup that
 // splits the reduction finishes its share of the blocks; wave-uniform)
+// m_end: one past the last pixel (flattened over batch and image) this tile may write
 template <int POUT, int MT, int NT, int NL, bool HZ, bool ZPRE>
 __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], const ZRegs<MT, NT>* zr, int oc_w,
-                                               int pix_w, int l32, int lh, int oc_end, int blk_mod = 1, int blk_rem = 0) {
+                                               int pix_w, int l32, int lh, int oc_end, int blk_mod, int blk_rem, int m_end) {
     const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(a.z, HZ ? a.z_bytes : 0);
+    // stores go through a buffer descriptor: a lane outside the tile carries the out-of-range offset and its store is
+    // dropped (no branch, no 64-bit address arithmetic); the channel block's offset is wave-uniform and scalar
+    const __amdgpu_buffer_rsrc_t rs_dst = make_rsrc(a.dst, a.dst_bytes);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
         const int m = pix_w + j * 32 + l32;
-        const bool pok = m < a.M;
+        const bool pok = m < m_end;
         const uint32_t mm = pok ? m : 0;
         const uint32_t n = fdiv(mm, a.div_ohw), rem = mm - n * a.OHW;
         const int d_pix = (int)n * a.dst_sn + (int)rem * POUT;
@@ -162,8 +168,12 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
                 // accumulator order -> stored order
                 auto s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
                 auto s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
-                u32x4 out = {s0[0], s0[1], s1[0], s1[1]};
-                if (pok) *reinterpret_cast<u32x4*>(a.dst + d_pix + blk_off) = out;
+                const v4i out = {(int)s0[0], (int)s0[1], (int)s1[0], (int)s1[1]};
+                __builtin_amdgcn_raw_buffer_store_b128(out, rs_dst, pok ? d_pix + lh * 16 : SENT, (ocb >> 5) * a.dst_scb, 0);
+                // A vector-memory store of more than 8 bytes reads its data registers for two more cycles after it
+                // issues, and the conversions that pack the next results are inline assembly, which the compiler's
+                // hazard check does not look into: hold the registers (as an operand of the two wait states) until then.
+                asm volatile("s_nop 1" ::"v"(out) : "memory");
             } else {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
@@ -174,7 +184,7 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
                     if (HZ) zw = ZPRE ? (uint32_t)zr->v[i][j][q]
                                       : (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_z, ok ? z_pix + off : -1, 0, 0);
                     uint32_t o = requant4_fast<NL, HZ>(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], zw, a.epi);
-                    if (ok) *reinterpret_cast<uint32_t*>(a.dst + d_pix + off) = o;
+                    __builtin_amdgcn_raw_buffer_store_b32(o, rs_dst, ok ? d_pix + off : SENT, 0, 0);
                 }
             }
         }
@@ -187,21 +197,22 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
 template <int POUT, int MT, int NT, bool ZPRE = false>
 __device__ __forceinline__ void igemm_run_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w, int l32,
                                                    int lh, const ZRegs<MT, NT>* zr = nullptr, int oc_end = -1, int blk_mod = 1,
-                                                   int blk_rem = 0) {
+                                                   int blk_rem = 0, int m_end = -1) {
     if (oc_end < 0) oc_end = a.OC;
+    if (m_end < 0) m_end = a.M;
     if (a.epi.lin) {
-        igemm_epilogue<POUT, MT, NT, NL_LIN, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem);
+        igemm_epilogue<POUT, MT, NT, NL_LIN, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem, m_end);
     } else if (a.epi.has_z) {
         switch (a.epi.nonline) {
-            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
-            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
-            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
+            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem, m_end); break;
+            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem, m_end); break;
+            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem, m_end); break;
         }
     } else {
         switch (a.epi.nonline) {
-            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
-            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
-            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem); break;
+            case NL_RELU: igemm_epilogue<POUT, MT, NT, NL_RELU, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem, m_end); break;
+            case NL_H_SWISH: igemm_epilogue<POUT, MT, NT, NL_H_SWISH, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem, m_end); break;
+            default: igemm_epilogue<POUT, MT, NT, NL_IDENTITY, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem, m_end); break;
         }
     }
 }
@@ -380,6 +391,13 @@ int igemm3_num_cfgs();
 const char* igemm3_cfg_name(int cfg);
 bool igemm3_can_run(const IgemmArgs& a, int pin, int pout, int cfg);
 int launch_igemm3(hipStream_t st, IgemmArgs& a, int pin, int pout, int cfg);
+
+// weight-resident kernel for 3x3 / stride 1 / pad 1 over 32 or 64 input channels, 32-packed (conv_igemm4.hip): the
+// reference filter layout only
+int igemm4_num_cfgs();
+const char* igemm4_cfg_name(int cfg);
+bool igemm4_can_run(const IgemmArgs& a, int pin, int pout, int cfg);
+int launch_igemm4(hipStream_t st, IgemmArgs& a, int pin, int pout, int cfg, int cu_count);
 
 // streaming kernel for 4-packed pointwise layers with few input or few output channels (conv_pw4.hip)
 bool pw4s_usable(const IgemmArgs& a);

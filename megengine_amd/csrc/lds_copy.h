@@ -42,6 +42,16 @@ __device__ __forceinline__ void lds_copy_row64x4(uint32_t lds_addr, int voff, in
         : "memory", "m0");
 }
 
+__device__ __forceinline__ void lds_copy_row64x16(uint32_t lds_addr, int voff, int soff, const v4i& rsrc) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dwordx4 %1, %2, %3 offen lds"
+        :
+        : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+        : "memory", "m0");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N < 64, "vmcnt range");

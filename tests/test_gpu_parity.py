@@ -399,6 +399,9 @@ def test_heuristic_picks(oracle):
         a, _ = ops.conv_bias_query(_abi.make_conv_desc("NCHW32", 64, ic, hw, hw, oc, f, pad=f // 2, **S8),
                                    _abi.ALGO_HEURISTIC_PREPROCESS)
         assert a.id == IGEMM and names[a.tile_cfg] == want, (ic, hw, oc, f, names[a.tile_cfg])
+    # the same 3x3 over 64 channels at batch 128, five tiles per workgroup: the weight-resident tile
+    a, _ = ops.conv_bias_query(_abi.make_conv_desc("NCHW32", 128, 64, 56, 56, 64, 3, pad=1, **S8), _abi.ALGO_HEURISTIC_PREPROCESS)
+    assert a.id == IGEMM and names[a.tile_cfg] == "v4_64x128res", names[a.tile_cfg]
 
 
 def test_general_epilogue_on_the_mfma_kernel(oracle):
@@ -707,6 +710,43 @@ def test_first_layer_kernel(oracle, i):
                             bias_mode=_abi.BIAS_NONE, src_stride_n=int(np.prod(ss[1:])) + 20,
                             dst_stride_n=int(np.prod(ds[1:])) + 12, z_stride_n=int(np.prod(ds[1:])) + 36, **S)
     check_case(oracle, d, seed=600 + i, tag="c4-%d-strided" % i)
+
+
+RESIDENT_CASES = [
+    # n, ic, ih, iw, oc: 3x3 / stride 1 / pad 1 over 32 or 64 channels, the shapes the weight-resident tile takes
+    (2, 64, 56, 56, 64),      # the ResNet-50 case: 24.5 tiles per image, the last one half full
+    (3, 32, 17, 23, 96),      # odd sizes, two channel tiles (the second one half full), rows of 23 pixels
+    (2, 64, 14, 14, 128),     # tiles of 128 pixels cover 9 rows; two channel tiles: weights reloaded between runs
+    (5, 64, 7, 7, 64),        # a whole image is less than half a tile
+    (1, 64, 28, 28, 192),     # three channel tiles
+    (4, 32, 60, 61, 64),      # rows wider than one copy of 64 pieces
+    (2, 32, 112, 112, 32),    # rows of four copies, half a channel tile
+]
+
+
+@pytest.mark.parametrize("i", range(len(RESIDENT_CASES)))
+def test_weight_resident_tile(oracle, i):
+    n, ic, ih, iw, oc = RESIDENT_CASES[i]
+    tile = lib.tile_names().index("v4_64x128res")
+    k = ic * 9
+    live = dict(scale_bias=2e-4, scale_z=0.02, scale_dst=float(np.float32(2e-4 * 73.9 * 73.3 * k ** 0.5 / 25.0)))
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        for has_z in (False, True):
+            d = _abi.make_conv_desc("NCHW32", n, ic, ih, iw, oc, 3, pad=1, nonline=nl, has_z=has_z, **live)
+            assert lib.tile_usable(d, tile)
+            check_case(oracle, d, seed=700 + i, algo=IGEMM, tile=tile, tag="resident-%d" % i)
+    # batch-strided views, no bias
+    d0 = _abi.make_conv_desc("NCHW32", n, ic, ih, iw, oc, 3, pad=1, nonline="RELU", has_z=True, **live)
+    ss, fs, bs, ds = _abi.conv_shapes(d0)
+    d = _abi.make_conv_desc("NCHW32", n, ic, ih, iw, oc, 3, pad=1, nonline="RELU", has_z=True, bias_mode=_abi.BIAS_NONE,
+                            src_stride_n=int(np.prod(ss[1:])) + 64, dst_stride_n=int(np.prod(ds[1:])) + 32,
+                            z_stride_n=int(np.prod(ds[1:])) + 96, **live)
+    check_case(oracle, d, seed=720 + i, algo=IGEMM, tile=tile, tag="resident-%d-strided" % i)
+    # what it does not take: other strides, paddings, filter sizes, channel counts
+    for kw in (dict(stride=2), dict(pad=0), dict(f=5, pad=2), dict(ic=128), dict(ic=96)):
+        dd = _abi.make_conv_desc("NCHW32", n, kw.get("ic", ic), ih, iw, oc, kw.get("f", 3), pad=kw.get("pad", 1),
+                                 stride=kw.get("stride", 1), **live)
+        assert not lib.tile_usable(dd, tile), kw
 
 
 def test_first_layer_kernel_on_random_shapes(oracle):

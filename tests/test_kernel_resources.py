@@ -88,3 +88,16 @@ def test_patch_staged_kernels_use_no_scratch(resources):
 def test_second_generation_kernels_use_no_scratch_in_the_tiles_the_heuristic_takes(resources):
     for name, r in kernels(resources, r"igemm2_kernel<(32|4), (128, 128, 2, 2, 2, 4|64, 128, 2, 2, 4, 3|64, 128, 2, 2, 2, 4|64, 64, 2, 2, 4, 4), \d, (true|false), (true|false), false, 1>").items():
         assert r["scratch"] == 0, (name, r)
+
+
+def test_ring_kernels_with_register_resident_weights_use_no_scratch(resources):
+    """c4_kernel and igemm4_kernel keep their weights in registers across a tile loop that has LDS-direct copies in
+    flight: a spill there is reloaded with vmcnt(0) inside the loop and empties the ring.  The first-layer kernel for the
+    7x7 stem must also leave room for four workgroups per CU."""
+    c4 = kernels(resources, r"c4_kernel<")
+    r4 = kernels(resources, r"igemm4_kernel<")
+    assert len(c4) == 12 and len(r4) == 4
+    for name, r in list(c4.items()) + list(r4.items()):
+        assert r["scratch"] == 0, (name, r)
+    for name, r in kernels(resources, r"c4_kernel<2, false, 7>").items():
+        assert r["vgprs"] <= 128, (name, r)
