@@ -250,12 +250,13 @@ int mi355_igemm_tile_usable(const mi355_conv_desc* d, int tile_cfg);
 int mi355_epilogue_linear_form(float scale_bias, float scale_dst, uint32_t nonline, float* c, float* d);
 
 /* The division r / scale_dst of the requantisation (dnn/include/megdnn/dtype.h:846) runs in the tiled kernels as
- *     q0 = r * y;  e = fma(-q0, scale_dst, r);  q = fma(e, y, q0)          y = RN(1 / scale_dst)
- * -- a faithful quotient, which can change a result only next to a rounding boundary of roundf.  The library uses it for
- * a dst scale only after it has evaluated this form and the literal chain (IEEE divide, roundf, clamp) on every float
- * around every such boundary and found them equal; other scales run the literal chain.  Returns 1 and y if the scale
- * has passed, 0 if not, a negative mi355_status on a bad argument.  Diagnostic: no counterpart in the reference. */
-int mi355_epilogue_quotient_form(float scale_dst, float* y);
+ *     t = r * y_lo;  q = fma(r, y_hi, t)          y_hi = RN(1 / scale_dst),  y_lo = RN(1 / scale_dst - y_hi)
+ * -- a quotient at most one ulp from the correctly rounded one, which can change a result only next to a rounding
+ * boundary of roundf.  The library uses it for a dst scale only after it has evaluated this form and the literal chain
+ * (IEEE divide, roundf, clamp) on every float around every such boundary and found them equal; other scales run the
+ * literal chain.  Returns 1 and the two parts of the reciprocal if the scale has passed, 0 if not, a negative
+ * mi355_status on a bad argument.  Diagnostic: no counterpart in the reference. */
+int mi355_epilogue_quotient_form(float scale_dst, float* y_hi, float* y_lo);
 
 /* ---- RelayoutFormat ---- */
 /* param::RelayoutFormat::Mode values (opr_param_defs.py:1069-1111); 32/33 and 34/35 are

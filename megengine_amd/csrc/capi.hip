@@ -57,25 +57,27 @@ bool epi_fast_ok(float s_b, float s_z, float s_d, bool has_z) {
 
 // ---- divide-free quotient of the fast epilogue form (epilogue.h): host-side proof per dst scale --------------------
 // From the float r on, the contract is  clamp(roundf(RN(r / s_d)))  and the fast form replaces RN(r / s_d) by
-//     q0 = RN(r y);  e = fma(-q0, s_d, r);  q = fma(e, y, q0)          y = RN(1 / s_d).
-// q0 is within two ulps of r / s_d (the rounding of y and its own), its residual e is r - q0 s_d to within one rounding
-// of a quantity of two ulps, and q = RN(q0 + e y) differs from r / s_d by less than one ulp before its own rounding: q
-// is a faithful quotient, |q - RN(r / s_d)| <= 1 ulp, for every s_d and r that epi_fast_ok admits (no intermediate
-// leaves the normal range).  A faithful quotient can change the result only where RN(r / s_d) lies within one ulp of a
-// rounding boundary k + 0.5 of roundf, i.e. for a handful of consecutive floats r around each of the 128 boundary
-// magnitudes.  The proof therefore finds every boundary of the literal chain by bisection over the floats and evaluates
-// BOTH forms, with the device's own operations (IEEE multiply and fma, clamp, the two integer conversions), on the 33
-// floats around it, on both signs.  Equal there = equal on every float r.  A scale that fails (none is known: 20 000
-// log-uniform draws and the special scales of the tests all pass) runs the literal chain with the IEEE divide.
+//     t = RN(r y_lo);  q = fma(r, y_hi, t)          y_hi = RN(1 / s_d),  y_lo = RN(1 / s_d - y_hi)
+// y_hi + y_lo is 1 / s_d to 2^-48 relative, t carries a rounding error 2^-24 below its own size, which is 2^-24 below q:
+// q is r / s_d with a relative error of about 2^-47 before its single rounding, i.e. the correctly rounded quotient
+// except where r / s_d lies that close to the midpoint of two floats, and never more than one ulp from it, for every
+// s_d and r that epi_fast_ok admits (no intermediate leaves the normal range).  Such a quotient can change the result
+// only where RN(r / s_d) lies within one ulp of a rounding boundary k + 0.5 of roundf, i.e. for a handful of consecutive
+// floats r around each of the 128 boundary magnitudes.  The proof therefore finds every boundary of the literal chain
+// by bisection over the floats and evaluates BOTH forms, with the device's own operations (IEEE multiply and fma, clamp,
+// the two integer conversions), on the 33 floats around it, on both signs.  Equal there = equal on every float r.  A
+// scale that fails (none is known: 20 000 log-uniform draws and the special scales of the tests all pass) runs the
+// literal chain with the IEEE divide.  (One instruction shorter than the reciprocal-times-residual correction it
+// replaces: q0 = r y; e = fma(-q0, s_d, r); q = fma(e, y, q0).)
+float epi_recip_lo(float s_d) { return (float)(1.0 / (double)s_d - (double)(1.0f / s_d)); }
 int epi_tail_contract(float r, float s_d) {
     float v = roundf(r / s_d);
     v = fminf(fmaxf(-128.f, v), 127.f);
     return (int)v;
 }
-int epi_tail_fast(float r, float s_d, float y_hi, bool relu) {
-    const float q0 = r * y_hi;
-    const float res = fmaf(-q0, s_d, r);
-    float q = fmaf(res, y_hi, q0);
+int epi_tail_fast(float r, float y_hi, float y_lo, bool relu) {
+    const float t = r * y_lo;
+    float q = fmaf(r, y_hi, t);
     if (relu) {
         q = fminf(fmaxf(q, 0.f), 127.f);
         return (int)floor((double)q + 0.5);  // v_cvt_rpi_i32_f32: floor(q + 0.5) without an intermediate rounding
@@ -89,7 +91,7 @@ float f_from_bits(uint32_t b) {
     return f;
 }
 bool epi_prove_quotient(float s_d) {
-    const float y_hi = 1.0f / s_d;
+    const float y_hi = 1.0f / s_d, y_lo = epi_recip_lo(s_d);
     const float top = 130.f * s_d;  // beyond the last boundary: finite by epi_fast_ok
     uint32_t top_bits;
     memcpy(&top_bits, &top, 4);
@@ -105,11 +107,11 @@ bool epi_prove_quotient(float s_d) {
             const int64_t b = (int64_t)hi + d;
             if (b <= 0 || b >= 0x7f800000) continue;
             const float m = f_from_bits((uint32_t)b);
-            if (epi_tail_fast(-m, s_d, y_hi, false) != epi_tail_contract(-m, s_d)) return false;
+            if (epi_tail_fast(-m, y_hi, y_lo, false) != epi_tail_contract(-m, s_d)) return false;
             // the positive side has the same boundaries (round half away from zero) up to the clamp at 127
-            if (epi_tail_fast(m, s_d, y_hi, false) != epi_tail_contract(m, s_d)) return false;
-            if (epi_tail_fast(m, s_d, y_hi, true) != epi_tail_contract(m, s_d)) return false;
-            if (epi_tail_fast(-m, s_d, y_hi, true) != 0) return false;  // RELU folded into the clamp
+            if (epi_tail_fast(m, y_hi, y_lo, false) != epi_tail_contract(m, s_d)) return false;
+            if (epi_tail_fast(m, y_hi, y_lo, true) != epi_tail_contract(m, s_d)) return false;
+            if (epi_tail_fast(-m, y_hi, y_lo, true) != 0) return false;  // RELU folded into the clamp
         }
     }
     return true;
@@ -261,6 +263,7 @@ void epi_fill(EpiParams* e, float s_b, float s_z, float s_d, uint32_t nonline, b
     e->has_z = has_z ? 1 : 0;
     e->fast = qs8 && epi_fast_ok(s_b, s_z, s_d, has_z) && epi_quotient_proved(s_d);
     e->y_hi = 1.0f / s_d;
+    e->y_lo = epi_recip_lo(s_d);
     e->lin = 0;
     e->lin_c = e->lin_d = 0.f;
     e->lin_lo = nonline == MI355_NL_RELU ? 0.f : -128.f;
@@ -871,9 +874,10 @@ int mi355_igemm_tile_usable(const mi355_conv_desc* d, int tile_cfg) {
     return MI355_OK;
 }
 
-int mi355_epilogue_quotient_form(float scale_dst, float* y) {
-    if (!y) return -fail(MI355_ERR_BAD_ARG, "null argument");
-    *y = 1.0f / scale_dst;
+int mi355_epilogue_quotient_form(float scale_dst, float* y_hi, float* y_lo) {
+    if (!y_hi || !y_lo) return -fail(MI355_ERR_BAD_ARG, "null argument");
+    *y_hi = 1.0f / scale_dst;
+    *y_lo = epi_recip_lo(scale_dst);
     if (!epi_fast_ok(1.f, 1.f, scale_dst, false)) return 0;
     return epi_quotient_proved(scale_dst) ? 1 : 0;
 }

@@ -10,11 +10,11 @@
 //     dst = (int8) min(max(-128, v), 127)
 //
 // The "fast" form below produces the same bits with no hardware divide:
-//   * division by the per-tensor constant s_dst: with y = RN(1/s_dst)
-//       q0 = r * y                       first estimate, within two ulps of r / s_dst
-//       e  = fma(-q0, s_dst, r)          its residual
-//       q  = fma(e, y, q0)               faithful quotient: less than one ulp from r / s_dst (Markstein's correction step)
-//     A faithful quotient can change the result only next to a rounding boundary of roundf; the host proves the form
+//   * division by the per-tensor constant s_dst: with the reciprocal as an unevaluated sum of two floats,
+//     y_hi = RN(1/s_dst), y_lo = RN(1/s_dst - y_hi) (computed in double precision on the host),
+//       t = r * y_lo                     the part of the quotient that y_hi misses (24 bits below it)
+//       q = fma(r, y_hi, t)              r (y_hi + y_lo) rounded once: less than one ulp from r / s_dst
+//     Such a quotient can change the result only next to a rounding boundary of roundf; the host proves the form
 //     for every dst scale before a kernel may use it (epi_prove_quotient in capi.hip).
 //   * RELU is folded into the clamp: for s_dst > 0, r <= 0 gives q <= 0 which clamps to 0.
 //   * roundf + clamp + convert: clamp first, then trunc(q + copysign(pred(0.5), q)); for
@@ -44,6 +44,7 @@ namespace mi355 {
 struct EpiParams {
     float s_b, s_z, s_d;
     float y_hi;   // RN(1 / s_d)
+    float y_lo;   // RN(1 / s_d - y_hi)
     int nonline;  // MI355_NL_*
     int has_z;
     int fast;     // 1: fast form allowed
@@ -112,9 +113,8 @@ __device__ __forceinline__ float requant_fast_value(int sfb, int z, const EpiPar
         float m = r * t;
         r = m * (1.f / 6.f);
     }
-    float q0 = r * e.y_hi;
-    float res = __builtin_fmaf(-q0, e.s_d, r);
-    float q = __builtin_fmaf(res, e.y_hi, q0);
+    float t = r * e.y_lo;
+    float q = __builtin_fmaf(r, e.y_hi, t);
     if (NL == NL_RELU) return __builtin_amdgcn_fmed3f(q, 0.f, 127.f);  // q is finite here: same as min(max(q, 0), 127)
     q = __builtin_amdgcn_fmed3f(q, -128.f, 127.f);
     return q + __builtin_copysignf(0.49999997f, q);

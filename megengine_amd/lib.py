@@ -76,7 +76,7 @@ def lib():
     L.mi355_igemm_tile_name.argtypes = [C.c_int]
     L.mi355_igemm_tile_usable.argtypes = [P(_abi.ConvDesc), C.c_int]
     L.mi355_epilogue_quotient_form.restype = C.c_int
-    L.mi355_epilogue_quotient_form.argtypes = [C.c_float, P(C.c_float)]
+    L.mi355_epilogue_quotient_form.argtypes = [C.c_float, P(C.c_float), P(C.c_float)]
     L.mi355_epilogue_linear_form.restype = C.c_int
     L.mi355_epilogue_linear_form.argtypes = [C.c_float, C.c_float, C.c_uint32, P(C.c_float), P(C.c_float)]
     L.mi355_relayout_deduce.argtypes = [P(_abi.RelayoutDesc), P(C.c_uint32), P(C.c_uint32)]

@@ -128,7 +128,8 @@ int main(int argc, char** argv) {
                 // the proofs directly, on scales that other threads prove at the same time
                 float y = 0.f, c = 0.f, dd = 0.f;
                 const float s = scales[r() % scales.size()];
-                (void)mi355_epilogue_quotient_form(s, &y);
+                float y2;
+                (void)mi355_epilogue_quotient_form(s, &y, &y2);
                 (void)mi355_epilogue_linear_form(s * 1e-2f, s, MI355_NL_RELU, &c, &dd);
             }
         });
