@@ -402,5 +402,8 @@ int launch_igemm4(hipStream_t st, IgemmArgs& a, int pin, int pout, int cfg, int 
 // streaming kernel for 4-packed pointwise layers with few input or few output channels (conv_pw4.hip)
 bool pw4s_usable(const IgemmArgs& a);
 int launch_pw4s(hipStream_t st, const IgemmArgs& a, int cu_count);
+// the same for 32-packed pointwise layers with at most 128 input channels (tile "pw32_stream")
+bool pw32s_usable(const IgemmArgs& a, int pin, int pout);
+int launch_pw32s(hipStream_t st, const IgemmArgs& a, int cu_count);
 
 }  // namespace mi355

@@ -399,6 +399,10 @@ def test_heuristic_picks(oracle):
         a, _ = ops.conv_bias_query(_abi.make_conv_desc("NCHW32", 64, ic, hw, hw, oc, f, pad=f // 2, **S8),
                                    _abi.ALGO_HEURISTIC_PREPROCESS)
         assert a.id == IGEMM and names[a.tile_cfg] == want, (ic, hw, oc, f, names[a.tile_cfg])
+    # pointwise over 64 channels on both sides: the streaming kernel, with or without weight pre-processing
+    for req in (_abi.ALGO_HEURISTIC, _abi.ALGO_HEURISTIC_PREPROCESS):
+        a, _ = ops.conv_bias_query(_abi.make_conv_desc("NCHW32", 64, 64, 56, 56, 64, 1, **S8), req)
+        assert a.id == IGEMM and names[a.tile_cfg] == "pw32_stream", names[a.tile_cfg]
     # the same 3x3 over 64 channels at batch 128, five tiles per workgroup: the weight-resident tile
     a, _ = ops.conv_bias_query(_abi.make_conv_desc("NCHW32", 128, 64, 56, 56, 64, 3, pad=1, **S8), _abi.ALGO_HEURISTIC_PREPROCESS)
     assert a.id == IGEMM and names[a.tile_cfg] == "v4_64x128res", names[a.tile_cfg]
@@ -746,6 +750,40 @@ def test_weight_resident_tile(oracle, i):
     for kw in (dict(stride=2), dict(pad=0), dict(f=5, pad=2), dict(ic=128), dict(ic=96)):
         dd = _abi.make_conv_desc("NCHW32", n, kw.get("ic", ic), ih, iw, oc, kw.get("f", 3), pad=kw.get("pad", 1),
                                  stride=kw.get("stride", 1), **live)
+        assert not lib.tile_usable(dd, tile), kw
+
+
+STREAM32_CASES = [
+    # n, ic, ih, iw, oc, stride: pointwise over 32 .. 128 channels, 32-packed -- what the streaming kernel takes
+    (2, 64, 56, 56, 256, 1),     # the expanding 1x1 of the first bottleneck
+    (3, 32, 17, 23, 96, 1),      # odd sizes; three channel blocks: the second wave group is half empty
+    (2, 128, 14, 14, 512, 1),    # four k-steps
+    (5, 64, 7, 7, 64, 1),        # a block of 32 pixels straddles images
+    (1, 96, 28, 28, 32, 1),      # a single channel block per wave, three k-steps
+    (4, 64, 30, 31, 160, 2),     # strided (a projection shortcut), five channel blocks
+    (2, 128, 28, 28, 1024, 2),   # the widest output it takes
+]
+
+
+@pytest.mark.parametrize("i", range(len(STREAM32_CASES)))
+def test_streaming_pointwise_kernel_32_packed(oracle, i):
+    n, ic, ih, iw, oc, stride = STREAM32_CASES[i]
+    tile = lib.tile_names().index("pw32_stream")
+    live = dict(scale_bias=2e-4, scale_z=0.02, scale_dst=float(np.float32(2e-4 * 73.9 * 73.3 * ic ** 0.5 / 25.0)))
+    for nl in ("IDENTITY", "RELU", "H_SWISH"):
+        for has_z in (False, True):
+            d = _abi.make_conv_desc("NCHW32", n, ic, ih, iw, oc, 1, stride=stride, nonline=nl, has_z=has_z, **live)
+            assert lib.tile_usable(d, tile)
+            check_case(oracle, d, seed=800 + i, algo=IGEMM, tile=tile, tag="stream32-%d" % i)
+    d0 = _abi.make_conv_desc("NCHW32", n, ic, ih, iw, oc, 1, stride=stride, nonline="RELU", has_z=True, **live)
+    ss, fs, bs, ds = _abi.conv_shapes(d0)
+    d = _abi.make_conv_desc("NCHW32", n, ic, ih, iw, oc, 1, stride=stride, nonline="RELU", has_z=True, bias_mode=_abi.BIAS_NONE,
+                            src_stride_n=int(np.prod(ss[1:])) + 64, dst_stride_n=int(np.prod(ds[1:])) + 32,
+                            z_stride_n=int(np.prod(ds[1:])) + 96, **live)
+    check_case(oracle, d, seed=820 + i, algo=IGEMM, tile=tile, tag="stream32-%d-strided" % i)
+    # what it does not take: a filter window, more than 128 input channels, more than 1024 output channels
+    for kw in (dict(f=3, pad=1), dict(ic=256), dict(oc=2048)):
+        dd = _abi.make_conv_desc("NCHW32", n, kw.get("ic", ic), ih, iw, kw.get("oc", oc), kw.get("f", 1), pad=kw.get("pad", 0), **live)
         assert not lib.tile_usable(dd, tile), kw
 
 
