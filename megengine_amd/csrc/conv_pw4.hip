@@ -99,8 +99,7 @@ __global__ __launch_bounds__(256) void pw4s_kernel(IgemmArgs a, int n_ocg, int n
 // of k-step kc is one 16-byte load -- half of its pixel's 32-byte block kc; 32 consecutive pixels are one contiguous
 // kilobyte -- and the stores are the 16-byte stores of the tiled kernels.
 template <int MT, int KC, bool HZ>
-__global__ __launch_bounds__(256) void pw32s_kernel(IgemmArgs a, int n_ocg, int n_pb) {
-    __shared__ __attribute__((aligned(16))) int sBias[PW4_MAX_OC + 96];
+__global__ __launch_bounds__(256, 2) void pw32s_kernel(IgemmArgs a, int n_ocg, int n_pb) {
     const int t = threadIdx.x;
     const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
@@ -110,6 +109,7 @@ __global__ __launch_bounds__(256) void pw32s_kernel(IgemmArgs a, int n_ocg, int 
     const int oc_w = ocg * MT * 32;
     const __amdgpu_buffer_rsrc_t rs_src = make_rsrc(a.src, a.src_bytes);
     const __amdgpu_buffer_rsrc_t rs_flt = make_rsrc(a.flt, a.flt_bytes);
+    const __amdgpu_buffer_rsrc_t rs_bias = make_rsrc(a.bias, a.has_bias ? a.OC * 4 : 0);
 
     v4i fa[MT][KC];
 #pragma unroll
@@ -119,6 +119,16 @@ __global__ __launch_bounds__(256) void pw32s_kernel(IgemmArgs a, int n_ocg, int 
         for (int kc = 0; kc < KC; ++kc)
             fa[i][kc] = __builtin_amdgcn_raw_buffer_load_b128(rs_flt, row < a.OC ? row * a.kbytes + kc * 32 + lh * 16 : SENT, 0, 0);
     }
+    // the bias of the wave's channels, in accumulator order: the first multiply of every block takes it as its addend
+    // (channels past the last one read as zero through the descriptor)
+    v16i bv[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const v4i b = __builtin_amdgcn_raw_buffer_load_b128(rs_bias, (oc_w + i * 32 + 8 * q + 4 * lh) * 4, 0, 0);
+            bv[i][4 * q + 0] = b[0]; bv[i][4 * q + 1] = b[1]; bv[i][4 * q + 2] = b[2]; bv[i][4 * q + 3] = b[3];
+        }
 
     auto load_b = [&](int pb, v4i (&x)[KC]) __attribute__((always_inline)) {
         const int m = pb * 32 + l32;
@@ -135,22 +145,15 @@ __global__ __launch_bounds__(256) void pw32s_kernel(IgemmArgs a, int n_ocg, int 
     ZRegs<HZ ? MT : 1, 1> zr, nz;
     load_b(pb0, fb);
     if constexpr (HZ) igemm_load_z<32, MT, 1>(a, zr, oc_w, pb0 * 32, l32, lh);
-    for (int i = t; i < PW4_MAX_OC + 96; i += 256) sBias[i] = (a.has_bias && i < a.OC) ? a.bias[i] : 0;
-    __syncthreads();
     for (int pb = pb0; pb < n_pb; pb += step) {
         // the next block's pixels and residual are in flight during the multiply and the epilogue
         load_b(pb + step, nb);
         if constexpr (HZ) igemm_load_z<32, MT, 1>(a, nz, oc_w, (pb + step) * 32, l32, lh);
         v16i acc[MT][1];
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
+        for (int i = 0; i < MT; ++i) acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i][0], fb[0], bv[i], 0, 0, 0);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const v4i b = *reinterpret_cast<const v4i*>(sBias + oc_w + i * 32 + 8 * q + 4 * lh);
-                acc[i][0][4 * q + 0] = b[0]; acc[i][0][4 * q + 1] = b[1]; acc[i][0][4 * q + 2] = b[2]; acc[i][0][4 * q + 3] = b[3];
-            }
-#pragma unroll
-        for (int kc = 0; kc < KC; ++kc)
+        for (int kc = 1; kc < KC; ++kc)
 #pragma unroll
             for (int i = 0; i < MT; ++i) acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i][kc], fb[kc], acc[i][0], 0, 0, 0);
         if constexpr (HZ)
