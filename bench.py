@@ -45,6 +45,8 @@ def main():
     ap.add_argument("--no-preprocess", action="store_true", help="exec with the filters in the reference layout only")
     ap.add_argument("--no-memory-plan", action="store_true",
                     help="one buffer per layer output instead of the static activation-memory plan")
+    ap.add_argument("--no-residual-in-place", action="store_true",
+                    help="memory plan without letting a layer write its output over a residual it reads last")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch one plain 256 MiB streaming kernel (counter calibration for profilers)")
     ap.add_argument("--layers-out", default=None, help="write the per-layer table to this JSON file")
@@ -88,8 +90,9 @@ def main():
     layers = workloads.resnet50(batch)
     plan = workloads.build_stack(layers, 7)
     # activation memory laid out once by liveness, as the graph runtime above the operator does before it runs a
-    # computing sequence (--no-memory-plan: one buffer per layer output)
-    mem = None if args.no_memory_plan else workloads.plan_memory(plan)
+    # computing sequence (--no-memory-plan: one buffer per layer output); a block's last layer writes its output over
+    # the residual it adds, which nothing reads after it
+    mem = None if args.no_memory_plan else workloads.plan_memory(plan, residual_in_place=not args.no_residual_in_place)
     # algorithm choice and weight pre-processing happen once, before the timed region (exec_preprocess is the
     # reference's own hook for hoisting filter re-tiling out of exec)
     workloads.choose_algorithms(plan, weight_preprocess=not args.no_preprocess)
@@ -248,8 +251,10 @@ def main():
                            batch=batch, layers=nl, launch=launch_mode, graph=graph_note,
                            activation_memory=("one buffer per layer output, %.0f MB" % (sum(p["dst"].numel() for p in plan) / 1e6)
                                               if mem is None else
-                                              "static plan by liveness: %.0f MB for the %.0f MB of layer outputs"
-                                              % (mem["planned"] / 1e6, mem["one_buffer_per_layer"] / 1e6)),
+                                              "static plan by liveness: %.0f MB for the %.0f MB of layer outputs%s"
+                                              % (mem["planned"] / 1e6, mem["one_buffer_per_layer"] / 1e6,
+                                                 "" if args.no_residual_in_place else
+                                                 ", outputs written over residuals read for the last time")),
                            weight_preprocess="%d of %d filters pre-processed once through exec_preprocess, outside the timed "
                                              "region" % (sum(p.get("pre") is not None for p in plan), nl)),
                eager_ms_per_step=round(eager_ms, 4),

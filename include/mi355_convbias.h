@@ -106,6 +106,9 @@ enum { MI355_DT_QS8 = 0, MI355_DT_QS32 = 1, MI355_DT_F32 = 2 /* Float32 dst: NCH
  *   bias: int32, (1, oc, 1, 1) / (1, oc/p, 1, 1, p) of the dst pack, or the full dst shape.
  *   z:    dst dtype and shape, own scale.
  * src/dst/z may have a non-contiguous batch dimension: *_stride_n are in elements, 0 = dense.
+ * dst may be the very buffer of z (same address, same batch stride, same dtype): every kernel reads the residual of an
+ * output element in the thread that writes that element, before the write, so the output replaces the residual in
+ * place.  Any other overlap of dst with an input is undefined.
  */
 typedef struct mi355_conv_desc {
     uint32_t format;

@@ -157,41 +157,64 @@ def build_stack(layers, seed):
 
 
 def first_fit_offsets(tensors, granule=4096):
-    """Offsets for tensors given as (bytes, index of the writing step, index of the last reading step), in writing
-    order: each goes to the lowest granule-aligned offset where it overlaps no tensor that is live at its writing step
-    (written earlier and read at that step or later).  Returns (offsets, arena bytes)."""
+    """Offsets for tensors given as (bytes, index of the writing step, index of the last reading step[, index of a
+    tensor whose range this one may take over]), in writing order: each goes to the lowest granule-aligned offset where
+    it overlaps no tensor that is live at its writing step (written earlier and read at that step or later).  A tensor
+    with a take-over candidate -- an earlier tensor of the same size whose last reading step is this tensor's writing
+    step -- gets that tensor's range instead.  Returns (offsets, arena bytes)."""
     live, offsets, top = [], [], 0
-    for size, i, last_read in tensors:
+    for k, spec in enumerate(tensors):
+        size, i, last_read = spec[:3]
+        over = spec[3] if len(spec) > 3 else None
         live = [r for r in live if r[2] >= i]
         size = (size + granule - 1) // granule * granule
-        off = 0
-        for o, sz, _ in sorted(live):
-            if off + size <= o:
-                break
-            off = max(off, o + sz)
-        live.append((off, size, max(last_read, i)))
+        off = None
+        if over is not None:
+            for r in live:
+                if r[3] == over and r[1] == size and r[2] == i:
+                    off = r[0]
+                    live.remove(r)
+                    break
+        if off is None:
+            off = 0
+            for o, sz, _, _ in sorted(live):
+                if off + size <= o:
+                    break
+                off = max(off, o + sz)
+        live.append((off, size, max(last_read, i), k))
         offsets.append(off)
         top = max(top, off + size)
     return offsets, top
 
 
-def plan_memory(plan):
+def plan_memory(plan, residual_in_place=False):
     """Static activation-memory plan for a layer list of build_stack, as a graph runtime lays out the variables of a
     computing sequence before it runs (the reference: StaticMemAlloc, src/core/impl/graph/var_node_mem_mgr/
     static_mem_alloc.h:18-40, intervals = first write to last read): every layer output becomes a range of ONE arena
     that no LIVE tensor occupies -- live = written and still to be read, as a source or a residual, by this layer or a
     later one -- at the lowest address where it fits (address-ordered first fit, 4 KiB granules), instead of a buffer
-    of its own.  Graph inputs (seeded tensors) keep theirs.  A layer never writes memory it reads.  Rewires src / z / dst
-    of the plan in place; returns the bytes of activation memory before and after."""
+    of its own.  Graph inputs (seeded tensors) keep theirs.  A layer never writes memory it reads as a source;
+    `residual_in_place`: a layer whose residual is read for the last time by that very layer writes its output over it
+    (every kernel reads the residual of an output element in the thread that writes the element, before the write).
+    Rewires src / z / dst of the plan in place; returns the bytes of activation memory before and after."""
     import torch
 
-    last = {}
+    last, producer = {}, {}
     for i, p in enumerate(plan):
         for t in (p["src"], p["z"]):
             if t is not None:
                 last[t.data_ptr()] = i
-    # an output nobody reads is dead after its own layer
-    offsets, top = first_fit_offsets([(p["dst"].numel(), i, last.get(p["dst"].data_ptr(), i)) for i, p in enumerate(plan)])
+        producer[p["dst"].data_ptr()] = i
+    specs = []
+    for i, p in enumerate(plan):
+        over = None
+        z = p["z"]
+        if residual_in_place and z is not None and z.data_ptr() in producer and last[z.data_ptr()] == i and \
+                z.numel() == p["dst"].numel() and z.data_ptr() != p["src"].data_ptr():
+            over = producer[z.data_ptr()]
+        # an output nobody reads is dead after its own layer
+        specs.append((p["dst"].numel(), i, last.get(p["dst"].data_ptr(), i), over))
+    offsets, top = first_fit_offsets(specs)
     before = sum(p["dst"].numel() for p in plan)
     arena = torch.empty(top, dtype=plan[0]["dst"].dtype, device=plan[0]["dst"].device)
     remap = {}    # data_ptr of the original output -> its range of the arena
@@ -207,16 +230,18 @@ def plan_memory(plan):
 
 
 def snapshot_run(plan, calls, images):
-    """Runs the launches of a plan once, in order, and copies the first `images` images of every layer's source,
-    residual and output to the host right after its launch: with planned activation memory a buffer holds a layer's
-    output only until its last reader has run."""
+    """Runs the launches of a plan once, in order, and copies the first `images` images of every layer's source and
+    residual to the host right before its launch and of its output right after: with planned activation memory a
+    buffer holds a tensor only until its last reader has run, and an output may replace the residual it was made from."""
     import torch
 
     snaps = []
     for p, c in zip(plan, calls):
+        torch.cuda.synchronize()
+        h_in = [None if t is None else t[:images].cpu().numpy() for t in (p["src"], p["z"])]
         c()
         torch.cuda.synchronize()
-        snaps.append(tuple(None if t is None else t[:images].cpu().numpy() for t in (p["src"], p["z"], p["dst"])))
+        snaps.append((h_in[0], h_in[1], p["dst"][:images].cpu().numpy()))
     return snaps
 
 

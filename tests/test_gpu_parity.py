@@ -960,3 +960,53 @@ def test_depthwise_random_descriptors(oracle):
         d = _abi.make_conv_desc("NCHW4", n, c, ih, iw, c, 3, **kw)
         assert ops.conv_bias_query(d)[0].id == DW
         check_case(oracle, d, seed=2000 + it, tag="dw random %d" % it)
+
+
+IN_PLACE_CASES = [
+    # fmt, n, ic, ih, iw, oc, f, stride, pad, group: one shape per kernel family and tile geometry
+    ("NCHW32", 3, 64, 28, 28, 256, 1, 1, 0, 1),     # pointwise, the expanding layer of a bottleneck block
+    ("NCHW32", 2, 128, 14, 14, 512, 1, 1, 0, 1),
+    ("NCHW32", 2, 256, 15, 13, 160, 1, 1, 0, 1),    # odd sizes, a partial channel tile
+    ("NCHW32", 2, 64, 28, 28, 64, 3, 1, 1, 1),      # 3x3 (the weight-resident and patch-staged tiles)
+    ("NCHW32", 2, 256, 14, 14, 256, 3, 1, 1, 1),
+    ("NCHW32", 2, 128, 28, 28, 128, 3, 2, 1, 1),
+    ("NCHW4", 2, 16, 28, 28, 96, 1, 1, 0, 1),       # 4-packed pointwise
+    ("NCHW4", 2, 64, 20, 20, 64, 3, 1, 1, 1),
+    ("NCHW4", 2, 4, 56, 56, 64, 7, 2, 3, 1),        # the first-layer kernel
+    ("NCHW4", 2, 96, 28, 28, 96, 3, 1, 1, 96),      # depthwise
+    ("NCHW", 2, 8, 12, 12, 8, 3, 1, 1, 1),          # the generic kernel
+]
+
+
+@pytest.mark.parametrize("i", range(len(IN_PLACE_CASES)))
+def test_output_may_replace_the_residual(i):
+    """dst == z (same buffer, same batch stride): every kernel reads the residual of an output element in the thread
+    that writes the element, before the write, so the result is that of separate buffers.  Every algorithm and every
+    tile that takes the shape, against the same launch with a buffer of its own for the output."""
+    fmt, n, ic, ih, iw, oc, f, stride, pad, group = IN_PLACE_CASES[i]
+    k = (ic // group) * f * f
+    kw = dict(scale_bias=2e-4, scale_z=0.02, scale_dst=float(np.float32(2e-4 * 73.9 * 73.3 * k ** 0.5 / 25.0)))
+    ran = 0
+    for nl in ("RELU", "H_SWISH"):
+        d = _abi.make_conv_desc(fmt, n, ic, ih, iw, oc, f, stride=stride, pad=pad, group=group, nonline=nl, has_z=True, **kw)
+        src, flt, bias, z = (to_dev(t) for t in util.make_tensors(d, seed=900 + i))
+        for algo_id in (DIRECT, IGEMM, DW, C4):
+            tiles = range(len(lib.tile_names())) if algo_id == IGEMM else [None]
+            for tile in tiles:
+                try:
+                    a, _ = ops.conv_bias_query(d, algo_id)
+                except Exception:
+                    break  # this algorithm does not take the problem
+                if tile is not None:
+                    if not lib.tile_usable(d, tile):
+                        continue
+                    a.tile_cfg = tile
+                say("in place: case", i, nl, "algo", algo_id, "tile", tile)
+                want = ops.conv_bias_exec(d, src, flt, bias, z, algo=a)
+                buf = z.clone()
+                got = ops.conv_bias_exec(d, src, flt, bias, buf, dst=buf, algo=a)
+                torch.cuda.synchronize()
+                assert got.data_ptr() == buf.data_ptr()
+                assert torch.equal(got, want), (i, nl, algo_id, tile)
+                ran += 1
+    assert ran >= 2
