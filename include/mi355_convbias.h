@@ -252,6 +252,18 @@ int mi355_igemm_tile_usable(const mi355_conv_desc* d, int tile_cfg);
  * no counterpart in the reference. */
 int mi355_epilogue_linear_form(float scale_bias, float scale_dst, uint32_t nonline, float* c, float* d);
 
+/* With a residual the same requantisation, dst = quantize_s8(act(float(sfb) * scale_bias + float(z) * scale_z)) with act
+ * IDENTITY or RELU (dnn/src/naive/conv_bias/opr_impl.cpp:21-98), is a step function of the integer sfb for each of the
+ * 256 values of the residual byte z.  When the library has proved, for every z and every int32 sfb, that
+ *     dst = floor(min(max(fma(float(sfb), c, table[z & 255]), lo), 127.5))         lo = 0 (RELU) or -128
+ * reproduces it, the kernels that hold the table in LDS use that form (five vector instructions and a table read per
+ * output instead of nine).  Returns 1 and writes c and the 256 offsets (indexed by the residual byte as an unsigned
+ * value) if it has such a proof for these scales -- it has none where scale_bias / scale_dst is below about 3e-3 --
+ * 0 if not (the kernels then run the multi-step form), a negative mi355_status on a bad argument.  The first call for
+ * a scale triple costs about a millisecond of host time.  Diagnostic: no counterpart in the reference. */
+int mi355_epilogue_residual_table(float scale_bias, float scale_z, float scale_dst, uint32_t nonline, float* c,
+                                  float* table);
+
 /* The division r / scale_dst of the requantisation (dnn/include/megdnn/dtype.h:846) runs in the tiled kernels as
  *     t = r * y_lo;  q = fma(r, y_hi, t)          y_hi = RN(1 / scale_dst),  y_lo = RN(1 / scale_dst - y_hi)
  * -- a quotient at most one ulp from the correctly rounded one, which can change a result only next to a rounding

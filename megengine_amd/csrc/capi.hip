@@ -9,6 +9,7 @@
 #include <mutex>
 #include <shared_mutex>
 #include <unordered_map>
+#include <vector>
 
 #include "common.h"
 
@@ -254,6 +255,154 @@ bool epi_linear_cached(float s_b, float s_d, bool relu, float* c, float* d) {
     return e.solved;
 }
 
+// ---- residual table form (epilogue.h): the linear form with a residual ------------------------------------------
+// The contract WITH z, as a function of the integer sfb and the residual byte (separately rounded binary32 operations):
+int epi_contract_z(int t, int z, float s_b, float s_z, float s_d, bool relu) {
+    float r = (float)t * s_b;
+    const float zf = (float)z * s_z;
+    r = r + zf;
+    if (relu) r = r <= 0.f ? 0.f : r;
+    float v = roundf(r / s_d);
+    v = fminf(fmaxf(-128.f, v), 127.f);
+    return (int)v;
+}
+
+// For every one of the 256 residual values the contract is a non-decreasing step function of sfb, like the contract
+// without z, and its steps are those of the others shifted by about z s_z / s_b: one slope c serves all of them and each
+// gets an offset of its own, tab[z].  Finds c and the 256 offsets such that epi_linear(t, c, tab[z], lo) ==
+// epi_contract_z(t, z) on EVERY int32 t for every z, or reports that it found none.  Per z this is epi_solve_linear's
+// argument: the step positions T[k] of the contract by bisection (started from the real-arithmetic position, a handful
+// of evaluations each), a candidate accepted only if it has step k at T[k] for every k, evaluated with the device's
+// arithmetic.  It fails where s_b / s_d is small (below about 3e-3: an offset then has less room than the literal
+// chain's own roundings move the steps).  ~1 ms of host time.
+bool epi_solve_table(float s_b, float s_z, float s_d, bool relu, float* c_out, float* tab) {
+    const int LIM = 1 << 24;
+    const int kmin = relu ? 1 : -127, kmax = 127, NK = kmax - kmin + 1;
+    const float c0 = (float)((double)s_b / (double)s_d);
+    if (!(c0 > 0.f) || !(c0 < 0x1p20f)) return false;
+    std::vector<int> T((size_t)256 * NK);
+    for (int zi = 0; zi < 256; ++zi) {
+        const int z = zi - 128;
+        if (epi_contract_z(LIM, z, s_b, s_z, s_d, relu) < kmax) return false;
+        if (epi_contract_z(-LIM, z, s_b, s_z, s_d, relu) >= kmin) return false;
+        for (int k = kmin; k <= kmax; ++k) {
+            const double g = (((double)k - 0.5) * (double)s_d - (double)z * (double)s_z) / (double)s_b;
+            int64_t gi = (int64_t)ceil(g);
+            if (gi > LIM - 1) gi = LIM - 1;
+            if (gi < -LIM + 1) gi = -LIM + 1;
+            int64_t lo, hi, step = 1;  // contract(lo) < k <= contract(hi)
+            if (epi_contract_z((int)gi, z, s_b, s_z, s_d, relu) >= k) {
+                hi = gi;
+                lo = gi - 1;
+                while (lo > -LIM && epi_contract_z((int)lo, z, s_b, s_z, s_d, relu) >= k) {
+                    hi = lo;
+                    lo -= step;
+                    step *= 2;
+                }
+                if (lo < -LIM) lo = -LIM;
+            } else {
+                lo = gi;
+                hi = gi + 1;
+                while (hi < LIM && epi_contract_z((int)hi, z, s_b, s_z, s_d, relu) < k) {
+                    lo = hi;
+                    hi += step;
+                    step *= 2;
+                }
+                if (hi > LIM) hi = LIM;
+            }
+            while (hi - lo > 1) {
+                const int64_t m = lo + (hi - lo) / 2;
+                if (epi_contract_z((int)m, z, s_b, s_z, s_d, relu) >= k) hi = m; else lo = m;
+            }
+            if (hi >= LIM || hi <= -LIM + 1) return false;  // float(t) must be exact around every step
+            T[(size_t)zi * NK + (k - kmin)] = (int)hi;
+        }
+    }
+    const float lo_clamp = relu ? 0.f : -128.f;
+    for (int u = 0; u <= 8; ++u) {
+        for (int sgn = -1; sgn <= 1; sgn += 2) {
+            if (u == 0 && sgn == 1) continue;
+            float c = c0;
+            for (int i = 0; i < u; ++i) c = nextafterf(c, sgn > 0 ? INFINITY : 0.f);
+            if (!(c > 0.f)) continue;
+            bool all = true;
+            for (int zi = 0; zi < 256 && all; ++zi) {
+                const int* Tz = &T[(size_t)zi * NK];
+                double dlo = -1e300, dhi = 1e300;
+                for (int k = kmin; k <= kmax; ++k) {
+                    const double a = (double)k - (double)Tz[k - kmin] * (double)c;
+                    if (a > dlo) dlo = a;
+                    if (a + (double)c < dhi) dhi = a + (double)c;
+                }
+                bool found = false;
+                for (int j = 1; j <= 3 && dlo < dhi && !found; ++j) {
+                    const float d = (float)(dlo + (dhi - dlo) * j / 4.0);
+                    bool ok = true;
+                    for (int k = kmin; k <= kmax && ok; ++k) {
+                        const int t = Tz[k - kmin];
+                        ok = epi_linear(t, c, d, lo_clamp) >= k && epi_linear(t - 1, c, d, lo_clamp) <= k - 1;
+                    }
+                    if (ok) {
+                        tab[zi] = d;
+                        found = true;
+                    }
+                }
+                all = found;
+            }
+            if (all) {
+                *c_out = c;
+                return true;
+            }
+        }
+    }
+    return false;
+}
+
+// One entry per (s_b, s_z, s_d, activation), kept for the life of the process like the other proofs (node-based map:
+// the address of an entry never changes, launches copy the table from it).  At most kTableCacheCap entries are stored
+// (1 KiB each); beyond that a new triple is reported unsolved and runs the multi-step form.
+struct TableKey {
+    uint32_t b, z, d, relu;
+    bool operator==(const TableKey& o) const { return b == o.b && z == o.z && d == o.d && relu == o.relu; }
+};
+struct TableKeyHash {
+    size_t operator()(const TableKey& k) const {
+        uint64_t h = ((uint64_t)k.b << 32 | k.d) * 0x9e3779b97f4a7c15ull;
+        h ^= ((uint64_t)k.z << 1 | k.relu) * 0xc2b2ae3d27d4eb4full;
+        return (size_t)(h ^ (h >> 29));
+    }
+};
+struct TableEntry {
+    bool solved;
+    float c;
+    float tab[256];  // indexed by the residual byte as an unsigned value
+};
+constexpr size_t kTableCacheCap = 4096;
+std::shared_mutex g_table_mu;
+std::unordered_map<TableKey, TableEntry, TableKeyHash> g_table;
+
+const TableEntry* epi_table_cached(float s_b, float s_z, float s_d, bool relu) {
+    TableKey key;
+    memcpy(&key.b, &s_b, 4);
+    memcpy(&key.z, &s_z, 4);
+    memcpy(&key.d, &s_d, 4);
+    key.relu = relu ? 1u : 0u;
+    {
+        std::shared_lock<std::shared_mutex> lk(g_table_mu);
+        auto it = g_table.find(key);
+        if (it != g_table.end()) return &it->second;
+        if (g_table.size() >= kTableCacheCap) return nullptr;
+    }
+    TableEntry e;
+    float by_z[256];
+    e.c = 0.f;
+    e.solved = epi_solve_table(s_b, s_z, s_d, relu, &e.c, by_z);
+    for (int u = 0; u < 256; ++u) e.tab[u] = e.solved ? by_z[(int)(int8_t)u + 128] : 0.f;
+    std::unique_lock<std::shared_mutex> lk(g_table_mu);
+    if (g_table.size() >= kTableCacheCap) return nullptr;
+    return &g_table.emplace(key, e).first->second;
+}
+
 // All epilogue parameters of one launch.  qs8: the destination is QuantizedS8 (the only dtype with the fast forms).
 void epi_fill(EpiParams* e, float s_b, float s_z, float s_d, uint32_t nonline, bool has_z, bool qs8) {
     e->s_b = s_b;
@@ -267,6 +416,7 @@ void epi_fill(EpiParams* e, float s_b, float s_z, float s_d, uint32_t nonline, b
     e->lin = 0;
     e->lin_c = e->lin_d = 0.f;
     e->lin_lo = nonline == MI355_NL_RELU ? 0.f : -128.f;
+    e->zlin = 0;
     if (e->fast && !has_z && (nonline == MI355_NL_IDENTITY || nonline == MI355_NL_RELU))
         e->lin = epi_linear_cached(s_b, s_d, nonline == MI355_NL_RELU, &e->lin_c, &e->lin_d) ? 1 : 0;
 }
@@ -409,6 +559,17 @@ size_t algo_workspace(const ConvProblem& p, int id) { return id == ALGO_NCHW_MFM
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 }  // namespace
+
+namespace mi355 {
+bool epi_residual_table(const EpiParams& e, float* c, const float** tab) {
+    if (!e.fast || !e.has_z || (e.nonline != MI355_NL_IDENTITY && e.nonline != MI355_NL_RELU)) return false;
+    const TableEntry* t = epi_table_cached(e.s_b, e.s_z, e.s_d, e.nonline == MI355_NL_RELU);
+    if (!t || !t->solved) return false;
+    *c = t->c;
+    *tab = t->tab;
+    return true;
+}
+}  // namespace mi355
 
 extern "C" {
 
@@ -891,6 +1052,18 @@ int mi355_epilogue_linear_form(float scale_bias, float scale_dst, uint32_t nonli
     *c = e.lin_c;
     *d = e.lin_d;
     return e.lin;
+}
+
+int mi355_epilogue_residual_table(float scale_bias, float scale_z, float scale_dst, uint32_t nonline, float* c, float* table) {
+    if (!c || !table) return -fail(MI355_ERR_BAD_ARG, "null output");
+    if (nonline != MI355_NL_IDENTITY && nonline != MI355_NL_RELU)
+        return -fail(MI355_ERR_BAD_ARG, "the residual table form exists for IDENTITY and RELU only");
+    EpiParams e;
+    epi_fill(&e, scale_bias, scale_z, scale_dst, nonline, true, true);
+    const float* t;
+    if (!epi_residual_table(e, c, &t)) return 0;
+    memcpy(table, t, 256 * sizeof(float));
+    return 1;
 }
 
 // ---- RelayoutFormat ----

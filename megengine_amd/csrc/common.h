@@ -30,6 +30,11 @@ struct ConvProblem {
     EpiParams epi;
 };
 
+// The residual table form of the requantisation (epilogue.h): true, the slope and the 256 offsets (indexed by the
+// residual byte as an unsigned value; the pointer stays valid for the life of the process) when the host has proved it
+// for these scales and this activation.  A hash lookup after the first call for a scale triple.
+bool epi_residual_table(const EpiParams& e, float* c, const float** tab);
+
 // ---- launchers (each returns a hipError_t-compatible int; 0 = success) ----
 int launch_conv_direct(hipStream_t st, const ConvProblem& p, const int8_t* src, const int8_t* flt,
                        const int32_t* bias, const void* z, void* dst);

@@ -595,6 +595,17 @@ static int pick_cfg_by_shape(const ConvProblem& p, int cu_count, bool will_prepr
         const int s = igemm_pw32s_cfg();
         if (igemm_resolve_cfg(p, s) == s) return s;
     }
+    if (p.pin == 32 && p.pout == 32 && d.group == 1 && !igemm_needs_general(p) && d.fh == 1 && d.fw == 1 && d.pad_h == 0 &&
+        d.pad_w == 0 && d.has_z && d.ic <= 128) {
+        // pointwise with a residual over at most 128 channels (the expanding 1x1 of a bottleneck block): bound by the
+        // vector instructions of the requantisation, which the residual table form halves -- the streaming kernel where
+        // the host has a proof for these scales (64 -> 256 at 56 x 56, batch 64: 20.5 against 23.4 us on the tiled kernel;
+        // 128 -> 512 at 28 x 28: 14.6 against 16.1)
+        float c;
+        const float* tab;
+        const int s = igemm_pw32s_cfg();
+        if (epi_residual_table(p.epi, &c, &tab) && igemm_resolve_cfg(p, s) == s) return s;
+    }
     if (will_preprocess && p.pin == 32 && p.pout == 32 && d.group == 1 && !igemm_needs_general(p)) {
         // The caller re-tiles the filter for the chosen algorithm (weight pre-processing): the second-generation tiles
         // then copy whole kilobytes for both operands.  Every tile was forced on every ResNet-50 shape in turn and timed
@@ -860,6 +871,19 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
         return launch_planar(st, a, cfg, cu_count);
     }
     const int first_v2 = igemm_first_v2_cfg();
+    if (cfg == igemm_pw32s_cfg() && !a.general) {
+        // the streaming kernel holds the residual table in LDS: it takes the table form where the host has proved it
+        // for these scales.  (The first-generation LDS-direct kernel with the table behind its ring, tried on the
+        // residual layers over 256 and 512 channels, changed the ResNet-50 step by +1 us: those are not bound by their
+        // vector instructions.)
+        float c;
+        const float* tab;
+        if (epi_residual_table(a.epi, &c, &tab)) {
+            a.epi.zlin = 1;
+            a.epi.lin_c = c;
+            memcpy(a.ztab, tab, sizeof(a.ztab));
+        }
+    }
     if (cfg == igemm_pw32s_cfg()) return launch_pw32s(st, a, cu_count);
     if (cfg >= igemm_first_v4_cfg()) return launch_igemm4(st, a, p.pin, p.pout, cfg - igemm_first_v4_cfg(), cu_count);
     if (cfg >= igemm_first_v3_cfg()) return launch_igemm3(st, a, p.pin, p.pout, cfg - igemm_first_v3_cfg());

@@ -110,6 +110,14 @@ __global__ __launch_bounds__(256, 2) void pw32s_kernel(IgemmArgs a, int n_ocg, i
     const __amdgpu_buffer_rsrc_t rs_src = make_rsrc(a.src, a.src_bytes);
     const __amdgpu_buffer_rsrc_t rs_flt = make_rsrc(a.flt, a.flt_bytes);
     const __amdgpu_buffer_rsrc_t rs_bias = make_rsrc(a.bias, a.has_bias ? a.OC * 4 : 0);
+    // residual table form: the 256 offsets from the kernel arguments into LDS, once per workgroup (ahead of the first
+    // loads: behind them, with the barrier holding every wave until the slowest wave's loads are back, the stack is 3 us
+    // slower)
+    __shared__ float zt[HZ ? 256 : 1];
+    if constexpr (HZ) {
+        if (a.epi.zlin) zt[t] = a.ztab[t];
+        __syncthreads();
+    }
 
     v4i fa[MT][KC];
 #pragma unroll
@@ -157,7 +165,7 @@ __global__ __launch_bounds__(256, 2) void pw32s_kernel(IgemmArgs a, int n_ocg, i
 #pragma unroll
             for (int i = 0; i < MT; ++i) acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i][kc], fb[kc], acc[i][0], 0, 0, 0);
         if constexpr (HZ)
-            igemm_run_epilogue<32, MT, 1, true>(a, acc, oc_w, pb * 32, l32, lh, &zr);
+            igemm_run_epilogue<32, MT, 1, true>(a, acc, oc_w, pb * 32, l32, lh, &zr, -1, 1, 0, -1, zt);
         else
             igemm_run_epilogue<32, MT, 1>(a, acc, oc_w, pb * 32, l32, lh);
 #pragma unroll

@@ -35,6 +35,13 @@
 // checks every step of the candidate against them with the device's own arithmetic (epi_solve_linear
 // in capi.hip).  Only a pair (c, d) that passes is ever handed to a kernel; when none passes, the
 // fast form runs.
+//
+// The "residual table" form (NL_ZLIN; IDENTITY or RELU with z) is the linear form with an offset per residual value:
+//     dst = floor(min(max(fma(float(sfb), c, tab[z]), lo), 127.5))          tab: 256 floats in LDS
+// For each of the 256 values of z the contract is a step function of sfb as above; the host finds the steps of all 256,
+// one slope c and an offset per z, and checks every step of every z with the device's arithmetic (epi_solve_table in
+// capi.hip).  Five vector instructions and an LDS read per output instead of nine; scale triples without a proof
+// (small s_bias / s_dst) run the fast form.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -50,10 +57,12 @@ struct EpiParams {
     int fast;     // 1: fast form allowed
     int lin;      // 1: linear form verified for (s_b, s_d, nonline); implies fast && !has_z
     float lin_c, lin_d, lin_lo;
+    int zlin;     // 1: residual table form (set by the launch code of a kernel that holds the table; slope in lin_c)
 };
 
 // NL_LIN is not an activation of the interface: it selects the linear form in the kernels' epilogue templates
-enum { NL_IDENTITY = 0, NL_RELU = 1, NL_H_SWISH = 3, NL_LIN = 4 };
+// and NL_ZLIN the residual table form
+enum { NL_IDENTITY = 0, NL_RELU = 1, NL_H_SWISH = 3, NL_LIN = 4, NL_ZLIN = 5 };
 
 __device__ __forceinline__ float act_f32(float r, int nl) {
     if (nl == NL_RELU) return r <= 0.f ? 0.f : r;
@@ -191,6 +200,21 @@ __device__ __forceinline__ uint32_t requant4_fast(int a0, int a1, int a2, int a3
     convert_into_byte<NL, 1>(o, x1);
     convert_into_byte<NL, 2>(o, x2);
     convert_into_byte<NL, 3>(o, x3);
+    return o;
+}
+
+// residual table form: zt = the table in LDS, zw = the four residual bytes of the four accumulators
+__device__ __forceinline__ uint32_t requant4_table(int a0, int a1, int a2, int a3, uint32_t zw, const EpiParams& e,
+                                                   const float* zt) {
+    const float x0 = __builtin_amdgcn_fmed3f(__builtin_fmaf((float)a0, e.lin_c, zt[zw & 0xffu]), e.lin_lo, 127.5f);
+    const float x1 = __builtin_amdgcn_fmed3f(__builtin_fmaf((float)a1, e.lin_c, zt[(zw >> 8) & 0xffu]), e.lin_lo, 127.5f);
+    const float x2 = __builtin_amdgcn_fmed3f(__builtin_fmaf((float)a2, e.lin_c, zt[(zw >> 16) & 0xffu]), e.lin_lo, 127.5f);
+    const float x3 = __builtin_amdgcn_fmed3f(__builtin_fmaf((float)a3, e.lin_c, zt[zw >> 24]), e.lin_lo, 127.5f);
+    uint32_t o;
+    convert_into_byte<NL_LIN, 0>(o, x0);
+    convert_into_byte<NL_LIN, 1>(o, x1);
+    convert_into_byte<NL_LIN, 2>(o, x2);
+    convert_into_byte<NL_LIN, 3>(o, x3);
     return o;
 }
 

@@ -55,6 +55,9 @@ struct IgemmArgs {
     int NB, p_w, p_himg, pxp, pcw, cbs;
     FastDiv div_pw, div_phimg;
     int dry_run;  // host only: the launch code stops before anything is launched and reports whether the tile fits
+    // residual table form (epi.zlin): the 256 offsets, indexed by the residual byte as an unsigned value; a kernel that
+    // takes the form copies them from here (the kernel-argument segment) into LDS
+    float ztab[256];
 };
 
 struct KEntry {
@@ -126,9 +129,11 @@ __device__ __forceinline__ void igemm_load_z(const IgemmArgs& a, ZRegs<MT, NT>& 
 // blk_mod > 1: only the blocks b = i * NT + j with b % blk_mod == blk_rem are written (a wave of a workgroup that
 // splits the reduction finishes its share of the blocks; wave-uniform)
 // m_end: one past the last pixel (flattened over batch and image) this tile may write
+// zt: the residual table in LDS (NL_ZLIN only)
 template <int POUT, int MT, int NT, int NL, bool HZ, bool ZPRE>
 __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], const ZRegs<MT, NT>* zr, int oc_w,
-                                               int pix_w, int l32, int lh, int oc_end, int blk_mod, int blk_rem, int m_end) {
+                                               int pix_w, int l32, int lh, int oc_end, int blk_mod, int blk_rem, int m_end,
+                                               const float* zt = nullptr) {
     const __amdgpu_buffer_rsrc_t rs_z = make_rsrc(a.z, HZ ? a.z_bytes : 0);
     // stores go through a buffer descriptor: a lane outside the tile carries the out-of-range offset and its store is
     // dropped (no branch, no 64-bit address arithmetic); the channel block's offset is wave-uniform and scalar
@@ -163,8 +168,12 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
                 }
                 uint32_t o[4];
 #pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    o[q] = requant4_fast<NL, HZ>(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], zq[q], a.epi);
+                for (int q = 0; q < 4; ++q) {
+                    if constexpr (NL == NL_ZLIN)
+                        o[q] = requant4_table(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], zq[q], a.epi, zt);
+                    else
+                        o[q] = requant4_fast<NL, HZ>(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], zq[q], a.epi);
+                }
                 // accumulator order -> stored order
                 auto s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
                 auto s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
@@ -183,7 +192,11 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
                     uint32_t zw = 0;
                     if (HZ) zw = ZPRE ? (uint32_t)zr->v[i][j][q]
                                       : (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_z, ok ? z_pix + off : -1, 0, 0);
-                    uint32_t o = requant4_fast<NL, HZ>(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], zw, a.epi);
+                    uint32_t o;
+                    if constexpr (NL == NL_ZLIN)
+                        o = requant4_table(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], zw, a.epi, zt);
+                    else
+                        o = requant4_fast<NL, HZ>(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], zw, a.epi);
                     __builtin_amdgcn_raw_buffer_store_b32(o, rs_dst, ok ? d_pix + off : SENT, 0, 0);
                 }
             }
@@ -194,13 +207,16 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmArgs& a, v16i (&acc)[M
 // Fused requantisation + store of one wave tile (MT x NT blocks of 32 channels x 32 pixels).
 // oc_end: one past the last output channel this tile may write (the layer's channel count, or the end of the tile's
 // group); negative = the layer's channel count.
+// zt: the kernel's LDS copy of the residual table, or null: a kernel without one never takes the table form
 template <int POUT, int MT, int NT, bool ZPRE = false>
 __device__ __forceinline__ void igemm_run_epilogue(const IgemmArgs& a, v16i (&acc)[MT][NT], int oc_w, int pix_w, int l32,
                                                    int lh, const ZRegs<MT, NT>* zr = nullptr, int oc_end = -1, int blk_mod = 1,
-                                                   int blk_rem = 0, int m_end = -1) {
+                                                   int blk_rem = 0, int m_end = -1, const float* zt = nullptr) {
     if (oc_end < 0) oc_end = a.OC;
     if (m_end < 0) m_end = a.M;
-    if (a.epi.lin) {
+    if (zt != nullptr && a.epi.zlin) {
+        igemm_epilogue<POUT, MT, NT, NL_ZLIN, true, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem, m_end, zt);
+    } else if (a.epi.lin) {
         igemm_epilogue<POUT, MT, NT, NL_LIN, false, ZPRE>(a, acc, zr, oc_w, pix_w, l32, lh, oc_end, blk_mod, blk_rem, m_end);
     } else if (a.epi.has_z) {
         switch (a.epi.nonline) {

@@ -17,7 +17,7 @@ EXPORTS = [
     "mi355_abi_version", "mi355_status_string", "mi355_last_error", "mi355_get_device_info", "mi355_stream_probe",
     "mi355_convbias_deduce_out", "mi355_convbias_algo_count", "mi355_convbias_algo_name",
     "mi355_convbias_algo_usable", "mi355_convbias_s8_query", "mi355_convbias_s8_exec",
-    "mi355_igemm_tile_count", "mi355_igemm_tile_name", "mi355_igemm_tile_usable", "mi355_epilogue_linear_form",
+    "mi355_igemm_tile_count", "mi355_igemm_tile_name", "mi355_igemm_tile_usable", "mi355_epilogue_linear_form", "mi355_epilogue_residual_table",
     "mi355_relayout_deduce", "mi355_relayout_exec", "mi355_requant_s32_s8_exec", "mi355_requant_s8_s8_exec", "mi355_elemwise_q_exec",
     "mi355_convbias_s8_profile",
     "mi355_pooling_deduce_out", "mi355_pooling_s8_exec", "mi355_typecvt_f32_s8_exec", "mi355_typecvt_s8_f32_exec",
@@ -77,6 +77,8 @@ def lib():
     L.mi355_igemm_tile_usable.argtypes = [P(_abi.ConvDesc), C.c_int]
     L.mi355_epilogue_quotient_form.restype = C.c_int
     L.mi355_epilogue_quotient_form.argtypes = [C.c_float, P(C.c_float), P(C.c_float)]
+    L.mi355_epilogue_residual_table.restype = C.c_int
+    L.mi355_epilogue_residual_table.argtypes = [C.c_float, C.c_float, C.c_float, C.c_uint32, P(C.c_float), P(C.c_float)]
     L.mi355_epilogue_linear_form.restype = C.c_int
     L.mi355_epilogue_linear_form.argtypes = [C.c_float, C.c_float, C.c_uint32, P(C.c_float), P(C.c_float)]
     L.mi355_relayout_deduce.argtypes = [P(_abi.RelayoutDesc), P(C.c_uint32), P(C.c_uint32)]

@@ -1010,3 +1010,46 @@ def test_output_may_replace_the_residual(i):
                 assert torch.equal(got, want), (i, nl, algo_id, tile)
                 ran += 1
     assert ran >= 2
+
+
+def _proved_triples(n, seed):
+    """scale triples (and scale_bias / scale_dst) for which the library holds a proof of the residual table form for
+    both activations that have one"""
+    import ctypes as C
+    rng = np.random.RandomState(seed)
+    proved = []
+    while len(proved) < n:
+        c0 = float(np.exp(rng.uniform(np.log(5e-3), np.log(0.2))))
+        s_d = float(np.float32(np.exp(rng.uniform(np.log(1e-3), np.log(5e-2)))))
+        s_z = float(np.float32(s_d * rng.uniform(0.3, 1.5)))
+        s_b = float(np.float32(c0 * s_d))
+        c, tab = C.c_float(), (C.c_float * 256)()
+        if all(lib.lib().mi355_epilogue_residual_table(s_b, s_z, s_d, nl, C.byref(c), tab) == 1
+               for nl in (_abi.NL_IDENTITY, _abi.NL_RELU)):
+            proved.append((s_b, s_z, s_d, c0))
+    return proved
+
+
+def test_residual_table_form_on_the_streaming_kernel(oracle):
+    """Scale triples for which the library holds a proof of the residual table form (one fused multiply-add and a table
+    read per output): the streaming kernel then runs that form, and its bytes must be the checker's.  Small operand
+    ranges keep most outputs inside the int8 range, so every residual value meets most output steps."""
+    tile = lib.tile_names().index("pw32_stream")
+    proved = _proved_triples(4, 31)
+    shapes = [(2, 64, 28, 28, 256, 1), (3, 32, 17, 23, 96, 1), (2, 128, 14, 14, 512, 1), (5, 64, 7, 7, 64, 1),
+              (4, 64, 30, 31, 160, 2)]
+    for i, (s_b, s_z, s_d, c0) in enumerate(proved):
+        n, ic, ih, iw, oc, stride = shapes[i % len(shapes)]
+        # accumulator sigma ~ 40 / c0 units: about 40 output steps
+        amp = max(1, min(127, int(round((40.0 / c0 / ic ** 0.5) ** 0.5 * 1.7))))
+        for nl in ("IDENTITY", "RELU"):
+            d = _abi.make_conv_desc("NCHW32", n, ic, ih, iw, oc, 1, stride=stride, nonline=nl, has_z=True,
+                                    scale_bias=s_b, scale_z=s_z, scale_dst=s_d)
+            assert lib.tile_usable(d, tile)
+            a, _ = ops.conv_bias_query(d, _abi.ALGO_HEURISTIC)
+            assert a.tile_cfg == tile, "the chooser takes the streaming kernel where the table is proved"
+            want = check_case(oracle, d, seed=950 + i, algo=IGEMM, tile=tile, tag="table-%d" % i, src_range=(-amp, amp),
+                              flt_range=(-amp, amp), bias_range=(-50, 50))
+            live = float(np.mean((want > -128) & (want < 127) & (want != 0)))
+            say("table form case", i, nl, "c0 %.3g" % c0, "amp", amp, "live outputs %.2f" % live)
+            assert live > 0.2

@@ -106,9 +106,10 @@ def test_ring_kernels_with_register_resident_weights_use_no_scratch(resources):
 def test_streaming_pointwise_kernels_keep_accumulators_in_vgprs(resources):
     """pw32s_kernel is bound by its vector instructions: accumulators in AGPRs would cost a move in and a move out per
     output (the compiler picks the VGPR form of the MFMA only when the launch bounds cap the register file at 256), and
-    three workgroups per CU must fit."""
+    three workgroups per CU must fit.  Its only LDS is the kilobyte of the residual table (variants with a residual)."""
     ks = kernels(resources, r"pw32s_kernel<")
     assert len(ks) == 16
     for name, r in ks.items():
-        assert r["agprs"] == 0 and r["scratch"] == 0 and r["lds"] == 0, (name, r)
+        assert r["agprs"] == 0 and r["scratch"] == 0, (name, r)
+        assert r["lds"] <= (1024 if ", true>" in name else 16), (name, r)
         assert r["occupancy"] >= 3, (name, r)
