@@ -871,6 +871,7 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
         return launch_planar(st, a, cfg, cu_count);
     }
     const int first_v2 = igemm_first_v2_cfg();
+    a.ztab = nullptr;
     if (cfg == igemm_pw32s_cfg() && !a.general) {
         // the streaming kernel holds the residual table in LDS: it takes the table form where the host has proved it
         // for these scales.  (The first-generation LDS-direct kernel with the table behind its ring, tried on the
@@ -881,7 +882,7 @@ int launch_conv_igemm(hipStream_t st, const ConvProblem& p, int cfg, int cu_coun
         if (epi_residual_table(a.epi, &c, &tab)) {
             a.epi.zlin = 1;
             a.epi.lin_c = c;
-            memcpy(a.ztab, tab, sizeof(a.ztab));
+            a.ztab = tab;
         }
     }
     if (cfg == igemm_pw32s_cfg()) return launch_pw32s(st, a, cu_count);

@@ -13,6 +13,8 @@
 //   * accumulators start from the bias (LDS copy), the fused epilogue and the NCHW4 stores are those of the tiled
 //     kernels (igemm_shared.h).
 // Channel blocks past the last one, and filter bytes past the end of a row, meet zero activations.
+#include <string.h>
+#include <type_traits>
 #include "igemm_shared.h"
 
 namespace mi355 {
@@ -99,23 +101,36 @@ __global__ __launch_bounds__(256) void pw4s_kernel(IgemmArgs a, int n_ocg, int n
 // of k-step kc is one 16-byte load -- half of its pixel's 32-byte block kc; 32 consecutive pixels are one contiguous
 // kilobyte -- and the stores are the 16-byte stores of the tiled kernels.
 template <int MT, int KC, bool HZ>
-__global__ __launch_bounds__(256, 2) void pw32s_kernel(IgemmArgs a, int n_ocg, int n_pb) {
+__global__ __launch_bounds__(256, 2) void pw32s_kernel(IgemmArgs a, int n_ocg, int n_pb,
+                                                       std::conditional_t<HZ, ResidualTable, NoResidualTable> tab) {
     const int t = threadIdx.x;
     const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
 
-    const int gw = blockIdx.x * 4 + wave, GW = gridDim.x * 4;  // GW is a multiple of n_ocg
-    const int pb0 = gw / n_ocg, ocg = gw - pb0 * n_ocg, step = GW / n_ocg;
+    // Pixel blocks by XCD, as the tiled kernels deal out their tiles: workgroup b runs on XCD b % 8 (round-robin
+    // dispatch) and each XCD takes one contiguous eighth of the pixel blocks, so that this layer finds its inputs in the
+    // L2 of the XCD that wrote them and leaves its outputs where the next layer's workgroups will look for them.
+    // (Grids that are no multiple of 8 n_ocg / 4 workgroups -- small problems -- interleave the blocks instead.)
+    int pb_lo = 0, pb_hi = n_pb, gw = blockIdx.x * 4 + wave, GW = gridDim.x * 4;  // GW is a multiple of n_ocg
+    if ((gridDim.x & 7) == 0 && ((gridDim.x >> 3) * 4) % n_ocg == 0) {
+        const int x = blockIdx.x & 7, per = n_pb >> 3, rem = n_pb & 7;
+        pb_lo = x * per + (x < rem ? x : rem);
+        pb_hi = pb_lo + per + (x < rem ? 1 : 0);
+        gw = (blockIdx.x >> 3) * 4 + wave;
+        GW = (gridDim.x >> 3) * 4;
+    }
+    const int q0 = gw / n_ocg, ocg = gw - q0 * n_ocg, step = GW / n_ocg;
+    const int pb0 = pb_lo + q0;
     const int oc_w = ocg * MT * 32;
     const __amdgpu_buffer_rsrc_t rs_src = make_rsrc(a.src, a.src_bytes);
     const __amdgpu_buffer_rsrc_t rs_flt = make_rsrc(a.flt, a.flt_bytes);
     const __amdgpu_buffer_rsrc_t rs_bias = make_rsrc(a.bias, a.has_bias ? a.OC * 4 : 0);
-    // residual table form: the 256 offsets from the kernel arguments into LDS, once per workgroup (ahead of the first
+    // residual table form: the 256 offsets from the kernel's last argument into LDS, once per workgroup (ahead of the first
     // loads: behind them, with the barrier holding every wave until the slowest wave's loads are back, the stack is 3 us
     // slower)
     __shared__ float zt[HZ ? 256 : 1];
     if constexpr (HZ) {
-        if (a.epi.zlin) zt[t] = a.ztab[t];
+        if (a.epi.zlin) zt[t] = tab.v[t];
         __syncthreads();
     }
 
@@ -151,12 +166,14 @@ __global__ __launch_bounds__(256, 2) void pw32s_kernel(IgemmArgs a, int n_ocg, i
 
     v4i fb[KC], nb[KC];
     ZRegs<HZ ? MT : 1, 1> zr, nz;
-    load_b(pb0, fb);
-    if constexpr (HZ) igemm_load_z<32, MT, 1>(a, zr, oc_w, pb0 * 32, l32, lh);
-    for (int pb = pb0; pb < n_pb; pb += step) {
-        // the next block's pixels and residual are in flight during the multiply and the epilogue
-        load_b(pb + step, nb);
-        if constexpr (HZ) igemm_load_z<32, MT, 1>(a, nz, oc_w, (pb + step) * 32, l32, lh);
+    load_b(pb0 < pb_hi ? pb0 : n_pb, fb);
+    if constexpr (HZ) igemm_load_z<32, MT, 1>(a, zr, oc_w, (pb0 < pb_hi ? pb0 : n_pb) * 32, l32, lh);
+    for (int pb = pb0; pb < pb_hi; pb += step) {
+        // the next block's pixels and residual are in flight during the multiply and the epilogue (past the end of this
+        // XCD's blocks: the block past the last one, whose lanes are all masked)
+        const int nx = pb + step < pb_hi ? pb + step : n_pb;
+        load_b(nx, nb);
+        if constexpr (HZ) igemm_load_z<32, MT, 1>(a, nz, oc_w, nx * 32, l32, lh);
         v16i acc[MT][1];
 #pragma unroll
         for (int i = 0; i < MT; ++i) acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i][0], fb[0], bv[i], 0, 0, 0);
@@ -184,10 +201,15 @@ int launch32_mt(hipStream_t st, const IgemmArgs& a, int cu_count) {
     const int64_t cap = (int64_t)cu_count * 3;  // 12 waves per CU
     if (blocks > cap) blocks = cap;
     blocks = (blocks + n_ocg - 1) / n_ocg * n_ocg;  // waves of one pixel block stay together; 4 * blocks % n_ocg == 0
-    if (a.epi.has_z)
-        hipLaunchKernelGGL((pw32s_kernel<MT, KC, true>), dim3((unsigned)blocks), dim3(256), 0, st, a, n_ocg, n_pb);
-    else
-        hipLaunchKernelGGL((pw32s_kernel<MT, KC, false>), dim3((unsigned)blocks), dim3(256), 0, st, a, n_ocg, n_pb);
+    // large grids: a multiple of 8 n_ocg workgroups, which the kernel splits into one slab of pixel blocks per XCD
+    if (blocks >= 16 * (int64_t)n_ocg) blocks = blocks / (8 * n_ocg) * (8 * n_ocg);
+    if (a.epi.has_z) {
+        ResidualTable tab;
+        if (a.epi.zlin) memcpy(tab.v, a.ztab, sizeof(tab.v)); else memset(tab.v, 0, sizeof(tab.v));
+        hipLaunchKernelGGL((pw32s_kernel<MT, KC, true>), dim3((unsigned)blocks), dim3(256), 0, st, a, n_ocg, n_pb, tab);
+    } else {
+        hipLaunchKernelGGL((pw32s_kernel<MT, KC, false>), dim3((unsigned)blocks), dim3(256), 0, st, a, n_ocg, n_pb, NoResidualTable{});
+    }
     return (int)hipGetLastError();
 }
 

@@ -55,10 +55,16 @@ struct IgemmArgs {
     int NB, p_w, p_himg, pxp, pcw, cbs;
     FastDiv div_pw, div_phimg;
     int dry_run;  // host only: the launch code stops before anything is launched and reports whether the tile fits
-    // residual table form (epi.zlin): the 256 offsets, indexed by the residual byte as an unsigned value; a kernel that
-    // takes the form copies them from here (the kernel-argument segment) into LDS
-    float ztab[256];
+    // residual table form (epi.zlin), host only: the 256 offsets, indexed by the residual byte as an unsigned value.  The
+    // launch code of a kernel that takes the form hands them over in a kernel argument of their own (ResidualTable): a
+    // kilobyte inside this struct made every launch of every kernel ~0.2 us slower.
+    const float* ztab;
 };
+
+struct ResidualTable {
+    float v[256];
+};
+struct NoResidualTable {};
 
 struct KEntry {
     int off;    // byte offset of the k-unit relative to the pixel's (ih0, iw0) base
