@@ -213,7 +213,7 @@ def main():
     t_launch = ms_per_step * 1e-3 / nl
     roofline = dict(bound="hbm", achieved=round(tot_bytes / nl / t_launch / 1e9, 1), peak=HBM_PEAK / 1e9,
                     unit="GB/s", frac=round(tot_bytes / nl / t_launch / HBM_PEAK, 4), traffic=None,
-                    kernel="ConvBias MFMA kernels (igemm2_kernel, igemm_dma_kernel, igemm_kernel, c4_kernel), 53 launches per step",
+                    kernel="ConvBias MFMA kernels (igemm2_kernel, igemm3_kernel, igemm_dma_kernel, pw32s_kernel, c4_kernel), 53 launches per step",
                     bytes_per_launch=round(tot_bytes / nl), avg_launch_us=round(t_launch * 1e6, 2),
                     per_launch_event_sum_ms=round(kern_ms, 4),
                     mfma_tops=round(tot_ops / (ms_per_step * 1e-3) / 1e12, 1),
