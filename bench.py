@@ -43,6 +43,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only")
     ap.add_argument("--no-preprocess", action="store_true", help="exec with the filters in the reference layout only")
+    ap.add_argument("--tiles", default="", metavar="LAYER=TILE,...",
+                    help="run the named layers of the stack on the named tiles instead of the heuristic's (measurements; "
+                         "the output line says so)")
     ap.add_argument("--no-memory-plan", action="store_true",
                     help="one buffer per layer output instead of the static activation-memory plan")
     ap.add_argument("--no-residual-in-place", action="store_true",
@@ -95,7 +98,8 @@ def main():
     mem = None if args.no_memory_plan else workloads.plan_memory(plan, residual_in_place=not args.no_residual_in_place)
     # algorithm choice and weight pre-processing happen once, before the timed region (exec_preprocess is the
     # reference's own hook for hoisting filter re-tiling out of exec)
-    workloads.choose_algorithms(plan, weight_preprocess=not args.no_preprocess)
+    forced = dict(item.split("=") for item in args.tiles.split(",") if item)
+    workloads.choose_algorithms(plan, weight_preprocess=not args.no_preprocess, tiles=forced)
     side = torch.cuda.Stream()          # default priority; every launch of the bench goes here
     torch.cuda.set_stream(side)
     stream = torch.cuda.current_stream()
@@ -158,7 +162,8 @@ def main():
     unplanned_ms = None
     if mem is not None and graph_ms is not None:
         try:
-            plan2 = workloads.choose_algorithms(workloads.build_stack(layers, 7), weight_preprocess=not args.no_preprocess)
+            plan2 = workloads.choose_algorithms(workloads.build_stack(layers, 7), weight_preprocess=not args.no_preprocess,
+                                                tiles=forced)
             calls2 = workloads.bind_plan(plan2)
             for c in calls2:
                 c()
@@ -249,6 +254,7 @@ def main():
                            workload="BASELINE configs[2]: ResNet-50 v1.5 int8 conv stack, batch 64, 224x224, "
                                     "NCHW4 stem + NCHW32, fused residual z + RELU, random per-tensor scales",
                            batch=batch, layers=nl, launch=launch_mode, graph=graph_note,
+                           **(dict(forced_tiles=forced) if forced else {}),
                            activation_memory=("one buffer per layer output, %.0f MB" % (sum(p["dst"].numel() for p in plan) / 1e6)
                                               if mem is None else
                                               "static plan by liveness: %.0f MB for the %.0f MB of layer outputs%s"

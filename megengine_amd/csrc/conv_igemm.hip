@@ -601,10 +601,12 @@ static int pick_cfg_by_shape(const ConvProblem& p, int cu_count, bool will_prepr
         // vector instructions of the requantisation, which the residual table form halves -- the streaming kernel where
         // the host has a proof for these scales (64 -> 256 at 56 x 56, batch 64: 20.5 against 23.4 us on the tiled kernel;
         // 128 -> 512 at 28 x 28: 14.6 against 16.1)
+        // Over at most 64 channels the streaming kernel wins without a table too (64 -> 256 at 56 x 56 with the
+        // multi-step form, inside the ResNet-50 stack: -4 us per step against the tiled kernel, alternating bench runs).
         float c;
         const float* tab;
         const int s = igemm_pw32s_cfg();
-        if (epi_residual_table(p.epi, &c, &tab) && igemm_resolve_cfg(p, s) == s) return s;
+        if ((d.ic <= 64 || epi_residual_table(p.epi, &c, &tab)) && igemm_resolve_cfg(p, s) == s) return s;
     }
     if (will_preprocess && p.pin == 32 && p.pout == 32 && d.group == 1 && !igemm_needs_general(p)) {
         // The caller re-tiles the filter for the chosen algorithm (weight pre-processing): the second-generation tiles

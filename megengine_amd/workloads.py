@@ -287,14 +287,19 @@ def run_calibrated(plan, seed, weight_preprocess=True):
     return live
 
 
-def choose_algorithms(plan, weight_preprocess=True):
+def choose_algorithms(plan, weight_preprocess=True, tiles=None):
     """Algorithm choice for every layer of a plan, as an inference graph does it once at load time: the heuristic
     (for a caller that pre-processes weights when `weight_preprocess`), then exec_preprocess of the filter where the
-    chosen algorithm has a pre-processed form.  Fills p["algo"] and p["pre"] (None: exec takes the filter)."""
-    from . import ops
+    chosen algorithm has a pre-processed form.  Fills p["algo"] and p["pre"] (None: exec takes the filter).
+    `tiles` = {layer name: tile name}: those layers run the named tile of the MFMA algorithm instead (measurements)."""
+    from . import lib, ops
+    names = lib.tile_names() if tiles else []
     for p in plan:
         req = _abi.ALGO_HEURISTIC_PREPROCESS if weight_preprocess else _abi.ALGO_HEURISTIC
         p["algo"], _ = ops.conv_bias_query(p["desc"], req)
+        if tiles and p["layer"].name in tiles:
+            p["algo"], _ = ops.conv_bias_query(p["desc"], 1)
+            p["algo"].tile_cfg = names.index(tiles[p["layer"].name])
         p["pre"] = ops.conv_bias_preprocess(p["desc"], p["flt"], p["algo"]) if weight_preprocess else None
     return plan
 
