@@ -131,6 +131,15 @@ int main(int argc, char** argv) {
                 float y2;
                 (void)mi355_epilogue_quotient_form(s, &y, &y2);
                 (void)mi355_epilogue_linear_form(s * 1e-2f, s, MI355_NL_RELU, &c, &dd);
+                // the residual table form on a few triples that several threads ask for at once: equal answers
+                if (r() % 16 == 0) {
+                    float tc = 0.f, tab[256];
+                    const float sd = scales[r() % 4];
+                    const int ok = mi355_epilogue_residual_table(sd * 0.028f, sd * 0.7f, sd, MI355_NL_RELU, &tc, tab);
+                    float tc2 = 0.f, tab2[256];
+                    const int ok2 = mi355_epilogue_residual_table(sd * 0.028f, sd * 0.7f, sd, MI355_NL_RELU, &tc2, tab2);
+                    if (ok != ok2 || (ok == 1 && (tc != tc2 || memcmp(tab, tab2, sizeof(tab)) != 0))) bad.fetch_add(1);
+                }
             }
         });
     for (auto& th : pool) th.join();
